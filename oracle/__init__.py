@@ -1,0 +1,333 @@
+"""TEST INFRASTRUCTURE -- NOT PART OF THE PRODUCT.
+
+CPU restatement of the reference's chunk-wise mixed-precision optimizer step,
+used only as the parity checker by ``tests/``, ``__graft_entry__.smoke()`` and
+the ``cpu_baseline`` leg of ``bench.py``.  ``patrickstar_amd`` never imports it.
+
+Contents
+--------
+``AdamOracle``            ctypes front-end of ``adam_oracle.c`` (the native operator,
+                          ``patrickstar/ops/csrc/adam/cpu_adam.cpp:33-185,700-742`` and
+                          ``csrc/includes/cpu_adam.h:143-175``).
+``cast_fp32_to_fp16``     whole-chunk RNE write-back (``patrickstar/ops/chunk_io_buff.py:116-126``).
+``has_inf_or_nan``        ``patrickstar/fp16/loss_scaler.py:133-155``.
+``ScalerOracle``          ``patrickstar/fp16/loss_scaler.py:107-182`` state machine.
+``StaticScalerOracle``    ``patrickstar/fp16/loss_scaler.py:46-76``.
+``scaler_from_config``    ``patrickstar/runtime/engine.py:79-99`` wiring (``hysteresis`` feeds
+                          ``scale_factor``; ``delayed_shift`` is always 1 through the engine).
+``optimizer_step_oracle`` sequencing of ``patrickstar/ops/fp16_cpu_adam.py:472-628`` over a
+                          chunk list held as numpy arrays.
+
+Pinning: see the header of ``adam_oracle.c`` for the Adam arithmetic and
+``tests/test_oracle_scaler.py`` for the state machine (hand-derived trajectories
+and invariants).  The reference's own tests hold no golden vectors for this
+path; its loss-scale sequence is asserted nowhere in the reference.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle_adam.so")
+_lib = None
+
+ISA_AUTO, ISA_SCALAR, ISA_AVX2, ISA_AVX512 = 0, 1, 2, 3
+
+
+def build(force=False):
+    """Compile ``adam_oracle.c`` with the Makefile beside it."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.check_call(["make", "-s", "-C", _HERE])
+    return _LIB_PATH
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = ctypes.CDLL(_LIB_PATH)
+        f, u64, sz, vp, ci = (
+            ctypes.c_float,
+            ctypes.c_uint64,
+            ctypes.c_size_t,
+            ctypes.c_void_p,
+            ctypes.c_int,
+        )
+        L.oracle_sizeof_state.restype = ci
+        L.oracle_adam_init.argtypes = [vp, f, f, f, f, f, ci]
+        L.oracle_adam_init.restype = None
+        L.oracle_adam_advance.argtypes = [vp, u64, f, f]
+        L.oracle_adam_advance.restype = None
+        L.oracle_adam_set.argtypes = [vp, f, f, f, ci]
+        L.oracle_adam_set.restype = None
+        L.oracle_adam_consts.argtypes = [vp, f, vp]
+        L.oracle_adam_consts.restype = None
+        L.oracle_adam_span.argtypes = [vp, vp, vp, ci, vp, vp, sz, f, ci]
+        L.oracle_adam_span.restype = ci
+        L.oracle_adam_update.argtypes = [vp, u64, f, f, f, f, f, ci, vp, vp, ci, vp, vp, sz, f, ci]
+        L.oracle_adam_update.restype = ci
+        L.oracle_f32_to_f16.argtypes = [f]
+        L.oracle_f32_to_f16.restype = ctypes.c_uint16
+        L.oracle_f16_to_f32.argtypes = [ctypes.c_uint16]
+        L.oracle_f16_to_f32.restype = f
+        L.oracle_cast_f32_to_f16.argtypes = [vp, vp, sz]
+        L.oracle_cast_f32_to_f16.restype = None
+        L.oracle_any_nonfinite_f16.argtypes = [vp, sz]
+        L.oracle_any_nonfinite_f16.restype = ci
+        _lib = L
+    return _lib
+
+
+def _ptr(a):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _check(a, dtype):
+    assert isinstance(a, np.ndarray) and a.dtype == dtype and a.flags["C_CONTIGUOUS"], (
+        type(a),
+        getattr(a, "dtype", None),
+    )
+
+
+class AdamOracle:
+    """One native optimizer object of the reference (``create_adam`` ... ``adam_update``)."""
+
+    def __init__(self, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0, adamw_mode=True):
+        self._L = lib()
+        self._buf = ctypes.create_string_buffer(self._L.oracle_sizeof_state())
+        self._L.oracle_adam_init(self._buf, lr, beta1, beta2, eps, weight_decay, int(adamw_mode))
+
+    def advance(self, step, beta1, beta2):
+        self._L.oracle_adam_advance(self._buf, step, beta1, beta2)
+
+    def set(self, lr, eps, weight_decay, bias_correction=True):
+        self._L.oracle_adam_set(self._buf, lr, eps, weight_decay, int(bias_correction))
+
+    def consts(self, loss_scale=-1.0):
+        """(1-beta1, 1-beta2, bc2inv, step_size, wd_term, bc1) as float32."""
+        out = np.zeros(6, dtype=np.float32)
+        self._L.oracle_adam_consts(self._buf, loss_scale, _ptr(out))
+        return out
+
+    def update(
+        self,
+        step,
+        lr,
+        beta1,
+        beta2,
+        eps,
+        weight_decay,
+        bias_correction,
+        params,
+        grads,
+        exp_avg,
+        exp_avg_sq,
+        loss_scale=-1.0,
+        isa=ISA_AUTO,
+    ):
+        """``adam_update`` of the reference on flat numpy arrays, in place.
+
+        ``grads`` is float32 or float16 (read only); the others are float32.
+        """
+        _check(params, np.float32)
+        _check(exp_avg, np.float32)
+        _check(exp_avg_sq, np.float32)
+        assert grads.dtype in (np.float16, np.float32) and grads.flags["C_CONTIGUOUS"]
+        n = params.size
+        assert grads.size == n and exp_avg.size == n and exp_avg_sq.size == n
+        took = self._L.oracle_adam_update(
+            self._buf,
+            int(step),
+            lr,
+            beta1,
+            beta2,
+            eps,
+            weight_decay,
+            int(bool(bias_correction)),
+            _ptr(params),
+            _ptr(grads),
+            int(grads.dtype == np.float16),
+            _ptr(exp_avg),
+            _ptr(exp_avg_sq),
+            n,
+            float(loss_scale),
+            isa,
+        )
+        if took < 0:
+            raise RuntimeError(f"oracle code path {isa} is not supported by this CPU")
+        return took
+
+
+def cast_fp32_to_fp16(src):
+    """Whole-array fp32 -> fp16 round-to-nearest-even (the write-back cast)."""
+    _check(src, np.float32)
+    dst = np.empty(src.shape, dtype=np.float16)
+    lib().oracle_cast_f32_to_f16(_ptr(src), _ptr(dst), src.size)
+    return dst
+
+
+def has_inf_or_nan(x):
+    """``DynamicLossScaler._has_inf_or_nan``: the float32 sum of ``x`` is +-inf or NaN.
+
+    For fp16 inputs of any realistic length this is "some element is not
+    finite" (a finite fp16 sum cannot reach the float32 range), which is the
+    form the C helper evaluates; both forms are compared in the tests.
+    """
+    if x.dtype == np.float16 and x.flags["C_CONTIGUOUS"]:
+        return bool(lib().oracle_any_nonfinite_f16(_ptr(x), x.size))
+    s = float(np.asarray(x, dtype=np.float32).sum(dtype=np.float32))
+    return s == float("inf") or s == -float("inf") or s != s
+
+
+class StaticScalerOracle:
+    """Static scale: never reports overflow, never changes."""
+
+    def __init__(self, scale=1):
+        self.cur_scale = scale
+
+    def has_overflow(self, grad):
+        return False
+
+    def update_scale(self, overflow):
+        return None
+
+    @property
+    def loss_scale(self):
+        return self.cur_scale
+
+
+class ScalerOracle:
+    """Dynamic loss-scale state machine, restated as one transition function.
+
+    Python number semantics are kept on purpose: ``cur_scale`` stays an ``int``
+    until the first true division, and ``max(x / f, min_scale)`` hands back the
+    ``min_scale`` object itself when the clamp bites.
+    """
+
+    def __init__(
+        self,
+        init_scale=2**32,
+        scale_factor=2.0,
+        scale_window=1000,
+        min_scale=1,
+        delayed_shift=1,
+        consecutive_hysteresis=False,
+    ):
+        self.cur_scale = init_scale
+        self.cur_iter = 0
+        self.last_overflow_iter = -1
+        self.scale_factor = scale_factor
+        self.scale_window = scale_window
+        self.min_scale = min_scale
+        self.delayed_shift = delayed_shift
+        self.cur_hysteresis = delayed_shift
+        self.consecutive_hysteresis = consecutive_hysteresis
+
+    def has_overflow(self, grad):
+        return has_inf_or_nan(grad)
+
+    def update_scale(self, overflow):
+        if overflow:
+            shrink_now = self.delayed_shift == 1 or self.cur_hysteresis == 1
+            if shrink_now:
+                self.cur_scale = max(self.cur_scale / self.scale_factor, self.min_scale)
+            else:
+                self.cur_hysteresis -= 1
+            self.last_overflow_iter = self.cur_iter
+        else:
+            if self.consecutive_hysteresis:
+                self.cur_hysteresis = self.delayed_shift
+            since = self.cur_iter - self.last_overflow_iter
+            if since % self.scale_window == 0:
+                if not self.consecutive_hysteresis:
+                    self.cur_hysteresis = self.delayed_shift
+                self.cur_scale *= self.scale_factor
+        self.cur_iter += 1
+
+    @property
+    def loss_scale(self):
+        return self.cur_scale
+
+
+def scaler_from_config(fp16_config):
+    """Scaler the reference engine builds from ``config["fp16"]`` (None if the block is absent)."""
+    if fp16_config is None:
+        return None
+    assert fp16_config["enabled"], "Must enable fp16 training."
+    assert "loss_scale" in fp16_config, "Must have `loss_scale` field set."
+    if fp16_config["loss_scale"] == 0:
+        return ScalerOracle(
+            init_scale=2 ** fp16_config.get("initial_scale_power", 16),
+            scale_factor=fp16_config.get("hysteresis", 2),
+            scale_window=fp16_config.get("loss_scale_window", 2000),
+            min_scale=fp16_config.get("min_loss_scale", 1),
+        )
+    return StaticScalerOracle(fp16_config["loss_scale"])
+
+
+class OptimizerStepOracle:
+    """``FP16Adam.step`` over a chunk list, one native call per step over each chunk.
+
+    Each chunk is a dict of flat numpy arrays ``p32``, ``m``, ``v`` (float32)
+    and ``p16`` (float16; holds the gradients on entry to ``step`` and the
+    refreshed fp16 parameters on exit, as in the reference where backward
+    overwrites the fp16 parameter slot with the gradient).
+
+    Sequencing restated from ``fp16_cpu_adam.py``: overflow gate first
+    (``:549-558``: on overflow restore fp16 from fp32, ``update_scale(True)``,
+    leave ``step`` alone), else ``step += 1`` (``:574``), update every chunk
+    with the scaler's current scale or -1 (``:227``), cast fp32 -> fp16
+    (``chunk_io_buff.py:116-126``), ``update_scale(False)`` (``:624-625``).
+    The native object sees one ``adam_update`` per step (the whole chunk list
+    is one flat tensor for it), so consecutive steps take the running-product
+    branch of ``cpu_adam.h:143-162``.
+    """
+
+    def __init__(self, chunks, loss_scaler=None, lr=1e-3, betas=(0.9, 0.999), eps=1e-8,
+                 weight_decay=0.0, use_adamw=False, isa=ISA_AUTO):
+        self.chunks = chunks
+        self.loss_scaler = loss_scaler
+        self.lr, self.betas, self.eps, self.weight_decay = lr, betas, eps, weight_decay
+        self.use_adamw = use_adamw
+        self.step_count = 0
+        self.has_overflow = False
+        self.isa = isa
+        self.native = AdamOracle(lr, betas[0], betas[1], eps, weight_decay, use_adamw)
+
+    def check_overflow(self):
+        """Sticky OR over every chunk's gradients (``fp16_cpu_adam.py:279-285``)."""
+        if self.loss_scaler is None:
+            return
+        for c in self.chunks:
+            if self.has_overflow:
+                break
+            if self.loss_scaler.has_overflow(c["p16"]):
+                self.has_overflow = True
+
+    def step(self):
+        """Returns True when the step was skipped."""
+        if self.has_overflow:
+            for c in self.chunks:
+                c["p16"][...] = cast_fp32_to_fp16(c["p32"])
+            self.has_overflow = False
+            self.loss_scaler.update_scale(True)
+            return True
+        self.step_count += 1
+        scale = self.loss_scaler.loss_scale if self.loss_scaler is not None else -1
+        self.native.advance(self.step_count, self.betas[0], self.betas[1])
+        self.native.set(self.lr, self.eps, self.weight_decay, True)
+        L = lib()
+        for c in self.chunks:
+            took = L.oracle_adam_span(
+                self.native._buf, _ptr(c["p32"]), _ptr(c["p16"]), 1, _ptr(c["m"]), _ptr(c["v"]),
+                c["p32"].size, float(scale), self.isa,
+            )
+            assert took > 0
+            c["p16"][...] = cast_fp32_to_fp16(c["p32"])
+        if self.loss_scaler:
+            self.loss_scaler.update_scale(False)
+        return False
