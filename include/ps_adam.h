@@ -1,0 +1,209 @@
+/*
+ * ps_adam.h -- C ABI of the MI355X (gfx950) chunk-wise mixed-precision Adam step.
+ *
+ * This is the drop-in boundary for ONE path of PatrickStar: the native operator
+ * `cpu_adam_op` {create_adam, adam_update, destroy_adam} (reference:
+ * patrickstar/ops/csrc/adam/cpu_adam.cpp:751-756) together with the work the
+ * reference does around it per optimizer step in Python: the whole-chunk
+ * fp32->fp16 write-back (patrickstar/ops/chunk_io_buff.py:85-151), the fp16
+ * gradient staging (chunk_io_buff.py:214-255), the inf/nan probe
+ * (patrickstar/fp16/loss_scaler.py:133-155) and the loss-scale state machine
+ * (loss_scaler.py:158-182).
+ *
+ * Conventions
+ *   - plain C types only; every pointer named d_* (and every pointer inside
+ *     ps_chunk) is a DEVICE address unless stated otherwise; the library never
+ *     allocates, frees or keeps tensor memory.
+ *   - every entry point that takes a stream only ENQUEUES work on it and
+ *     returns; nothing here synchronises with the host except ps_state_read.
+ *   - return value: 0 on success; a negative value on failure
+ *     (-hipError_t for a HIP runtime error, PS_ERR_* otherwise);
+ *     ps_last_error() gives the text.  Nothing throws across this boundary.
+ *   - vector (16-byte) accesses are used when the four base addresses of a
+ *     chunk / tensor are 16-byte aligned; otherwise a slower element-wise path
+ *     produces the same bits.
+ */
+#ifndef PS_ADAM_H
+#define PS_ADAM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PS_ABI_VERSION 1
+
+#define PS_ERR_BAD_ARG (-10001)     /* null pointer, negative count, unknown mode */
+#define PS_ERR_UNKNOWN_ID (-10002)  /* optimizer id was never created (the reference dereferences null here) */
+#define PS_ERR_NO_DEVICE (-10003)   /* no usable GPU */
+
+typedef void* ps_stream_t; /* a hipStream_t; NULL is the null stream */
+
+/*
+ * One position of the four parallel chunk lists (reference: ChunkType in
+ * patrickstar/core/const.py:76-81; optimizer-state chunks are mapped 1:1 to
+ * the fp16 parameter chunk, patrickstar/core/client.py:282-309).  All four
+ * payloads have `chunk_numel` elements and identical tensor offsets.
+ * `param_fp16` holds the fp16 GRADIENTS when a step starts (backward writes each
+ * gradient over its parameter's slot, patrickstar/core/hook.py:212-216) and the
+ * refreshed fp16 PARAMETERS when it ends.
+ */
+typedef struct ps_chunk {
+    float* param_fp32;    /* ChunkType.PARAM_FP32 payload */
+    float* exp_avg;       /* ChunkType.MOMENTUM payload   */
+    float* exp_avg_sq;    /* ChunkType.VARIANCE payload   */
+    uint16_t* param_fp16; /* ChunkType.PARAM_FP16 payload (IEEE binary16 bit patterns) */
+} ps_chunk;
+
+/*
+ * Device-resident state of the optimizer step: the DynamicLossScaler fields
+ * (loss_scaler.py:107-125), the sticky overflow flag of FP16Adam
+ * (fp16_cpu_adam.py:279-285) and the Adam step counter with its float
+ * beta^t running products (cpu_adam.h:143-162).  It lives in device memory
+ * so that "was there an overflow -> skip, restore, halve" needs no host
+ * round trip.  128 bytes, 16-byte aligned.
+ */
+typedef struct ps_step_state {
+    double cur_scale;           /* loss_scale; Python float semantics (binary64) */
+    double scale_factor;
+    double min_scale;
+    int64_t cur_iter;           /* update_scale calls so far */
+    int64_t last_overflow_iter; /* -1 initially */
+    int64_t scale_window;
+    int64_t adam_step;          /* completed (not skipped) optimizer steps == state[p]["step"] */
+    int64_t skipped_steps;
+    int32_t delayed_shift;
+    int32_t cur_hysteresis;
+    int32_t consecutive_hysteresis;
+    int32_t scale_is_int;       /* Python type of cur_scale: int until the first true division */
+    int32_t factor_is_int;
+    int32_t min_is_int;
+    uint32_t overflow;          /* sticky flag of the step being assembled (0/1) */
+    uint32_t last_skipped;      /* what the latest ps_scaler_update decided */
+    float beta1;
+    float beta2;
+    float beta1_t_next;         /* beta1^t for t = adam_step + 1 */
+    float beta2_t_next;
+    uint32_t reserved[4];
+} ps_step_state;
+
+/* One entry of the optional per-iteration log written by ps_scaler_update. */
+typedef struct ps_scale_record {
+    double scale_after;   /* loss_scale after the call */
+    uint32_t overflow;    /* the flag the call consumed */
+    uint32_t scale_is_int;
+} ps_scale_record;
+
+/* ---- library ---------------------------------------------------------- */
+
+int ps_abi_version(void);
+const char* ps_last_error(void); /* text of the calling thread's latest failure */
+
+/* ---- native operator (replaces pybind module cpu_adam_op) --------------- */
+
+/* create_adam (cpu_adam.cpp:379-417).  Holds the host-side scalar state of
+ * one optimizer (alpha, betas, eps, weight decay, beta^t, step); ids are
+ * chosen by the caller (FP16Adam.optimizer_id, fp16_cpu_adam.py:62,175-176).
+ * Re-creating an id replaces it.  should_log prints one line like the reference. */
+int ps_adam_create(int optimizer_id, float alpha, float beta1, float beta2, float eps,
+                   float weight_decay, int adamw_mode, int should_log);
+
+/* destroy_adam (cpu_adam.cpp:744-749).  Unknown ids are ignored, as there. */
+int ps_adam_destroy(int optimizer_id);
+
+/* adam_update (cpu_adam.cpp:700-742) on ONE flat tensor in device memory:
+ * advances the host scalar state exactly like Adam_Optimizer::IncrementStep /
+ * update_state (cpu_adam.h:143-175) and applies the update of
+ * Adam_Optimizer::Step (cpu_adam.cpp:91-141) to every element.
+ *   d_grads          fp16 (grads_are_half != 0) or fp32; never written
+ *   loss_scale <= 0  no unscale (cpu_adam.cpp:101)
+ *   d_param_fp16_out optional: receives RNE(fp32 param) per element (the
+ *                    write-back of chunk_io_buff.py:116-126); may alias d_grads
+ *                    when the gradients are fp16; NULL to skip. */
+int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float beta2, float epsilon,
+                   float weight_decay, int bias_correction, float* d_params, const void* d_grads,
+                   int grads_are_half, float* d_exp_avg, float* d_exp_avg_sq, size_t numel,
+                   float loss_scale, uint16_t* d_param_fp16_out, ps_stream_t stream);
+
+/* ---- chunk-list step (what FP16Adam.step does per step, fp16_cpu_adam.py:312-470,609) */
+
+/* One fused pass over a whole chunk list: for every element of every chunk
+ * read fp16 grad, fp32 param, m, v once; write fp32 param, m, v and the fp16
+ * param (over the grad) once: 28 bytes per element.  Host scalar state is
+ * advanced ONCE for the call (the chunk list is one flat tensor for the
+ * operator).  d_chunks is a device array of n_chunks descriptors. */
+int ps_adam_step_chunks(int optimizer_id, size_t step, float lr, float beta1, float beta2,
+                        float epsilon, float weight_decay, int bias_correction,
+                        const ps_chunk* d_chunks, int n_chunks, size_t chunk_numel,
+                        float loss_scale, ps_stream_t stream);
+
+/* Same pass, decided on the device: if d_state->overflow is set, every chunk's
+ * fp16 payload is restored from the fp32 master copy (fp16_cpu_adam.py:298-309)
+ * and nothing else changes; otherwise the Adam update runs with
+ * loss_scale = (float)d_state->cur_scale and t = d_state->adam_step + 1
+ * (beta^t from d_state).  Follow with ps_scaler_update(..., PS_FLAG_FROM_DEVICE). */
+int ps_adam_step_chunks_gated(int optimizer_id, float lr, float epsilon, float weight_decay,
+                              int bias_correction, const ps_chunk* d_chunks, int n_chunks,
+                              size_t chunk_numel, const ps_step_state* d_state,
+                              ps_stream_t stream);
+
+/* Unconditional restore p16 = RNE(p32) of a chunk list (FP16ChunkWriteBuffer,
+ * chunk_io_buff.py:85-151), or only when d_state->overflow is set if d_state != NULL. */
+int ps_restore_fp16_chunks(const ps_chunk* d_chunks, int n_chunks, size_t chunk_numel,
+                           const ps_step_state* d_state, ps_stream_t stream);
+
+/* Whole-buffer RNE cast (payload_fp16.copy_(payload_fp32), chunk_io_buff.py:116-126). */
+int ps_cast_fp32_to_fp16(const float* d_src, uint16_t* d_dst, size_t numel, ps_stream_t stream);
+
+/* ---- overflow probe and device-resident loss scaler --------------------- */
+
+/* Initialise *d_state (DynamicLossScaler.__init__, loss_scaler.py:107-125, plus
+ * adam_step = 0, beta^t_next = beta).  *_is_int carry the Python types of the
+ * three numbers so that loss_scale reads back as int or float like the reference. */
+int ps_state_init(ps_step_state* d_state, double init_scale, int init_is_int, double scale_factor,
+                  int factor_is_int, int64_t scale_window, double min_scale, int min_is_int,
+                  int delayed_shift, int consecutive_hysteresis, float beta1, float beta2,
+                  ps_stream_t stream);
+
+/* Set the Adam step counter (load_state_dict, fp16_cpu_adam.py:660-694) and
+ * betas; beta^t for the next step is pow(beta, adam_step + 1) evaluated in
+ * double on the host and narrowed, i.e. the reference's cold branch. */
+int ps_state_seed_step(ps_step_state* d_state, int64_t adam_step, float beta1, float beta2,
+                       ps_stream_t stream);
+
+/* Overwrite the loss-scaler fields only (restoring a checkpointed scaler). */
+int ps_state_set_scaler(ps_step_state* d_state, double cur_scale, int scale_is_int,
+                        int64_t cur_iter, int64_t last_overflow_iter, int cur_hysteresis,
+                        ps_stream_t stream);
+
+/* _has_inf_or_nan (loss_scaler.py:133-155) over fp16 data, OR-ed into
+ * d_state->overflow.  Wave shuffle + LDS reduction, one atomic per block
+ * that saw a hit.  2 bytes per element. */
+int ps_overflow_scan(const uint16_t* d_grads_fp16, size_t numel, ps_step_state* d_state,
+                     ps_stream_t stream);
+int ps_overflow_scan_f32(const float* d_grads_fp32, size_t numel, ps_step_state* d_state,
+                         ps_stream_t stream);
+int ps_overflow_scan_chunks(const ps_chunk* d_chunks, int n_chunks, size_t chunk_numel,
+                            ps_step_state* d_state, ps_stream_t stream);
+
+#define PS_FLAG_FALSE 0
+#define PS_FLAG_TRUE 1
+#define PS_FLAG_FROM_DEVICE 2
+/* DynamicLossScaler.update_scale (loss_scaler.py:158-182) on the device.
+ * flag_mode chooses the `overflow` argument: a host-given bool or the sticky
+ * device flag.  A clean step also advances adam_step and beta^t (the float
+ * running product of cpu_adam.h:158-159).  Clears the sticky flag.  If d_log
+ * is not NULL, entry [cur_iter % log_capacity] (cur_iter before the
+ * increment) records the decision. */
+int ps_scaler_update(ps_step_state* d_state, int flag_mode, ps_scale_record* d_log,
+                     int64_t log_capacity, ps_stream_t stream);
+
+/* Copy *d_state to host memory and wait for it: the only synchronising call. */
+int ps_state_read(const ps_step_state* d_state, ps_step_state* host_out, ps_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PS_ADAM_H */

@@ -1,0 +1,51 @@
+"""Builds libps_adam.so (the C-ABI HIP library) for gfx950 with hipcc, in-tree."""
+import os
+import shutil
+import subprocess
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG_DIR)
+LIB_PATH = os.path.join(PKG_DIR, "libps_adam.so")
+SOURCES = [os.path.join(PKG_DIR, "csrc", "ps_adam.hip")]
+INCLUDE = os.path.join(ROOT, "include")
+
+# -ffp-contract=off: fused multiply-adds are written out explicitly; the compiler must not add or remove any.
+# -fhip-fp32-correctly-rounded-divide-sqrt: IEEE-rounded '/' and sqrtf (hipcc's default, stated on purpose).
+# -fno-gpu-flush-denormals-to-zero? not a flag: denormals are kept with -fgpu-flush-denormals-to-zero absent.
+# packed-fp32 ops are switched off: the compiler otherwise pairs independent float ops into v_pk_* forms.
+HIPCC_FLAGS = [
+    "-O3",
+    "-std=c++17",
+    "--offload-arch=gfx950",
+    "-fPIC",
+    "-shared",
+    "-ffp-contract=off",
+    "-fhip-fp32-correctly-rounded-divide-sqrt",
+    "-fno-fast-math",
+    "-Xclang",
+    "-target-feature",
+    "-Xclang",
+    "-packed-fp32-ops",
+    "-Wall",
+    "-Wno-unused-function",
+]
+
+
+def hipcc_path():
+    for cand in (shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found: the HIP library cannot be built")
+
+
+def build(verbose=False, extra_flags=()):
+    """Compile every HIP source into patrickstar_amd/libps_adam.so; returns its path."""
+    cmd = [hipcc_path(), *HIPCC_FLAGS, *extra_flags, "-I", INCLUDE, *SOURCES, "-o", LIB_PATH]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

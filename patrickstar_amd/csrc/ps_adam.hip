@@ -1,0 +1,1044 @@
+// Chunk-wise mixed-precision Adam step for MI355X (gfx950, wave64).
+//
+// Everything here is HBM-bandwidth bound: 28 bytes move per element per step
+// (read fp16 grad + fp32 param/m/v, write fp32 param/m/v + fp16 param) for
+// ~20 flops, so the kernels are organised around 16-byte per-lane accesses,
+// enough independent loads in flight per lane to cover HBM latency, and
+// exactly one pass over the data.  No matrix cores are involved.
+//
+// Arithmetic contract (bit-exact with the explicit-intrinsic body of the
+// reference operator, patrickstar/ops/csrc/adam/cpu_adam.cpp:91-141): every
+// a*b+c the reference writes as SIMD_FMA is one __builtin_fmaf; every other
+// operation is an individually rounded IEEE binary32 op.  The file must be
+// compiled with -ffp-contract=off and with correctly rounded fp32 divide and
+// sqrt (hipcc's default), denormals preserved.
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <memory>
+#include <mutex>
+#include <unordered_map>
+
+#include "ps_adam.h"
+
+// Build-time tuning knobs.
+#ifndef PS_UNROLL
+#define PS_UNROLL 2  // 16-byte vector steps per lane per tile
+#endif
+#ifndef PS_STREAMING
+#define PS_STREAMING 1  // mark chunk payload accesses non-temporal
+#endif
+
+namespace {
+
+// ------------------------------------------------------------------ errors
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int hip_fail(hipError_t e, const char* what)
+{
+    return fail(-(int)e, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define PS_HIP(call)                                   \
+    do {                                               \
+        hipError_t e_ = (call);                        \
+        if (e_ != hipSuccess) return hip_fail(e_, #call); \
+    } while (0)
+
+// ------------------------------------------------------- host scalar state
+//
+// One object per optimizer id: the float scalars the reference keeps in
+// Adam_Optimizer (cpu_adam.h:177-197) and their update rules.
+
+struct HostAdam {
+    float alpha, beta1, beta2, eps, weight_decay;
+    float beta1_t = 1.0f, beta2_t = 1.0f;
+    size_t step = 0;
+    float bc1 = 1.0f, bc2inv = 1.0f;
+    bool adamw;
+
+    // cpu_adam.h:143-162
+    void advance(size_t s, float b1, float b2)
+    {
+        if (b1 != beta1 || b2 != beta2) {
+            step = s;
+            beta1 = b1;
+            beta2 = b2;
+            beta1_t = (float)std::pow((double)b1, (double)s);
+            beta2_t = (float)std::pow((double)b2, (double)s);
+            return;
+        }
+        step += 1;
+        if (step != s) {
+            beta1_t = (float)std::pow((double)beta1, (double)s);
+            beta2_t = (float)std::pow((double)beta2, (double)s);
+            step = s;
+        } else {
+            beta1_t = beta1_t * beta1;
+            beta2_t = beta2_t * beta2;
+        }
+    }
+    // cpu_adam.h:163-175
+    void set(float lr, float epsilon, float wd, bool bias_correction)
+    {
+        alpha = lr;
+        eps = epsilon;
+        weight_decay = wd;
+        bc1 = 1.0f;
+        bc2inv = 1.0f;
+        if (bias_correction) {
+            bc1 = 1.0f - beta1_t;
+            bc2inv = 1.0f / sqrtf(1.0f - beta2_t);
+        }
+    }
+};
+
+std::mutex g_registry_mutex;
+std::unordered_map<int, std::shared_ptr<HostAdam>> g_registry;
+
+std::shared_ptr<HostAdam> find_opt(int id)
+{
+    std::lock_guard<std::mutex> lock(g_registry_mutex);
+    auto it = g_registry.find(id);
+    return it == g_registry.end() ? nullptr : it->second;
+}
+
+// ------------------------------------------------------------ device math
+
+enum WdMode { WD_NONE = 0, WD_L2 = 1, WD_DECOUPLED = 2 };
+enum Unscale { UNSCALE_NONE = 0, UNSCALE_DIV = 1, UNSCALE_MUL = 2 };
+
+// Per-launch constants (cpu_adam.cpp:39-46 and the SIMD_SET block at :55-77).
+struct StepConsts {
+    float beta1, beta2, b1m, b2m, bc2inv, eps, step_size, wd_term;
+    float scale;  // loss scale (UNSCALE_DIV) or its exact reciprocal (UNSCALE_MUL)
+    int wd_mode;
+    int unscale;
+};
+
+// A power-of-two scale 2^k with 2^-k a normal float: g/scale == g*(1/scale)
+// bit for bit (the quotient is the same exact real number before the single
+// rounding), so the 10-instruction IEEE divide can become one multiply.
+__host__ __device__ inline bool exact_reciprocal(float s, float* inv)
+{
+    uint32_t b;
+    memcpy(&b, &s, 4);
+    uint32_t e = (b >> 23) & 0xFFu;
+    if ((b & 0x807FFFFFu) != 0 || e < 1 || e > 253) return false;
+    uint32_t r = (254u - e) << 23;
+    memcpy(inv, &r, 4);
+    return true;
+}
+
+__host__ __device__ inline void finish_consts(StepConsts& c, float lr, float beta1, float beta2,
+                                              float eps, float wd, bool adamw, float beta1_t,
+                                              float beta2_t, bool bias_correction,
+                                              float loss_scale)
+{
+    float bc1 = 1.0f, bc2inv = 1.0f;
+    if (bias_correction) {
+        bc1 = 1.0f - beta1_t;
+        bc2inv = 1.0f / sqrtf(1.0f - beta2_t);
+    }
+    c.beta1 = beta1;
+    c.beta2 = beta2;
+    c.b1m = 1.0f - beta1;
+    c.b2m = 1.0f - beta2;
+    c.bc2inv = bc2inv;
+    c.eps = eps;
+    c.step_size = (-1.0f * lr) / bc1;
+    c.wd_mode = wd > 0.0f ? (adamw ? WD_DECOUPLED : WD_L2) : WD_NONE;
+    c.wd_term = adamw ? (-1.0f * lr) * wd : wd;
+    c.unscale = UNSCALE_NONE;
+    c.scale = 1.0f;
+    if (loss_scale > 0.0f) {
+        float inv;
+        if (exact_reciprocal(loss_scale, &inv)) {
+            c.unscale = UNSCALE_MUL;
+            c.scale = inv;
+        } else {
+            c.unscale = UNSCALE_DIV;
+            c.scale = loss_scale;
+        }
+    }
+}
+
+template <int WD, int UNS>
+__device__ __forceinline__ void adam_element(const StepConsts& c, float g, float& p, float& m,
+                                             float& v)
+{
+    if (UNS == UNSCALE_DIV) g = g / c.scale;
+    if (UNS == UNSCALE_MUL) g = g * c.scale;
+    if (WD == WD_L2) g = __builtin_fmaf(p, c.wd_term, g);
+    m = m * c.beta1;
+    m = __builtin_fmaf(g, c.b1m, m);
+    v = v * c.beta2;
+    float gg = g * g;
+    v = __builtin_fmaf(gg, c.b2m, v);
+    float d = __builtin_sqrtf(v);
+    d = __builtin_fmaf(d, c.bc2inv, c.eps);
+    float u = m / d;
+    if (WD == WD_DECOUPLED) p = __builtin_fmaf(p, c.wd_term, p);
+    p = __builtin_fmaf(u, c.step_size, p);
+}
+
+__device__ __forceinline__ float half_bits_to_float(uint32_t h)
+{
+    return __half2float(__ushort_as_half((unsigned short)h));
+}
+
+// RNE binary32 -> binary16 of a value that has ALREADY been rounded to binary32.
+// The empty asm makes the float opaque at this point: without it the compiler
+// folds "convert(fma(a, b, c))" into v_fma_mixlo_f16, which rounds the exact
+// fused result straight to fp16 and so differs from RNE(fp32 param) on about
+// one element in 10^4 (double-rounding cases).
+__device__ __forceinline__ uint32_t float_to_half_bits(float f)
+{
+    asm("" : "+v"(f));
+    return (uint32_t)__half_as_ushort(__float2half_rn(f));
+}
+
+// 16-byte global accesses.  The data is touched exactly once per step, so
+// loads and stores are marked non-temporal (streaming) to keep them from
+// displacing anything useful in L2 / MALL.
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+
+// Chunk payload addresses are read from a descriptor array in memory, so the
+// compiler cannot tell their address space and would fall back to flat_*
+// instructions.  They are always device-global: say so.
+#define PS_GLOBAL __attribute__((address_space(1)))
+typedef PS_GLOBAL float4v gfloat4v;
+typedef PS_GLOBAL uint4v guint4v;
+typedef PS_GLOBAL float gfloat;
+typedef PS_GLOBAL uint16_t ghalf;
+
+__device__ __forceinline__ const gfloat4v* gvec(const float* p) { return (const gfloat4v*)(p); }
+__device__ __forceinline__ gfloat4v* gvec(float* p) { return (gfloat4v*)(p); }
+__device__ __forceinline__ const guint4v* gvec(const uint16_t* p) { return (const guint4v*)(p); }
+__device__ __forceinline__ guint4v* gvec(uint16_t* p) { return (guint4v*)(p); }
+
+__device__ __forceinline__ float4v ld_stream(const gfloat4v* p)
+{
+#if PS_STREAMING
+    return __builtin_nontemporal_load(p);
+#else
+    return *p;
+#endif
+}
+__device__ __forceinline__ uint4v ld_stream(const guint4v* p)
+{
+#if PS_STREAMING
+    return __builtin_nontemporal_load(p);
+#else
+    return *p;
+#endif
+}
+__device__ __forceinline__ void st_stream(gfloat4v* p, float4v v)
+{
+#if PS_STREAMING
+    __builtin_nontemporal_store(v, p);
+#else
+    *p = v;
+#endif
+}
+__device__ __forceinline__ void st_stream(guint4v* p, uint4v v)
+{
+#if PS_STREAMING
+    __builtin_nontemporal_store(v, p);
+#else
+    *p = v;
+#endif
+}
+
+constexpr int kBlock = 256;        // 4 waves
+constexpr int kLaneElems = 8;      // elements per lane per vector step: 16 B of fp16, 2 x 16 B of each fp32 array
+constexpr int kUnroll = PS_UNROLL; // vector steps per lane per tile
+constexpr int kTile = kBlock * kLaneElems * kUnroll;  // 4096 elements = 112 KiB of traffic per tile
+
+constexpr int UNSCALE_RUNTIME = -1;  // template value: look at StepConsts::unscale (uniform branch)
+
+// The registers of one lane for one tile.
+struct LaneTile {
+    uint4v g[kUnroll];
+    float4v p[kUnroll][2], m[kUnroll][2], v[kUnroll][2];
+    uint4v h[kUnroll];
+};
+
+template <int WD, int UNS>
+__device__ __forceinline__ void lane_math(const StepConsts& c, LaneTile& r)
+{
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            uint32_t word = r.g[u][w];
+            float g0 = half_bits_to_float(word & 0xFFFFu);
+            float g1 = half_bits_to_float(word >> 16);
+            const int e0 = 2 * w, e1 = 2 * w + 1;
+            float p0 = r.p[u][e0 >> 2][e0 & 3], m0 = r.m[u][e0 >> 2][e0 & 3],
+                  v0 = r.v[u][e0 >> 2][e0 & 3];
+            float p1 = r.p[u][e1 >> 2][e1 & 3], m1 = r.m[u][e1 >> 2][e1 & 3],
+                  v1 = r.v[u][e1 >> 2][e1 & 3];
+            adam_element<WD, UNS>(c, g0, p0, m0, v0);
+            adam_element<WD, UNS>(c, g1, p1, m1, v1);
+            r.p[u][e0 >> 2][e0 & 3] = p0;
+            r.m[u][e0 >> 2][e0 & 3] = m0;
+            r.v[u][e0 >> 2][e0 & 3] = v0;
+            r.p[u][e1 >> 2][e1 & 3] = p1;
+            r.m[u][e1 >> 2][e1 & 3] = m1;
+            r.v[u][e1 >> 2][e1 & 3] = v1;
+            r.h[u][w] = float_to_half_bits(p0) | (float_to_half_bits(p1) << 16);
+        }
+    }
+}
+
+// One tile of one chunk, fast path: the whole tile is in range and all four
+// bases are 16-byte aligned.  All loads of the tile are issued before the
+// first use so that each lane has 7 * kUnroll independent 16-byte loads in
+// flight.  Loads and stores are written once, outside any branch on the
+// arithmetic variant.
+template <int WD, int UNS>
+__device__ __forceinline__ void adam_tile_vec(const StepConsts& c, float* __restrict__ p32,
+                                              float* __restrict__ m32, float* __restrict__ v32,
+                                              uint16_t* __restrict__ h16, size_t base)
+{
+    LaneTile r;
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        size_t i = base + ((size_t)u * kBlock + threadIdx.x) * kLaneElems;
+        r.g[u] = ld_stream(gvec(h16 + i));
+        r.p[u][0] = ld_stream(gvec(p32 + i));
+        r.p[u][1] = ld_stream(gvec(p32 + i + 4));
+        r.m[u][0] = ld_stream(gvec(m32 + i));
+        r.m[u][1] = ld_stream(gvec(m32 + i + 4));
+        r.v[u][0] = ld_stream(gvec(v32 + i));
+        r.v[u][1] = ld_stream(gvec(v32 + i + 4));
+    }
+    if (UNS != UNSCALE_RUNTIME) {
+        lane_math<WD, UNS>(c, r);
+    } else if (c.unscale == UNSCALE_MUL) {
+        lane_math<WD, UNSCALE_MUL>(c, r);
+    } else if (c.unscale == UNSCALE_DIV) {
+        lane_math<WD, UNSCALE_DIV>(c, r);
+    } else {
+        lane_math<WD, UNSCALE_NONE>(c, r);
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        size_t i = base + ((size_t)u * kBlock + threadIdx.x) * kLaneElems;
+        st_stream(gvec(p32 + i), r.p[u][0]);
+        st_stream(gvec(p32 + i + 4), r.p[u][1]);
+        st_stream(gvec(m32 + i), r.m[u][0]);
+        st_stream(gvec(m32 + i + 4), r.m[u][1]);
+        st_stream(gvec(v32 + i), r.v[u][0]);
+        st_stream(gvec(v32 + i + 4), r.v[u][1]);
+        st_stream(gvec(h16 + i), r.h[u]);
+    }
+}
+
+template <int WD, int UNS>
+__device__ __forceinline__ void element_any(const StepConsts& c, float g, float& p, float& m,
+                                            float& v)
+{
+    if (UNS != UNSCALE_RUNTIME)
+        adam_element<WD, UNS>(c, g, p, m, v);
+    else if (c.unscale == UNSCALE_MUL)
+        adam_element<WD, UNSCALE_MUL>(c, g, p, m, v);
+    else if (c.unscale == UNSCALE_DIV)
+        adam_element<WD, UNSCALE_DIV>(c, g, p, m, v);
+    else
+        adam_element<WD, UNSCALE_NONE>(c, g, p, m, v);
+}
+
+// Same elements, one at a time: ragged tile ends and unaligned bases.
+template <int WD, int UNS>
+__device__ __forceinline__ void adam_tile_scalar(const StepConsts& c, float* p32, float* m32,
+                                                 float* v32, uint16_t* h16, size_t base, size_t end)
+{
+    for (size_t i = base + threadIdx.x; i < end; i += kBlock) {
+        float g = half_bits_to_float(h16[i]);
+        float p = p32[i], m = m32[i], v = v32[i];
+        element_any<WD, UNS>(c, g, p, m, v);
+        p32[i] = p;
+        m32[i] = m;
+        v32[i] = v;
+        h16[i] = (uint16_t)float_to_half_bits(p);
+    }
+}
+
+__device__ __forceinline__ bool aligned16(const void* a, const void* b, const void* c,
+                                          const void* d)
+{
+    return (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)d) & 15u) == 0;
+}
+
+template <int WD, int UNS>
+__device__ __forceinline__ void adam_tile(const StepConsts& c, const ps_chunk& ch, size_t base,
+                                          size_t chunk_numel)
+{
+    size_t end = base + kTile;
+    if (end <= chunk_numel && aligned16(ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16)) {
+        adam_tile_vec<WD, UNS>(c, ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16, base);
+    } else {
+        if (end > chunk_numel) end = chunk_numel;
+        adam_tile_scalar<WD, UNS>(c, ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16, base,
+                                  end);
+    }
+}
+
+// fp16 <- RNE(fp32) for one tile (the restore of a skipped step and the
+// stand-alone write-back).
+__device__ __forceinline__ void restore_tile(const float* __restrict__ p32,
+                                             uint16_t* __restrict__ h16, size_t base,
+                                             size_t numel)
+{
+    size_t end = base + kTile;
+    if (end <= numel && ((((uintptr_t)p32 | (uintptr_t)h16) & 15u) == 0)) {
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            size_t i = base + ((size_t)u * kBlock + threadIdx.x) * kLaneElems;
+            float4v a = ld_stream(gvec(p32 + i));
+            float4v b = ld_stream(gvec(p32 + i + 4));
+            uint4v out;
+            out[0] = float_to_half_bits(a[0]) | (float_to_half_bits(a[1]) << 16);
+            out[1] = float_to_half_bits(a[2]) | (float_to_half_bits(a[3]) << 16);
+            out[2] = float_to_half_bits(b[0]) | (float_to_half_bits(b[1]) << 16);
+            out[3] = float_to_half_bits(b[2]) | (float_to_half_bits(b[3]) << 16);
+            st_stream(gvec(h16 + i), out);
+        }
+    } else {
+        if (end > numel) end = numel;
+        for (size_t i = base + threadIdx.x; i < end; i += kBlock)
+            h16[i] = (uint16_t)float_to_half_bits(p32[i]);
+    }
+}
+
+// ---------------------------------------------------------------- kernels
+
+struct ChunkListArgs {
+    const ps_chunk* chunks;
+    int n_chunks;
+    size_t chunk_numel;
+    size_t tiles_per_chunk;
+    size_t n_tiles;
+};
+
+template <int WD, int UNS>
+__device__ __forceinline__ void chunk_list_pass(const ChunkListArgs& a, const StepConsts& c)
+{
+    for (size_t t = blockIdx.x; t < a.n_tiles; t += gridDim.x) {
+        size_t ci = t / a.tiles_per_chunk;
+        size_t base = (t - ci * a.tiles_per_chunk) * (size_t)kTile;
+        ps_chunk ch = a.chunks[ci];
+        adam_tile<WD, UNS>(c, ch, base, a.chunk_numel);
+    }
+}
+
+// Host-decided step: all scalars arrive as kernel arguments and the
+// arithmetic variant is a compile-time property of the kernel.
+template <int WD, int UNS>
+__global__ void __launch_bounds__(kBlock) adam_chunks_kernel(ChunkListArgs a, StepConsts c)
+{
+    chunk_list_pass<WD, UNS>(a, c);
+}
+
+struct GatedArgs {
+    float lr, eps, wd;
+    int adamw;
+    int bias_correction;
+};
+
+// Device-decided step: overflow flag, loss scale and beta^t come from the
+// device-resident state; a flagged step restores fp16 from fp32 instead.
+// The weight-decay form is known to the host; the unscale form depends on
+// the device-resident scale and is a uniform branch around the arithmetic.
+template <int WD>
+__global__ void __launch_bounds__(kBlock)
+    adam_chunks_gated_kernel(ChunkListArgs a, GatedArgs ga, const ps_step_state* __restrict__ st)
+{
+    if (st->overflow) {
+        for (size_t t = blockIdx.x; t < a.n_tiles; t += gridDim.x) {
+            size_t ci = t / a.tiles_per_chunk;
+            size_t base = (t - ci * a.tiles_per_chunk) * (size_t)kTile;
+            ps_chunk ch = a.chunks[ci];
+            restore_tile(ch.param_fp32, ch.param_fp16, base, a.chunk_numel);
+        }
+        return;
+    }
+    StepConsts c;
+    // The operator takes loss_scale as a C float: the Python number narrows (RNE).
+    finish_consts(c, ga.lr, st->beta1, st->beta2, ga.eps, ga.wd, ga.adamw != 0, st->beta1_t_next,
+                  st->beta2_t_next, ga.bias_correction != 0, (float)st->cur_scale);
+    chunk_list_pass<WD, UNSCALE_RUNTIME>(a, c);
+}
+
+__global__ void __launch_bounds__(kBlock)
+    restore_chunks_kernel(ChunkListArgs a, const ps_step_state* __restrict__ st)
+{
+    if (st != nullptr && !st->overflow) return;
+    for (size_t t = blockIdx.x; t < a.n_tiles; t += gridDim.x) {
+        size_t ci = t / a.tiles_per_chunk;
+        size_t base = (t - ci * a.tiles_per_chunk) * (size_t)kTile;
+        ps_chunk ch = a.chunks[ci];
+        restore_tile(ch.param_fp32, ch.param_fp16, base, a.chunk_numel);
+    }
+}
+
+__global__ void __launch_bounds__(kBlock)
+    cast_kernel(const float* __restrict__ src, uint16_t* __restrict__ dst, size_t numel,
+                size_t n_tiles)
+{
+    for (size_t t = blockIdx.x; t < n_tiles; t += gridDim.x)
+        restore_tile(src, dst, t * (size_t)kTile, numel);
+}
+
+// Flat tensor, any grad dtype, optional fp16 output (adam_update of the operator).
+// Element-wise accesses: tensors handed to the operator are views at arbitrary
+// element offsets inside a chunk, so no alignment can be assumed.
+template <int WD, bool GRAD_HALF>
+__global__ void __launch_bounds__(kBlock)
+    adam_flat_kernel(StepConsts c, float* p32, const void* grads, float* m32, float* v32,
+                     uint16_t* out16, size_t numel)
+{
+    const uint16_t* gh = static_cast<const uint16_t*>(grads);
+    const float* gf = static_cast<const float*>(grads);
+    size_t stride = (size_t)gridDim.x * kBlock;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < numel; i += stride) {
+        float g = GRAD_HALF ? half_bits_to_float(gh[i]) : gf[i];
+        float p = p32[i], m = m32[i], v = v32[i];
+        element_any<WD, UNSCALE_RUNTIME>(c, g, p, m, v);
+        p32[i] = p;
+        m32[i] = m;
+        v32[i] = v;
+        if (out16) out16[i] = (uint16_t)float_to_half_bits(p);
+    }
+}
+
+// ----------------------------------------------------------- overflow scan
+//
+// A binary16 value is inf or nan iff its five exponent bits are all set.
+// For a 32-bit word holding two halves: mask the exponents, add one unit of
+// the lowest exponent bit to each; an all-ones exponent carries into bit 15 /
+// bit 31 (the masked low half is at most 0x7C00, so its carry stops at bit 15).
+
+__device__ __forceinline__ uint32_t nonfinite_halves(uint32_t w)
+{
+    return ((w & 0x7C007C00u) + 0x04000400u) & 0x80008000u;
+}
+
+// OR across the block: shuffle butterfly inside each wave, LDS across the
+// four waves, then at most one atomic per block (none when nothing was seen).
+__device__ __forceinline__ void block_flag_commit(uint32_t hit, uint32_t* flag)
+{
+    __shared__ uint32_t wave_hit[kBlock / 64];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) hit |= (uint32_t)__shfl_xor((int)hit, off, 64);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) wave_hit[wave] = hit;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t any = 0;
+#pragma unroll
+        for (int w = 0; w < kBlock / 64; ++w) any |= wave_hit[w];
+        if (any) atomicOr(flag, 1u);
+    }
+}
+
+constexpr int kScanUnroll = 4;
+constexpr int kScanTile = kBlock * kLaneElems * kScanUnroll;  // 8192 halves = 16 KiB
+
+__device__ __forceinline__ uint32_t scan_span_f16(const uint16_t* __restrict__ h, size_t numel,
+                                                  size_t first_tile, size_t tile_stride)
+{
+    uint32_t hit = 0;
+    const bool aligned = (((uintptr_t)h) & 15u) == 0;
+    size_t n_tiles = (numel + kScanTile - 1) / kScanTile;
+    for (size_t t = first_tile; t < n_tiles; t += tile_stride) {
+        size_t base = t * (size_t)kScanTile;
+        if (aligned && base + kScanTile <= numel) {
+            uint4v w[kScanUnroll];
+#pragma unroll
+            for (int u = 0; u < kScanUnroll; ++u)
+                w[u] = ld_stream(gvec(
+                    h + base + ((size_t)u * kBlock + threadIdx.x) * kLaneElems));
+#pragma unroll
+            for (int u = 0; u < kScanUnroll; ++u)
+                hit |= nonfinite_halves(w[u][0]) | nonfinite_halves(w[u][1]) |
+                       nonfinite_halves(w[u][2]) | nonfinite_halves(w[u][3]);
+        } else {
+            size_t end = base + kScanTile < numel ? base + kScanTile : numel;
+            for (size_t i = base + threadIdx.x; i < end; i += kBlock)
+                hit |= ((h[i] & 0x7C00u) == 0x7C00u) ? 1u : 0u;
+        }
+    }
+    return hit;
+}
+
+__global__ void __launch_bounds__(kBlock)
+    scan_f16_kernel(const uint16_t* __restrict__ h, size_t numel, ps_step_state* st)
+{
+    uint32_t hit = scan_span_f16(h, numel, blockIdx.x, gridDim.x);
+    block_flag_commit(hit, &st->overflow);
+}
+
+__global__ void __launch_bounds__(kBlock)
+    scan_f32_kernel(const float* __restrict__ f, size_t numel, ps_step_state* st)
+{
+    uint32_t hit = 0;
+    const uint32_t* w = reinterpret_cast<const uint32_t*>(f);
+    size_t stride = (size_t)gridDim.x * kBlock;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < numel; i += stride)
+        hit |= ((w[i] & 0x7F800000u) == 0x7F800000u) ? 1u : 0u;
+    block_flag_commit(hit, &st->overflow);
+}
+
+__global__ void __launch_bounds__(kBlock)
+    scan_chunks_kernel(ChunkListArgs a, ps_step_state* st)
+{
+    // blocks are dealt over (chunk, tile) pairs of the whole list
+    uint32_t hit = 0;
+    size_t tiles_per_chunk = (a.chunk_numel + kScanTile - 1) / kScanTile;
+    size_t n_tiles = tiles_per_chunk * (size_t)a.n_chunks;
+    for (size_t t = blockIdx.x; t < n_tiles; t += gridDim.x) {
+        size_t ci = t / tiles_per_chunk;
+        size_t tile = t - ci * tiles_per_chunk;
+        // a one-tile span: first_tile = tile, stride large enough to stop after it
+        hit |= scan_span_f16(a.chunks[ci].param_fp16, a.chunk_numel, tile, tiles_per_chunk);
+    }
+    block_flag_commit(hit, &st->overflow);
+}
+
+// ------------------------------------------------ device-resident step state
+
+__global__ void state_init_kernel(ps_step_state* st, ps_step_state init)
+{
+    if (threadIdx.x == 0 && blockIdx.x == 0) *st = init;
+}
+
+__global__ void state_seed_kernel(ps_step_state* st, int64_t adam_step, float beta1, float beta2,
+                                  float b1t_next, float b2t_next)
+{
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        st->adam_step = adam_step;
+        st->beta1 = beta1;
+        st->beta2 = beta2;
+        st->beta1_t_next = b1t_next;
+        st->beta2_t_next = b2t_next;
+    }
+}
+
+__global__ void state_set_scaler_kernel(ps_step_state* st, double cur_scale, int scale_is_int,
+                                        int64_t cur_iter, int64_t last_overflow_iter,
+                                        int cur_hysteresis)
+{
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        st->cur_scale = cur_scale;
+        st->scale_is_int = scale_is_int;
+        st->cur_iter = cur_iter;
+        st->last_overflow_iter = last_overflow_iter;
+        st->cur_hysteresis = cur_hysteresis;
+    }
+}
+
+// DynamicLossScaler.update_scale (loss_scaler.py:158-182), one lane.
+__global__ void scaler_update_kernel(ps_step_state* st, int flag_mode, ps_scale_record* log,
+                                     int64_t log_capacity)
+{
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    ps_step_state s = *st;
+    const bool overflow = flag_mode == PS_FLAG_FROM_DEVICE ? (s.overflow != 0) : (flag_mode != 0);
+    if (overflow) {
+        if (s.delayed_shift == 1 || s.cur_hysteresis == 1) {
+            // Python: max(cur_scale / scale_factor, min_scale) -- true division gives a
+            // float; max keeps its first argument unless the second is strictly greater.
+            double q = s.cur_scale / s.scale_factor;
+            if (s.min_scale > q) {
+                s.cur_scale = s.min_scale;
+                s.scale_is_int = s.min_is_int;
+            } else {
+                s.cur_scale = q;
+                s.scale_is_int = 0;
+            }
+        } else {
+            s.cur_hysteresis -= 1;
+        }
+        s.last_overflow_iter = s.cur_iter;
+        s.skipped_steps += 1;
+    } else {
+        if (s.consecutive_hysteresis) s.cur_hysteresis = s.delayed_shift;
+        if ((s.cur_iter - s.last_overflow_iter) % s.scale_window == 0) {
+            if (!s.consecutive_hysteresis) s.cur_hysteresis = s.delayed_shift;
+            s.cur_scale = s.cur_scale * s.scale_factor;
+            s.scale_is_int = s.scale_is_int && s.factor_is_int;
+        }
+        // the step ran: state["step"] += 1 and the float running products advance
+        s.adam_step += 1;
+        s.beta1_t_next = s.beta1_t_next * s.beta1;
+        s.beta2_t_next = s.beta2_t_next * s.beta2;
+    }
+    if (log != nullptr && log_capacity > 0) {
+        ps_scale_record r;
+        r.scale_after = s.cur_scale;
+        r.overflow = overflow ? 1u : 0u;
+        r.scale_is_int = (uint32_t)s.scale_is_int;
+        log[s.cur_iter % log_capacity] = r;
+    }
+    s.cur_iter += 1;
+    s.last_skipped = overflow ? 1u : 0u;
+    s.overflow = 0;
+    *st = s;
+}
+
+// ------------------------------------------------------------ launch shapes
+
+// The grid is capped so that very long chunk lists run as a grid-stride loop
+// of resident blocks rather than millions of tiny ones: enough blocks to give
+// every CU (256 on MI355X) several rounds of full occupancy.
+int g_grid_cap = 0;
+
+int grid_cap()
+{
+    if (g_grid_cap > 0) return g_grid_cap;
+    int cap = 256 * 8 * 64;
+    if (const char* e = getenv("PS_ADAM_GRID_CAP")) {
+        int v = atoi(e);
+        if (v > 0) cap = v;
+    }
+    g_grid_cap = cap;
+    return cap;
+}
+
+unsigned grid_for(size_t n_tiles)
+{
+    size_t cap = (size_t)grid_cap();
+    size_t g = n_tiles < cap ? n_tiles : cap;
+    return (unsigned)(g ? g : 1);
+}
+
+int make_chunk_args(ChunkListArgs& a, const ps_chunk* d_chunks, int n_chunks, size_t chunk_numel)
+{
+    if (d_chunks == nullptr && n_chunks > 0) return fail(PS_ERR_BAD_ARG, "d_chunks is NULL");
+    if (n_chunks < 0) return fail(PS_ERR_BAD_ARG, "n_chunks = %d is negative", n_chunks);
+    a.chunks = d_chunks;
+    a.n_chunks = n_chunks;
+    a.chunk_numel = chunk_numel;
+    a.tiles_per_chunk = (chunk_numel + kTile - 1) / kTile;
+    a.n_tiles = a.tiles_per_chunk * (size_t)n_chunks;
+    return 0;
+}
+
+template <int WD>
+void launch_adam_chunks_wd(const ChunkListArgs& a, const StepConsts& c, hipStream_t s)
+{
+    dim3 grid(grid_for(a.n_tiles)), block(kBlock);
+    if (c.unscale == UNSCALE_MUL)
+        hipLaunchKernelGGL((adam_chunks_kernel<WD, UNSCALE_MUL>), grid, block, 0, s, a, c);
+    else if (c.unscale == UNSCALE_DIV)
+        hipLaunchKernelGGL((adam_chunks_kernel<WD, UNSCALE_DIV>), grid, block, 0, s, a, c);
+    else
+        hipLaunchKernelGGL((adam_chunks_kernel<WD, UNSCALE_NONE>), grid, block, 0, s, a, c);
+}
+
+void launch_adam_chunks(const ChunkListArgs& a, const StepConsts& c, hipStream_t s)
+{
+    if (c.wd_mode == WD_DECOUPLED)
+        launch_adam_chunks_wd<WD_DECOUPLED>(a, c, s);
+    else if (c.wd_mode == WD_L2)
+        launch_adam_chunks_wd<WD_L2>(a, c, s);
+    else
+        launch_adam_chunks_wd<WD_NONE>(a, c, s);
+}
+
+}  // namespace
+
+// ====================================================================== ABI
+
+extern "C" {
+
+int ps_abi_version(void) { return PS_ABI_VERSION; }
+
+const char* ps_last_error(void) { return g_err; }
+
+int ps_adam_create(int optimizer_id, float alpha, float beta1, float beta2, float eps,
+                   float weight_decay, int adamw_mode, int should_log)
+{
+    auto o = std::make_shared<HostAdam>();
+    o->alpha = alpha;
+    o->beta1 = beta1;
+    o->beta2 = beta2;
+    o->eps = eps;
+    o->weight_decay = weight_decay;
+    o->adamw = adamw_mode != 0;
+    {
+        std::lock_guard<std::mutex> lock(g_registry_mutex);
+        g_registry[optimizer_id] = o;
+    }
+    if (should_log) {
+        printf("Adam Optimizer #%d is created with gfx950 HIP arithmetic capability.\n",
+               optimizer_id);
+        printf("Config: alpha=%f, betas=(%f, %f), weight_decay=%f, adam_w=%d\n", alpha, beta1,
+               beta2, weight_decay, (int)(adamw_mode != 0));
+    }
+    return 0;
+}
+
+int ps_adam_destroy(int optimizer_id)
+{
+    std::lock_guard<std::mutex> lock(g_registry_mutex);
+    g_registry.erase(optimizer_id);
+    return 0;
+}
+
+int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float beta2, float epsilon,
+                   float weight_decay, int bias_correction, float* d_params, const void* d_grads,
+                   int grads_are_half, float* d_exp_avg, float* d_exp_avg_sq, size_t numel,
+                   float loss_scale, uint16_t* d_param_fp16_out, ps_stream_t stream)
+{
+    auto o = find_opt(optimizer_id);
+    if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
+    if (numel > 0 && (!d_params || !d_grads || !d_exp_avg || !d_exp_avg_sq))
+        return fail(PS_ERR_BAD_ARG, "ps_adam_update: NULL tensor pointer");
+    o->advance(step, beta1, beta2);
+    o->set(lr, epsilon, weight_decay, bias_correction != 0);
+    if (numel == 0) return 0;
+    StepConsts c;
+    finish_consts(c, o->alpha, o->beta1, o->beta2, o->eps, o->weight_decay, o->adamw, o->beta1_t,
+                  o->beta2_t, bias_correction != 0, loss_scale);
+    size_t blocks = (numel + kBlock - 1) / kBlock;
+    unsigned grid = grid_for(blocks);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+#define PS_FLAT(WD, HALF)                                                                     \
+    hipLaunchKernelGGL((adam_flat_kernel<WD, HALF>), dim3(grid), dim3(kBlock), 0, s, c, d_params, \
+                       d_grads, d_exp_avg, d_exp_avg_sq, d_param_fp16_out, numel)
+    if (grads_are_half) {
+        if (c.wd_mode == WD_DECOUPLED) PS_FLAT(WD_DECOUPLED, true);
+        else if (c.wd_mode == WD_L2) PS_FLAT(WD_L2, true);
+        else PS_FLAT(WD_NONE, true);
+    } else {
+        if (c.wd_mode == WD_DECOUPLED) PS_FLAT(WD_DECOUPLED, false);
+        else if (c.wd_mode == WD_L2) PS_FLAT(WD_L2, false);
+        else PS_FLAT(WD_NONE, false);
+    }
+#undef PS_FLAT
+    PS_HIP(hipGetLastError());
+    return 0;
+}
+
+int ps_adam_step_chunks(int optimizer_id, size_t step, float lr, float beta1, float beta2,
+                        float epsilon, float weight_decay, int bias_correction,
+                        const ps_chunk* d_chunks, int n_chunks, size_t chunk_numel,
+                        float loss_scale, ps_stream_t stream)
+{
+    auto o = find_opt(optimizer_id);
+    if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
+    ChunkListArgs a;
+    if (int rc = make_chunk_args(a, d_chunks, n_chunks, chunk_numel)) return rc;
+    o->advance(step, beta1, beta2);
+    o->set(lr, epsilon, weight_decay, bias_correction != 0);
+    if (a.n_tiles == 0) return 0;
+    StepConsts c;
+    finish_consts(c, o->alpha, o->beta1, o->beta2, o->eps, o->weight_decay, o->adamw, o->beta1_t,
+                  o->beta2_t, bias_correction != 0, loss_scale);
+    launch_adam_chunks(a, c, static_cast<hipStream_t>(stream));
+    PS_HIP(hipGetLastError());
+    return 0;
+}
+
+int ps_adam_step_chunks_gated(int optimizer_id, float lr, float epsilon, float weight_decay,
+                              int bias_correction, const ps_chunk* d_chunks, int n_chunks,
+                              size_t chunk_numel, const ps_step_state* d_state,
+                              ps_stream_t stream)
+{
+    auto o = find_opt(optimizer_id);
+    if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
+    if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
+    ChunkListArgs a;
+    if (int rc = make_chunk_args(a, d_chunks, n_chunks, chunk_numel)) return rc;
+    if (a.n_tiles == 0) return 0;
+    GatedArgs ga;
+    ga.lr = lr;
+    ga.eps = epsilon;
+    ga.wd = weight_decay;
+    ga.adamw = o->adamw ? 1 : 0;
+    ga.bias_correction = bias_correction;
+    {
+        dim3 grid(grid_for(a.n_tiles)), block(kBlock);
+        hipStream_t s = static_cast<hipStream_t>(stream);
+        const bool decay = weight_decay > 0.0f;
+        if (decay && o->adamw)
+            hipLaunchKernelGGL(adam_chunks_gated_kernel<WD_DECOUPLED>, grid, block, 0, s, a, ga, d_state);
+        else if (decay)
+            hipLaunchKernelGGL(adam_chunks_gated_kernel<WD_L2>, grid, block, 0, s, a, ga, d_state);
+        else
+            hipLaunchKernelGGL(adam_chunks_gated_kernel<WD_NONE>, grid, block, 0, s, a, ga, d_state);
+    }
+    PS_HIP(hipGetLastError());
+    return 0;
+}
+
+int ps_restore_fp16_chunks(const ps_chunk* d_chunks, int n_chunks, size_t chunk_numel,
+                           const ps_step_state* d_state, ps_stream_t stream)
+{
+    ChunkListArgs a;
+    if (int rc = make_chunk_args(a, d_chunks, n_chunks, chunk_numel)) return rc;
+    if (a.n_tiles == 0) return 0;
+    hipLaunchKernelGGL(restore_chunks_kernel, dim3(grid_for(a.n_tiles)), dim3(kBlock), 0,
+                       static_cast<hipStream_t>(stream), a, d_state);
+    PS_HIP(hipGetLastError());
+    return 0;
+}
+
+int ps_cast_fp32_to_fp16(const float* d_src, uint16_t* d_dst, size_t numel, ps_stream_t stream)
+{
+    if (numel == 0) return 0;
+    if (!d_src || !d_dst) return fail(PS_ERR_BAD_ARG, "ps_cast_fp32_to_fp16: NULL pointer");
+    size_t n_tiles = (numel + kTile - 1) / kTile;
+    hipLaunchKernelGGL(cast_kernel, dim3(grid_for(n_tiles)), dim3(kBlock), 0,
+                       static_cast<hipStream_t>(stream), d_src, d_dst, numel, n_tiles);
+    PS_HIP(hipGetLastError());
+    return 0;
+}
+
+int ps_state_init(ps_step_state* d_state, double init_scale, int init_is_int, double scale_factor,
+                  int factor_is_int, int64_t scale_window, double min_scale, int min_is_int,
+                  int delayed_shift, int consecutive_hysteresis, float beta1, float beta2,
+                  ps_stream_t stream)
+{
+    if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
+    if (scale_window <= 0)
+        return fail(PS_ERR_BAD_ARG, "scale_window = %lld must be positive", (long long)scale_window);
+    ps_step_state s;
+    memset(&s, 0, sizeof(s));
+    s.cur_scale = init_scale;
+    s.scale_is_int = init_is_int != 0;
+    s.scale_factor = scale_factor;
+    s.factor_is_int = factor_is_int != 0;
+    s.min_scale = min_scale;
+    s.min_is_int = min_is_int != 0;
+    s.cur_iter = 0;
+    s.last_overflow_iter = -1;
+    s.scale_window = scale_window;
+    s.delayed_shift = delayed_shift;
+    s.cur_hysteresis = delayed_shift;
+    s.consecutive_hysteresis = consecutive_hysteresis != 0;
+    s.beta1 = beta1;
+    s.beta2 = beta2;
+    // Adam_Optimizer starts with beta^t = 1 and step 0; the first update multiplies once.
+    s.beta1_t_next = 1.0f * beta1;
+    s.beta2_t_next = 1.0f * beta2;
+    hipLaunchKernelGGL(state_init_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
+                       d_state, s);
+    PS_HIP(hipGetLastError());
+    return 0;
+}
+
+int ps_state_seed_step(ps_step_state* d_state, int64_t adam_step, float beta1, float beta2,
+                       ps_stream_t stream)
+{
+    if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
+    if (adam_step < 0) return fail(PS_ERR_BAD_ARG, "adam_step is negative");
+    float b1t, b2t;
+    if (adam_step == 0) {
+        b1t = 1.0f * beta1;
+        b2t = 1.0f * beta2;
+    } else {
+        // a fresh native object that is first asked for step adam_step + 1 takes the pow branch
+        b1t = (float)std::pow((double)beta1, (double)(adam_step + 1));
+        b2t = (float)std::pow((double)beta2, (double)(adam_step + 1));
+    }
+    hipLaunchKernelGGL(state_seed_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
+                       d_state, adam_step, beta1, beta2, b1t, b2t);
+    PS_HIP(hipGetLastError());
+    return 0;
+}
+
+int ps_state_set_scaler(ps_step_state* d_state, double cur_scale, int scale_is_int,
+                        int64_t cur_iter, int64_t last_overflow_iter, int cur_hysteresis,
+                        ps_stream_t stream)
+{
+    if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
+    hipLaunchKernelGGL(state_set_scaler_kernel, dim3(1), dim3(64), 0,
+                       static_cast<hipStream_t>(stream), d_state, cur_scale, scale_is_int, cur_iter,
+                       last_overflow_iter, cur_hysteresis);
+    PS_HIP(hipGetLastError());
+    return 0;
+}
+
+int ps_overflow_scan(const uint16_t* d_grads_fp16, size_t numel, ps_step_state* d_state,
+                     ps_stream_t stream)
+{
+    if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
+    if (numel == 0) return 0;
+    if (!d_grads_fp16) return fail(PS_ERR_BAD_ARG, "d_grads_fp16 is NULL");
+    size_t n_tiles = (numel + kScanTile - 1) / kScanTile;
+    hipLaunchKernelGGL(scan_f16_kernel, dim3(grid_for(n_tiles)), dim3(kBlock), 0,
+                       static_cast<hipStream_t>(stream), d_grads_fp16, numel, d_state);
+    PS_HIP(hipGetLastError());
+    return 0;
+}
+
+int ps_overflow_scan_f32(const float* d_grads_fp32, size_t numel, ps_step_state* d_state,
+                         ps_stream_t stream)
+{
+    if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
+    if (numel == 0) return 0;
+    if (!d_grads_fp32) return fail(PS_ERR_BAD_ARG, "d_grads_fp32 is NULL");
+    size_t blocks = (numel + (size_t)kBlock * 16 - 1) / ((size_t)kBlock * 16);
+    hipLaunchKernelGGL(scan_f32_kernel, dim3(grid_for(blocks)), dim3(kBlock), 0,
+                       static_cast<hipStream_t>(stream), d_grads_fp32, numel, d_state);
+    PS_HIP(hipGetLastError());
+    return 0;
+}
+
+int ps_overflow_scan_chunks(const ps_chunk* d_chunks, int n_chunks, size_t chunk_numel,
+                            ps_step_state* d_state, ps_stream_t stream)
+{
+    if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
+    ChunkListArgs a;
+    if (int rc = make_chunk_args(a, d_chunks, n_chunks, chunk_numel)) return rc;
+    if (a.n_tiles == 0) return 0;
+    size_t scan_tiles = ((chunk_numel + kScanTile - 1) / kScanTile) * (size_t)n_chunks;
+    hipLaunchKernelGGL(scan_chunks_kernel, dim3(grid_for(scan_tiles)), dim3(kBlock), 0,
+                       static_cast<hipStream_t>(stream), a, d_state);
+    PS_HIP(hipGetLastError());
+    return 0;
+}
+
+int ps_scaler_update(ps_step_state* d_state, int flag_mode, ps_scale_record* d_log,
+                     int64_t log_capacity, ps_stream_t stream)
+{
+    if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
+    if (flag_mode < 0 || flag_mode > 2) return fail(PS_ERR_BAD_ARG, "flag_mode = %d", flag_mode);
+    if (d_log != nullptr && log_capacity <= 0)
+        return fail(PS_ERR_BAD_ARG, "log_capacity must be positive when d_log is given");
+    hipLaunchKernelGGL(scaler_update_kernel, dim3(1), dim3(64), 0,
+                       static_cast<hipStream_t>(stream), d_state, flag_mode, d_log, log_capacity);
+    PS_HIP(hipGetLastError());
+    return 0;
+}
+
+int ps_state_read(const ps_step_state* d_state, ps_step_state* host_out, ps_stream_t stream)
+{
+    if (!d_state || !host_out) return fail(PS_ERR_BAD_ARG, "ps_state_read: NULL pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    PS_HIP(hipMemcpyAsync(host_out, d_state, sizeof(ps_step_state), hipMemcpyDeviceToHost, s));
+    PS_HIP(hipStreamSynchronize(s));
+    return 0;
+}
+
+}  // extern "C"
