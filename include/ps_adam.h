@@ -188,6 +188,14 @@ int ps_overflow_scan_f32(const float* d_grads_fp32, size_t numel, ps_step_state*
 int ps_overflow_scan_chunks(const ps_chunk* d_chunks, int n_chunks, size_t chunk_numel,
                             ps_step_state* d_state, ps_stream_t stream);
 
+/* Backward-side producer (patrickstar/core/hook.py:200-230): copy one parameter's
+ * gradient (fp16, or fp32 rounded RNE) into its slot of the fp16 chunk and, in
+ * the same pass, OR "holds inf/nan" into d_state->overflow (skipped when
+ * d_state is NULL).  Replaces tmp_tensor.copy_(param.grad) plus
+ * optimizer.check_overflow(param) and its host sync. */
+int ps_grad_to_chunk(const void* d_grad, int grad_is_half, uint16_t* d_slot_fp16, size_t numel,
+                     ps_step_state* d_state, ps_stream_t stream);
+
 #define PS_FLAG_FALSE 0
 #define PS_FLAG_TRUE 1
 #define PS_FLAG_FROM_DEVICE 2

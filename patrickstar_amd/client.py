@@ -1,0 +1,252 @@
+"""Chunk client for one GPU: builds the four chunk lists and hands out views.
+
+MI355X has 288 GB of HBM, so by default every chunk is resident in HBM and a
+tensor "access" is just a view into its chunk payload: there is nothing to
+move, evict or fetch.  Chunks may instead be placed in pinned host memory
+(``host_chunk_policy``) to be streamed through HBM staging buffers by the
+optimizer step.
+
+Reference for the rules: ``patrickstar/core/client.py:187-309`` (append_chunk,
+append_tensor, append_tensor_as_ref), ``patrickstar/core/preprocess.py:341-435``
+(per-module registration of fp16 params and their fp32 shadows, in module
+construction order) and ``:289-320`` (initial values copied into both payloads).
+"""
+from typing import Callable, Dict, List, Optional
+
+import torch
+
+from .chunk_layout import (
+    AccessType,
+    ChunkList,
+    ChunkTensorIndex,
+    ChunkType,
+    ParamType,
+    is_param_registered,
+    register_param,
+)
+
+_DTYPE_OF_LIST = {
+    ChunkType.PARAM_FP16: torch.half,
+    ChunkType.PARAM_FP32: torch.float,
+    ChunkType.MOMENTUM: torch.float,
+    ChunkType.VARIANCE: torch.float,
+}
+
+
+class ChunkPosition:
+    """The four chunks that sit at the same place of the four lists."""
+
+    __slots__ = ("fp16", "fp32", "exp_avg", "exp_avg_sq", "on_host")
+
+    def __init__(self, fp16, fp32, exp_avg, exp_avg_sq, on_host):
+        self.fp16, self.fp32, self.exp_avg, self.exp_avg_sq, self.on_host = fp16, fp32, exp_avg, exp_avg_sq, on_host
+
+
+class PatrickStarClient:
+    def __init__(self, rank: int, default_chunk_size: int, config=None, device=None):
+        self.local_rank = rank
+        self.device = torch.device(device) if device is not None else torch.device(f"cuda:{rank}")
+        self.default_chunk_size = default_chunk_size
+        self.chunk_list = ChunkList(rank)
+        self.chunk_tensor_index = ChunkTensorIndex(default_chunk_size)
+        self.param_fp16_to_param_fp32_map: Dict[torch.nn.Parameter, torch.nn.Parameter] = {}
+        self.chunk_based_param_fp16: List[torch.nn.Parameter] = []
+        self.module = None
+        self.optimizer = None
+        self._param_idx = 0
+        # fp16 chunk ids kept in pinned host memory together with their fp32 / m / v chunks
+        self.host_fp16_chunk_ids = set()
+        # called with (position index among fp16 chunks) -> True to keep that position in host memory
+        self.host_chunk_policy: Optional[Callable[[int], bool]] = None
+        default_opts = {"with_mem_saving_comm": False, "with_mem_cache": False, "with_async_move": False}
+        self.opt_config = dict(default_opts)
+        if config is not None:
+            self.opt_config.update(config.get("opts", {}))
+            if "host_chunk_policy" in config:
+                self.host_chunk_policy = config["host_chunk_policy"]
+
+    # -- building the lists -----------------------------------------------
+    def append_chunk(self, data_type, chunk_type):
+        chunk_id = self.chunk_list.generate_chunk_id()
+        self.chunk_list.new_chunk(chunk_id, self.default_chunk_size, data_type, chunk_type)
+        self.chunk_tensor_index.add_chunk(chunk_id, chunk_type)
+        return chunk_id
+
+    def append_tensor(self, param_list, data_type, access_type, chunk_type):
+        """All of ``param_list`` goes into the last chunk of the list, or, if it does not fit, into a new one."""
+        assert isinstance(data_type, torch.dtype)
+        assert isinstance(access_type, AccessType)
+        if not self.chunk_list.is_empty(chunk_type):
+            last = self.chunk_list.last_chunk_id(chunk_type)
+            if self.chunk_tensor_index.try_insert_tensor_list(last, param_list, access_type):
+                return
+        chunk_id = self.append_chunk(data_type, chunk_type)
+        if not self.chunk_tensor_index.try_insert_tensor_list(chunk_id, param_list, access_type):
+            raise RuntimeError(
+                f"Can not append a tensor to chunk_tensor_index. "
+                f"Overall size of param list is larger than the default chunk size {self.default_chunk_size}."
+            )
+
+    def append_tensor_as_ref(self, param, data_type, access_type, chunk_type, ref_param):
+        """Place an optimizer-state tensor in the state chunk that shadows ``ref_param``'s fp16 chunk,
+        at ``ref_param``'s own offset, so that all four lists share one layout and a whole chunk
+        can be updated by a single pass."""
+        index = self.chunk_tensor_index
+        chunk_id = index.get_optimizer_state_chunk_id(ref_param, access_type, chunk_type)
+        if chunk_id is None:
+            chunk_id = self.append_chunk(data_type, chunk_type)
+        ref_info = index.get_tensor_info(ref_param.ps_attr.get_tensor_id(access_type))
+        if ref_info.numel != param.ps_attr.numel:
+            raise RuntimeError("Failed to insert optimizer param w.r.t its ref_param.")
+        tensor_id = param.ps_attr.get_tensor_id(access_type)
+        if index.tensor_id_to_chunk_id(tensor_id) is None:
+            index.add_tensor(chunk_id, tensor_id, ref_info.start_offset, ref_info.numel, param, access_type)
+        index.register_optimizer_state_chunk_id(ref_param, access_type, chunk_type, chunk_id)
+
+    def register_module_params(self, module, init_values=True):
+        """Register the parameters a module owns directly as fp16 chunk tensors with fp32 shadows."""
+        fp16_list, fp32_list = [], []
+        for name, param in module.named_parameters(recurse=False):
+            if is_param_registered(param):
+                continue
+            full = f"{module.__class__.__name__}.{name}_{self._param_idx}"
+            self._param_idx += 1
+            register_param(param, ParamType.CHUNK_BASED, torch.half, full)
+            shadow = torch.nn.Parameter(torch.tensor([], dtype=torch.float), requires_grad=False)
+            register_param(shadow, ParamType.CHUNK_BASED, torch.float, f"{full}_fp32")
+            shadow.ps_attr.reset_shape(param.shape)
+            self.param_fp16_to_param_fp32_map[param] = shadow
+            self.chunk_based_param_fp16.append(param)
+            fp16_list.append(param)
+            fp32_list.append(shadow)
+        if fp16_list:
+            self.append_tensor(fp16_list, torch.half, AccessType.DATA, ChunkType.PARAM_FP16)
+            self.append_tensor(fp32_list, torch.float, AccessType.DATA, ChunkType.PARAM_FP32)
+
+    def register_model(self, model):
+        """Register every module's own parameters in module CONSTRUCTION order (children finish
+        constructing before their parent does), copy the initial values into the fp16 and fp32
+        payloads and re-point each parameter at its fp16 chunk slot."""
+        self.module = model
+
+        def visit(m):
+            for child in m.children():
+                visit(child)
+            self.register_module_params(m)
+
+        visit(model)
+        self.allocate_payloads()
+        for p16 in self.chunk_based_param_fp16:
+            init = p16.data
+            slot16 = self.access_data(p16)
+            slot32 = self.access_data(self.param_fp16_to_param_fp32_map[p16])
+            slot32.copy_(init.to(slot32.device, torch.float))
+            slot16.copy_(slot32)
+            if slot16.device.type != "cpu":
+                p16.data = slot16
+            else:
+                p16.data = init.to(torch.half)
+        return model
+
+    def append_flat_chunks(self, n_chunks: int, used_numel_last: Optional[int] = None):
+        """Synthetic chunk lists: one flat fp16 parameter per chunk (the last may be shorter; its tail
+        stays zero).  Returns the fp16 parameters."""
+        params = []
+        for c in range(n_chunks):
+            numel = self.default_chunk_size if (c < n_chunks - 1 or used_numel_last is None) else used_numel_last
+            p16 = torch.nn.Parameter(torch.tensor([], dtype=torch.half), requires_grad=True)
+            register_param(p16, ParamType.CHUNK_BASED, torch.half, f"flat_{self._param_idx}")
+            p16.ps_attr.reset_shape(torch.Size([numel]))
+            shadow = torch.nn.Parameter(torch.tensor([], dtype=torch.float), requires_grad=False)
+            register_param(shadow, ParamType.CHUNK_BASED, torch.float, f"flat_{self._param_idx}_fp32")
+            shadow.ps_attr.reset_shape(torch.Size([numel]))
+            self._param_idx += 1
+            self.param_fp16_to_param_fp32_map[p16] = shadow
+            self.chunk_based_param_fp16.append(p16)
+            # a new chunk per parameter, also when a short one would still fit behind the previous
+            for plist, dt, ct in (([p16], torch.half, ChunkType.PARAM_FP16), ([shadow], torch.float, ChunkType.PARAM_FP32)):
+                cid = self.append_chunk(dt, ct)
+                assert self.chunk_tensor_index.try_insert_tensor_list(cid, plist, AccessType.DATA)
+            params.append(p16)
+        self.allocate_payloads()
+        return params
+
+    # -- payloads -------------------------------------------------------------
+    def _fp16_chunk_of_position(self, chunk_id):
+        """The fp16 chunk id whose list position a chunk of any list shares."""
+        ctype = self.chunk_tensor_index.chunk_id_to_chunk_type_map[chunk_id]
+        ids16 = self.chunk_tensor_index.chunk_type_to_chunk_id_list_map.get(ChunkType.PARAM_FP16, [])
+        if ctype == ChunkType.PARAM_FP16:
+            return chunk_id
+        if ctype == ChunkType.PARAM_FP32:
+            ids32 = self.chunk_tensor_index.chunk_type_to_chunk_id_list_map[ChunkType.PARAM_FP32]
+            return ids16[ids32.index(chunk_id)]
+        for ref_id, os_map in self.chunk_tensor_index.param_chunk_id_to_os_chunk_id_map.items():
+            if os_map.get(ctype) == chunk_id:
+                return ref_id
+        raise KeyError(chunk_id)
+
+    def allocate_payloads(self):
+        """Give every chunk that has none a zero-filled payload (HBM, or pinned host memory
+        for positions the host-chunk policy selects).  Safe to call repeatedly."""
+        ids16 = self.chunk_tensor_index.chunk_type_to_chunk_id_list_map.get(ChunkType.PARAM_FP16, [])
+        if self.host_chunk_policy is not None:
+            for pos, cid in enumerate(ids16):
+                if self.host_chunk_policy(pos):
+                    self.host_fp16_chunk_ids.add(cid)
+        for chunk_id, chunk in self.chunk_list.generate_chunk():
+            if chunk.payload is not None:
+                continue
+            on_host = self._fp16_chunk_of_position(chunk_id) in self.host_fp16_chunk_ids
+            if on_host:
+                chunk.allocate_payload("cpu", pin_memory=True)
+            else:
+                chunk.allocate_payload(self.device)
+
+    def chunk_ids_generator(self, chunk_type):
+        for cid in self.chunk_tensor_index.chunk_type_to_chunk_id_list_map.get(chunk_type, []):
+            yield cid
+
+    def positions(self) -> List[ChunkPosition]:
+        """Chunk ids of the four lists, position by position (needs the optimizer-state lists)."""
+        idx = self.chunk_tensor_index
+        ids16 = idx.chunk_type_to_chunk_id_list_map.get(ChunkType.PARAM_FP16, [])
+        ids32 = idx.chunk_type_to_chunk_id_list_map.get(ChunkType.PARAM_FP32, [])
+        out = []
+        for c16, c32 in zip(ids16, ids32):
+            os_map = idx.param_chunk_id_to_os_chunk_id_map.get(c16, {})
+            out.append(
+                ChunkPosition(
+                    c16, c32, os_map.get(ChunkType.MOMENTUM), os_map.get(ChunkType.VARIANCE),
+                    c16 in self.host_fp16_chunk_ids,
+                )
+            )
+        return out
+
+    # -- tensor views -----------------------------------------------------------
+    def access_data(self, param, device=None):
+        """The tensor of ``param`` inside its chunk payload (a view; nothing moves)."""
+        info = self.chunk_tensor_index.get_tensor_info(param.ps_attr.data_id())
+        payload = self.chunk_list[info.chunk_id].payload
+        if payload is None:
+            raise RuntimeError(f"chunk {info.chunk_id} has no payload; call allocate_payloads() first")
+        view = payload.narrow(0, info.start_offset, info.numel).view(param.ps_attr.shape)
+        if device is not None and torch.device(device).type != view.device.type:
+            # a copy would silently detach the caller from the chunk
+            raise RuntimeError(
+                f"{param.ps_attr.name} lives on {view.device}; this client does not move chunks (asked for {device})"
+            )
+        return view
+
+    def release_data(self, param, reset_state=None):
+        return None
+
+    def is_local_param(self, param, access_type):
+        return True
+
+    def init(self, model, optimizer):
+        self.module = model
+        self.optimizer = optimizer
+
+    def start_mem_tracer(self):
+        return None

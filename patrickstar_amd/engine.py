@@ -1,0 +1,144 @@
+"""``initialize_engine(model_func, local_rank, config)`` -> ``(engine, optimizer)`` for one MI355X.
+
+Only the configuration surface and the optimizer / loss-scaler wiring of
+``patrickstar/runtime/__init__.py:40-93`` and ``patrickstar/runtime/engine.py:45-132,204-224``
+are kept; the reference's hook-driven chunk movement, memory tracer and
+collectives are not part of this path.  With 288 GB of HBM every chunk stays
+resident: module parameters are fp16 views into the fp16 chunk payloads, so
+forward and backward are ordinary PyTorch, and ``backward`` ends by writing each
+gradient over its parameter's chunk slot while probing it for inf/nan (one
+fused pass per parameter, no host sync), which is the state ``optimizer.step()``
+expects.
+"""
+import torch
+
+from . import _lib
+from .client import PatrickStarClient
+from .fp16_adam import FP16Adam
+from .loss_scaler import DynamicLossScaler, LossScaler
+
+DEFAULT_CHUNK_SIZE = 32 * 1024 * 1024
+
+
+def default_optim_config():
+    return {
+        "type": "Adam",
+        "params": {"lr": 0.01, "betas": (0.9, 0.999), "eps": 1e-8, "weight_decay": 0, "use_hybrid_adam": True},
+    }
+
+
+def parse_config(config):
+    """Config dict -> (optimizer type, optimizer params, loss scaler, gradient clipping).
+
+    Same defaults, checks and quirks as the reference engine: the fp16 block's
+    ``hysteresis`` value is handed to the scaler as its ``scale_factor``,
+    ``delayed_shift`` is left at 1, ``loss_scale_window`` defaults to 2000.
+    """
+    default = default_optim_config()
+    if config is None:
+        return default["type"], default["params"], None, -1
+    optim_config = config.get("optimizer", default)
+    optim_type = optim_config.get("type", default["type"])
+    if optim_type not in ["Adam", "AdamW"]:
+        raise ValueError(f"Only support Adam and AdamW at the moment. Get optimizer type {optim_type}")
+    optim_params = optim_config.get("params", default["params"])
+    for key, val in default["params"].items():
+        if key not in optim_params:
+            optim_params[key] = val
+
+    if "fp16" not in config:
+        loss_scaler = None
+    else:
+        fp16 = config["fp16"]
+        assert fp16["enabled"], "Must enable fp16 training."
+        assert "loss_scale" in fp16, "Must have `loss_scale` field set."
+        if fp16["loss_scale"] == 0:
+            loss_scaler = DynamicLossScaler(
+                init_scale=2 ** fp16.get("initial_scale_power", 16),
+                scale_factor=fp16.get("hysteresis", 2),
+                scale_window=fp16.get("loss_scale_window", 2000),
+                min_scale=fp16.get("min_loss_scale", 1),
+            )
+        else:
+            loss_scaler = LossScaler(fp16["loss_scale"])
+    gradient_clipping = config["gradient_clipping"] if "gradient_clipping" in config else -1
+    return optim_type, optim_params, loss_scaler, gradient_clipping
+
+
+class PatrickStarEngine(torch.nn.Module):
+    def __init__(self, model, client, config):
+        super().__init__()
+        self.module = model
+        self.module.train()
+        self.client = client
+        optim_type, optim_params, self.loss_scaler, self.gradient_clipping = parse_config(config)
+        self.optimizer = FP16Adam(
+            self.client,
+            self.module.parameters(),
+            loss_scaler=self.loss_scaler,
+            gradient_clipping=self.gradient_clipping,
+            lr=optim_params["lr"],
+            betas=optim_params["betas"],
+            eps=optim_params["eps"],
+            weight_decay=optim_params["weight_decay"],
+            use_adamw=(optim_type == "AdamW"),
+            use_hybrid_adam=optim_params["use_hybrid_adam"],
+            scan_in_step=False,  # backward() probes while it copies the gradients
+        )
+        self.client.init(self.module, self.optimizer)
+        self.iteration_cnt_ = 0
+
+    def forward(self, *inputs, **kwargs):
+        return self.module(*inputs, **kwargs)
+
+    def _gradients_to_chunks(self):
+        """Write every gradient over its parameter's fp16 chunk slot, probing for inf/nan on the way."""
+        lib = _lib.load()
+        scaler = self.loss_scaler
+        state_ptr = scaler.state_ptr if isinstance(scaler, DynamicLossScaler) else None
+        stream = _lib.current_stream_handle()
+        for p in self.client.chunk_based_param_fp16:
+            slot = self.client.access_data(p)
+            if p.grad is None:
+                slot.zero_()
+                continue
+            g = p.grad if p.grad.is_contiguous() else p.grad.contiguous()
+            if g.dtype not in (torch.half, torch.float):
+                raise TypeError(f"gradient dtype {g.dtype} is not supported")
+            _lib.check(
+                lib.ps_grad_to_chunk(g.data_ptr(), int(g.dtype == torch.half), slot.data_ptr(), g.numel(), state_ptr, stream),
+                "ps_grad_to_chunk",
+            )
+            p.grad = None
+
+    def backward(self, loss):
+        self.optimizer.zero_grad()
+        if self.loss_scaler:
+            self.loss_scaler.backward(loss)
+        else:
+            loss.backward()
+        with torch.cuda.device(self.client.device):
+            self._gradients_to_chunks()
+        self.iteration_cnt_ += 1
+
+
+def initialize_engine(model_func, local_rank, config=None, client=None):
+    """Build the model inside a chunk client and wrap it.
+
+    Returns ``(engine, optimizer)``.  ``model_func`` is a callable returning an
+    ``nn.Module`` (or an ``nn.Module`` whose parameters were already registered
+    with ``client``).
+    """
+    if isinstance(model_func, torch.nn.Module):
+        assert client is not None, "Must pass the client when passing a nn.Module."
+        model = model_func
+    else:
+        assert callable(model_func), "model_func need to be callable."
+        cfg = config if config is not None else {}
+        default_chunk_size = cfg.get("default_chunk_size", DEFAULT_CHUNK_SIZE)
+        client = PatrickStarClient(rank=local_rank, default_chunk_size=default_chunk_size, config=cfg.get("client", None))
+        model = model_func()
+        client.register_model(model)
+    engine = PatrickStarEngine(model=model, client=client, config=config)
+    client.start_mem_tracer()
+    return (engine, engine.optimizer)

@@ -1,0 +1,347 @@
+"""FP16Adam: the chunk-wise mixed-precision Adam/AdamW step on MI355X.
+
+Keeps the constructor, attributes and ``step()`` / ``state_dict()`` /
+``load_state_dict()`` behaviour of ``patrickstar/ops/fp16_cpu_adam.py:61-694``.
+Where the reference walks the chunk lists tensor by tensor (staging each fp16
+gradient chunk, calling a CPU operator or ~10 torch kernels per tensor, then
+casting each fp32 chunk back to fp16), this implementation hands the whole
+chunk list to ONE fused HIP kernel per step through the C ABI in
+``include/ps_adam.h``.
+
+With a dynamic loss scaler the step is decided on the device: the overflow flag,
+the loss scale and the step counter live in a device struct, a flagged step
+restores the fp16 parameters from the fp32 master copy and halves the scale,
+and ``step()`` returns without synchronising.  ``state[p]["step"]`` and
+``has_overflow`` read that struct back on demand.
+"""
+import weakref
+from copy import deepcopy
+
+import torch
+
+from . import _lib
+from .chunk_layout import AccessType, ChunkType, ParamType, register_param
+from .loss_scaler import DynamicLossScaler
+
+
+def _empty_fp32_param():
+    return torch.nn.Parameter(torch.tensor([], dtype=torch.float), requires_grad=False)
+
+
+class _ParamState(dict):
+    """Per-parameter optimizer state whose ``step`` entry may live on the device."""
+
+    def __init__(self, owner):
+        super().__init__()
+        self._owner = weakref.ref(owner)
+
+    def _sync(self):
+        owner = self._owner()
+        if owner is not None:
+            owner._sync_steps()
+
+    def __getitem__(self, key):
+        if key == "step":
+            self._sync()
+        return super().__getitem__(key)
+
+    def items(self):
+        self._sync()
+        return super().items()
+
+    def values(self):
+        self._sync()
+        return super().values()
+
+
+class FP16Adam(torch.optim.Optimizer):
+    optimizer_id = 0
+
+    def __init__(
+        self,
+        client,
+        params,
+        loss_scaler=None,
+        gradient_clipping=-1,
+        lr=1e-3,
+        betas=(0.9, 0.999),
+        eps=1e-8,
+        weight_decay=0,
+        use_adamw=False,
+        amsgrad=False,
+        use_hybrid_adam=True,
+        scan_in_step=True,
+    ):
+        if not 0.0 <= lr:
+            raise ValueError("Invalid learning rate: {}".format(lr))
+        if not 0.0 <= eps:
+            raise ValueError("Invalid epsilon value: {}".format(eps))
+        if not 0.0 <= betas[0] < 1.0:
+            raise ValueError("Invalid beta parameter at index 0: {}".format(betas[0]))
+        if not 0.0 <= betas[1] < 1.0:
+            raise ValueError("Invalid beta parameter at index 1: {}".format(betas[1]))
+        if not 0.0 <= weight_decay:
+            raise ValueError("Invalid weight_decay value: {}".format(weight_decay))
+        if gradient_clipping is not None and gradient_clipping > 0:
+            raise NotImplementedError(
+                "element-wise gradient clamping (gradient_clipping > 0) is not part of the fused step yet"
+            )
+        # fail now, not at the first step, if the HIP library was never built
+        self._lib = _lib.load()
+        defaults = dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay, amsgrad=amsgrad)
+        super().__init__(params, defaults)
+        self.client = client
+        self.loss_scaler = loss_scaler
+        self.gradient_clipping = gradient_clipping
+        self.use_hybrid_adam = use_hybrid_adam
+        self.use_adamw = use_adamw
+        # True: step() itself probes every fp16 gradient chunk for inf/nan (one extra 2 B/element
+        # pass).  False: the caller has already fed the flag through check_overflow().
+        self.scan_in_step = scan_in_step
+        self._dynamic = isinstance(loss_scaler, DynamicLossScaler)
+        self._host_overflow = False
+        self._steps_dirty = False
+
+        assert len(self.param_groups) == 1, "Only support one param group at the moment."
+        # Eager state initialisation: m and v are chunk tensors shadowing the fp16 parameter chunks.
+        for group in self.param_groups:
+            for p in group["params"]:
+                st = _ParamState(self)
+                self.state[p] = st
+                dict.__setitem__(st, "betas", group["betas"])
+                dict.__setitem__(st, "lr", group["lr"])
+                dict.__setitem__(st, "weight_decay", group["weight_decay"])
+                dict.__setitem__(st, "eps", group["eps"])
+                dict.__setitem__(st, "step", 0)
+                if p.ps_attr.param_type == ParamType.TORCH_BASED:
+                    raise NotImplementedError("torch-managed (CPU embedding) parameters are outside this path")
+                if not p.ps_attr.is_local():
+                    continue
+                name = p.ps_attr.name
+                for key, ctype in (("exp_avg", ChunkType.MOMENTUM), ("exp_avg_sq", ChunkType.VARIANCE)):
+                    sp = _empty_fp32_param()
+                    register_param(sp, ParamType.CHUNK_BASED, torch.float, f"{name}.{key}")
+                    sp.ps_attr.reset_shape(p.ps_attr.shape)
+                    sp.ps_attr._is_local = p.ps_attr.is_local()
+                    dict.__setitem__(st, key, sp)
+                    # the layout of momentum and variance chunks follows the fp16 parameter chunks
+                    self.client.append_tensor_as_ref(sp, torch.float, AccessType.DATA, ctype, p)
+        self.client.allocate_payloads()
+
+        self.opt_id = FP16Adam.optimizer_id
+        FP16Adam.optimizer_id = FP16Adam.optimizer_id + 1
+        _lib.check(
+            self._lib.ps_adam_create(self.opt_id, lr, betas[0], betas[1], eps, weight_decay, int(bool(use_adamw)), 0),
+            "ps_adam_create",
+        )
+        self._created = True
+        self._tables = None
+        if self._dynamic and torch.cuda.is_available():
+            self.loss_scaler.materialize(self.client.device, betas=betas)
+
+    def __del__(self):
+        # the native object is per id and process-global: drop it with the optimizer
+        if getattr(self, "_created", False):
+            self._lib.ps_adam_destroy(self.opt_id)
+            self._created = False
+
+    def __setstate__(self, state):
+        super().__setstate__(state)
+        for group in self.param_groups:
+            group.setdefault("amsgrad", False)
+
+    # -- chunk descriptor tables -------------------------------------------------
+    def _build_tables(self):
+        """Device array of ps_chunk descriptors for HBM-resident positions; list of host-resident ones."""
+        dev_rows, host_positions = [], []
+        cl = self.client.chunk_list
+        for pos in self.client.positions():
+            if pos.exp_avg is None or pos.exp_avg_sq is None:
+                continue  # a chunk position without trainable parameters
+            if pos.on_host:
+                host_positions.append(pos)
+            else:
+                dev_rows.append(
+                    [
+                        cl[pos.fp32].payload.data_ptr(),
+                        cl[pos.exp_avg].payload.data_ptr(),
+                        cl[pos.exp_avg_sq].payload.data_ptr(),
+                        cl[pos.fp16].payload.data_ptr(),
+                    ]
+                )
+        table = None
+        if dev_rows:
+            table = torch.tensor(dev_rows, dtype=torch.int64).to(self.client.device)
+        self._tables = (table, len(dev_rows), host_positions)
+        if host_positions:
+            from .hybrid import HostChunkStreamer
+
+            self._streamer = HostChunkStreamer(self.client, host_positions)
+        return self._tables
+
+    def invalidate_tables(self):
+        """Call after re-allocating chunk payloads."""
+        self._tables = None
+
+    # -- overflow flag ------------------------------------------------------------
+    @property
+    def has_overflow(self):
+        if self._dynamic:
+            return self.loss_scaler.overflow_flag
+        return self._host_overflow
+
+    @has_overflow.setter
+    def has_overflow(self, value):
+        if self._dynamic:
+            self.loss_scaler.materialize(self.client.device)
+            off = _lib.ps_step_state.overflow.offset
+            self.loss_scaler._state[off : off + 4].view(torch.int32).fill_(1 if value else 0)
+        else:
+            self._host_overflow = bool(value)
+
+    def check_overflow(self, param):
+        """OR "param.grad holds an inf/nan" into the sticky flag (no-op for static or absent scalers).
+        Asynchronous: nothing is read back."""
+        if self._dynamic and param.grad is not None:
+            self.loss_scaler.scan(param.grad)
+
+    def check_overflow_chunks(self):
+        """Probe the fp16 gradient payload of every chunk (asynchronous)."""
+        if not self._dynamic:
+            return
+        table, n_dev, host_positions = self._tables or self._build_tables()
+        stream = _lib.current_stream_handle()
+        if n_dev:
+            _lib.check(
+                self._lib.ps_overflow_scan_chunks(
+                    table.data_ptr(), n_dev, self.client.default_chunk_size, self.loss_scaler.state_ptr, stream
+                ),
+                "ps_overflow_scan_chunks",
+            )
+        if host_positions:
+            self._streamer.scan_gradients(self.loss_scaler)
+
+    # -- the step -----------------------------------------------------------------
+    def _hyper(self):
+        for group in self.param_groups:
+            for p in group["params"]:
+                if p.requires_grad:
+                    st = self.state[p]
+                    g = dict.__getitem__
+                    return g(st, "lr"), g(st, "betas"), g(st, "eps"), g(st, "weight_decay")
+        return None
+
+    def _sync_steps(self):
+        if not self._steps_dirty:
+            return
+        self._steps_dirty = False
+        step = self.loss_scaler.adam_step
+        for group in self.param_groups:
+            for p in group["params"]:
+                if p.requires_grad:
+                    dict.__setitem__(self.state[p], "step", step)
+
+    @torch.no_grad()
+    def step(self, closure=None):
+        """One optimizer step over the whole chunk list.  Returns the closure's loss (or None)."""
+        loss = None
+        if closure is not None:
+            with torch.enable_grad():
+                loss = closure()
+        hyper = self._hyper()
+        if hyper is None:
+            return loss
+        lr, (beta1, beta2), eps, weight_decay = hyper
+        table, n_dev, host_positions = self._tables or self._build_tables()
+        chunk_numel = self.client.default_chunk_size
+        with torch.cuda.device(self.client.device):
+            stream = _lib.current_stream_handle()
+            if self._dynamic:
+                scaler = self.loss_scaler
+                if self.scan_in_step:
+                    self.check_overflow_chunks()
+                if n_dev:
+                    _lib.check(
+                        self._lib.ps_adam_step_chunks_gated(
+                            self.opt_id, lr, eps, weight_decay, 1, table.data_ptr(), n_dev, chunk_numel,
+                            scaler.state_ptr, stream,
+                        ),
+                        "ps_adam_step_chunks_gated",
+                    )
+                if host_positions:
+                    self._streamer.step_gated(self.opt_id, lr, eps, weight_decay, scaler)
+                scaler.update_scale(None)  # consume the device flag; advances state["step"] on a clean step
+                self._steps_dirty = True
+                return loss
+
+            # Static or absent scaler: the host knows every scalar (the static scaler never reports overflow).
+            step_no = None
+            for group in self.param_groups:
+                for p in group["params"]:
+                    if p.requires_grad:
+                        st = self.state[p]
+                        step_no = dict.__getitem__(st, "step") + 1
+                        dict.__setitem__(st, "step", step_no)
+            loss_scale = self.loss_scaler.loss_scale if self.loss_scaler is not None else -1
+            if n_dev:
+                _lib.check(
+                    self._lib.ps_adam_step_chunks(
+                        self.opt_id, step_no, lr, beta1, beta2, eps, weight_decay, 1, table.data_ptr(), n_dev,
+                        chunk_numel, float(loss_scale), stream,
+                    ),
+                    "ps_adam_step_chunks",
+                )
+            if host_positions:
+                self._streamer.step_static(
+                    self.opt_id, step_no, lr, beta1, beta2, eps, weight_decay, float(loss_scale), advance=(n_dev == 0)
+                )
+            if self.loss_scaler:
+                self.loss_scaler.update_scale(False)
+        return loss
+
+    # -- checkpointing --------------------------------------------------------------
+    def state_dict(self):
+        """``{"state": ..., "param_groups": ...}`` with chunk-backed m and v cloned to CPU tensors.
+        A ``"loss_scaler"`` entry is added (the reference loses its scaler state on resume)."""
+        self._sync_steps()
+        raw = super().state_dict()
+        assert len(raw["param_groups"]) == 1
+        packed = {}
+        for idx, entries in raw["state"].items():
+            packed[idx] = {}
+            for k, v in dict.items(entries):
+                if isinstance(v, torch.nn.Parameter):
+                    packed[idx][k] = self.client.access_data(v).detach().to("cpu", copy=True)
+                else:
+                    packed[idx][k] = v
+        out = {"state": packed, "param_groups": raw["param_groups"]}
+        if self.loss_scaler is not None and hasattr(self.loss_scaler, "state_dict"):
+            out["loss_scaler"] = self.loss_scaler.state_dict()
+        return out
+
+    def load_state_dict(self, state_dict):
+        state_dict = deepcopy(state_dict)
+        saved_groups = state_dict["param_groups"]
+        saved_state = state_dict["state"]
+        assert len(saved_groups) == 1
+        assert len(saved_groups[0]["params"]) == len(self.param_groups[0]["params"])
+        assert len(saved_state) == len(self.state)
+        self._sync_steps()
+        step_seen = None
+        for old_id, p in zip(saved_groups[0]["params"], self.param_groups[0]["params"]):
+            saved = saved_state[old_id]
+            mine = self.state[p]
+            assert len(saved) == len(mine)
+            for k, v in list(dict.items(mine)):
+                if isinstance(v, torch.nn.Parameter):
+                    self.client.access_data(v).copy_(saved[k])
+                else:
+                    dict.__setitem__(mine, k, saved[k])
+                    if k == "step":
+                        step_seen = saved[k]
+        if self._dynamic:
+            self.loss_scaler.materialize(self.client.device)
+            if step_seen is not None:
+                self.loss_scaler._seed_step(step_seen)
+            if "loss_scaler" in state_dict:
+                self.loss_scaler.load_state_dict(state_dict["loss_scaler"])

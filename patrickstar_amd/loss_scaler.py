@@ -1,0 +1,274 @@
+"""Loss scalers with the reference's interface, the dynamic one resident on the GPU.
+
+``LossScaler`` (static) and ``DynamicLossScaler`` keep the constructor
+arguments, methods and semantics of ``patrickstar/fp16/loss_scaler.py:46-190``.
+The dynamic scaler's state (current scale, iteration, last overflow iteration,
+hysteresis credit) lives in a 128-byte device struct (``ps_step_state``) that the
+HIP kernels read and update, so the optimizer step never has to ask the host
+whether gradients overflowed.  Reading a field from Python
+(``loss_scale``, ``cur_iter``, ...) copies the struct back, which is the only
+synchronisation point.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+
+
+class LossScaler:
+    """Static loss scale: never reports overflow, never changes
+    (``patrickstar/fp16/loss_scaler.py:46-76``)."""
+
+    def __init__(self, scale=1):
+        self.cur_scale = scale
+
+    def has_overflow(self, param):
+        return False
+
+    def _has_inf_or_nan(x):
+        return False
+
+    def update_scale(self, overflow):
+        pass
+
+    @property
+    def loss_scale(self):
+        return self.cur_scale
+
+    def backward(self, loss, retain_graph=False):
+        scaled_loss = loss * self.loss_scale
+        scaled_loss.backward(retain_graph=retain_graph)
+
+
+def _is_int(x):
+    return isinstance(x, int) and not isinstance(x, bool)
+
+
+class DynamicLossScaler:
+    """Dynamic loss scale (``patrickstar/fp16/loss_scaler.py:79-190``), device resident.
+
+    Number semantics follow Python's, as in the reference: ``loss_scale`` is an
+    ``int`` until the first halving (a true division) and the ``min_scale``
+    object's own type when the clamp bites.  Scales beyond 2**53 are not
+    representable exactly (the device keeps a binary64).
+    """
+
+    def __init__(
+        self,
+        init_scale=2**32,
+        scale_factor=2.0,
+        scale_window=1000,
+        min_scale=1,
+        delayed_shift=1,
+        consecutive_hysteresis=False,
+    ):
+        self._init = dict(
+            init_scale=init_scale,
+            scale_factor=scale_factor,
+            scale_window=scale_window,
+            min_scale=min_scale,
+            delayed_shift=delayed_shift,
+            consecutive_hysteresis=consecutive_hysteresis,
+        )
+        self.scale_factor = scale_factor
+        self.scale_window = scale_window
+        self.min_scale = min_scale
+        self.delayed_shift = delayed_shift
+        self.consecutive_hysteresis = consecutive_hysteresis
+        self._state = None  # device tensor holding one ps_step_state
+        self._log = None  # optional device tensor of ps_scale_record
+        self._log_capacity = 0
+        self._betas = (0.9, 0.999)
+
+    # -- device state ---------------------------------------------------------
+    def materialize(self, device=None, betas=None):
+        """Create the device-resident state (idempotent).  ``betas`` seeds the Adam beta^t products."""
+        if betas is not None:
+            self._betas = (float(betas[0]), float(betas[1]))
+        if self._state is not None:
+            if betas is not None:
+                self._seed_step(self.adam_step)
+            return self
+        if not torch.cuda.is_available():
+            raise RuntimeError("DynamicLossScaler keeps its state on the GPU; no GPU is available")
+        lib = _lib.load()
+        device = torch.device(device) if device is not None else torch.device("cuda", torch.cuda.current_device())
+        self._state = torch.zeros(ctypes.sizeof(_lib.ps_step_state), dtype=torch.uint8, device=device)
+        i = self._init
+        if not i["scale_window"] > 0:
+            raise ValueError(f"scale_window must be positive, got {i['scale_window']}")
+        with torch.cuda.device(device):
+            _lib.check(
+                lib.ps_state_init(
+                    self._state.data_ptr(),
+                    float(i["init_scale"]),
+                    int(_is_int(i["init_scale"])),
+                    float(i["scale_factor"]),
+                    int(_is_int(i["scale_factor"])),
+                    int(i["scale_window"]),
+                    float(i["min_scale"]),
+                    int(_is_int(i["min_scale"])),
+                    int(i["delayed_shift"]),
+                    int(bool(i["consecutive_hysteresis"])),
+                    self._betas[0],
+                    self._betas[1],
+                    _lib.current_stream_handle(),
+                ),
+                "ps_state_init",
+            )
+        return self
+
+    def _seed_step(self, adam_step):
+        _lib.check(
+            _lib.load().ps_state_seed_step(
+                self._state.data_ptr(), int(adam_step), self._betas[0], self._betas[1], _lib.current_stream_handle()
+            ),
+            "ps_state_seed_step",
+        )
+
+    def enable_log(self, capacity):
+        """Record (overflow flag, scale after) of every ``update_scale`` in a device ring of ``capacity`` entries."""
+        self.materialize()
+        self._log = torch.zeros(capacity * ctypes.sizeof(_lib.ps_scale_record), dtype=torch.uint8, device=self._state.device)
+        self._log_capacity = capacity
+
+    def read_log(self):
+        """[(overflow: bool, loss_scale)] for the iterations recorded so far (synchronises)."""
+        n = min(self.cur_iter, self._log_capacity)
+        raw = self._log.cpu().numpy().tobytes()
+        recs = (_lib.ps_scale_record * self._log_capacity).from_buffer_copy(raw)
+        start = self.cur_iter - n
+        out = []
+        for it in range(start, start + n):
+            r = recs[it % self._log_capacity]
+            out.append((bool(r.overflow), int(r.scale_after) if r.scale_is_int else float(r.scale_after)))
+        return out
+
+    def _read(self):
+        host = _lib.ps_step_state()
+        with torch.cuda.device(self._state.device):
+            _lib.check(
+                _lib.load().ps_state_read(self._state.data_ptr(), ctypes.byref(host), _lib.current_stream_handle()),
+                "ps_state_read",
+            )
+        return host
+
+    @property
+    def state_ptr(self):
+        self.materialize()
+        return self._state.data_ptr()
+
+    # -- reference attributes (read back lazily) --------------------------------
+    @property
+    def cur_scale(self):
+        if self._state is None:
+            return self._init["init_scale"]
+        s = self._read()
+        return int(s.cur_scale) if s.scale_is_int else float(s.cur_scale)
+
+    @property
+    def cur_iter(self):
+        return 0 if self._state is None else int(self._read().cur_iter)
+
+    @property
+    def last_overflow_iter(self):
+        return -1 if self._state is None else int(self._read().last_overflow_iter)
+
+    @property
+    def cur_hysteresis(self):
+        return self.delayed_shift if self._state is None else int(self._read().cur_hysteresis)
+
+    @property
+    def adam_step(self):
+        return 0 if self._state is None else int(self._read().adam_step)
+
+    @property
+    def skipped_steps(self):
+        return 0 if self._state is None else int(self._read().skipped_steps)
+
+    @property
+    def overflow_flag(self):
+        """The sticky device flag of the step being assembled (synchronises)."""
+        return False if self._state is None else bool(self._read().overflow)
+
+    @property
+    def last_step_skipped(self):
+        return False if self._state is None else bool(self._read().last_skipped)
+
+    @property
+    def loss_scale(self):
+        return self.cur_scale
+
+    # -- overflow probe -----------------------------------------------------------
+    def scan(self, x):
+        """OR "x holds an inf or nan" into the device flag; asynchronous."""
+        self.materialize(x.device)
+        if x.numel() == 0:
+            return
+        if not x.is_contiguous():
+            x = x.contiguous()
+        lib = _lib.load()
+        with torch.cuda.device(x.device):
+            if x.dtype == torch.half:
+                rc = lib.ps_overflow_scan(x.data_ptr(), x.numel(), self._state.data_ptr(), _lib.current_stream_handle())
+            elif x.dtype == torch.float:
+                rc = lib.ps_overflow_scan_f32(x.data_ptr(), x.numel(), self._state.data_ptr(), _lib.current_stream_handle())
+            else:
+                raise TypeError(f"overflow probe supports fp16 and fp32 gradients, got {x.dtype}")
+        _lib.check(rc, "ps_overflow_scan")
+
+    def has_overflow(self, param):
+        """True if ``param.grad`` holds an inf or nan (synchronises, like the reference's ``float(sum)``).
+        The sticky flag of the optimizer is left as it was."""
+        return DynamicLossScaler._has_inf_or_nan(param.grad)
+
+    @staticmethod
+    def _has_inf_or_nan(x):
+        if not x.is_cuda:
+            raise RuntimeError("the overflow probe runs on the GPU; got a tensor on " + str(x.device))
+        probe = DynamicLossScaler(init_scale=1)
+        probe.scan(x)
+        return probe.overflow_flag
+
+    # -- state machine ----------------------------------------------------------------
+    def update_scale(self, overflow):
+        """``overflow`` is a bool, or None to consume the sticky device flag; asynchronous."""
+        self.materialize()
+        mode = _lib.PS_FLAG_FROM_DEVICE if overflow is None else (_lib.PS_FLAG_TRUE if overflow else _lib.PS_FLAG_FALSE)
+        log_ptr = self._log.data_ptr() if self._log is not None else None
+        with torch.cuda.device(self._state.device):
+            _lib.check(
+                _lib.load().ps_scaler_update(
+                    self._state.data_ptr(), mode, log_ptr, self._log_capacity, _lib.current_stream_handle()
+                ),
+                "ps_scaler_update",
+            )
+
+    def backward(self, loss, retain_graph=False):
+        scaled_loss = loss * self.loss_scale
+        scaled_loss.backward(retain_graph=retain_graph)
+
+    # -- checkpointing (the reference does not save its scaler; this is an addition) ----
+    def state_dict(self):
+        if self._state is None:
+            return {"cur_scale": self._init["init_scale"], "cur_iter": 0, "last_overflow_iter": -1,
+                    "cur_hysteresis": self.delayed_shift}
+        s = self._read()
+        return {
+            "cur_scale": int(s.cur_scale) if s.scale_is_int else float(s.cur_scale),
+            "cur_iter": int(s.cur_iter),
+            "last_overflow_iter": int(s.last_overflow_iter),
+            "cur_hysteresis": int(s.cur_hysteresis),
+        }
+
+    def load_state_dict(self, sd):
+        self.materialize()
+        with torch.cuda.device(self._state.device):
+            _lib.check(
+                _lib.load().ps_state_set_scaler(
+                    self._state.data_ptr(), float(sd["cur_scale"]), int(_is_int(sd["cur_scale"])), int(sd["cur_iter"]),
+                    int(sd["last_overflow_iter"]), int(sd["cur_hysteresis"]), _lib.current_stream_handle(),
+                ),
+                "ps_state_set_scaler",
+            )
