@@ -1,0 +1,271 @@
+"""GPU parity of the overflow probe, the device-resident loss scaler and the device-gated step.
+
+Bar: skipped-step flags and the loss-scale sequence BIT-EXACT (value and Python type) against the
+oracle state machine; on a skipped step fp32 param / m / v / step untouched and fp16 == RNE(fp32).
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import patrickstar_amd as ps
+from patrickstar_amd import _lib
+from _harness import N_FULL, ChunkHarness, assert_bits_equal
+
+pytestmark = pytest.mark.gpu
+
+
+def same_typed(a, b):
+    return len(a) == len(b) and all(x == y and type(x) is type(y) for x, y in zip(a, b))
+
+
+# ---------------------------------------------------------------- probe
+
+@pytest.mark.parametrize("n", [1, 7, 2047, 2048, 8192, 8192 * 3 + 5, 1 << 20])
+def test_overflow_scan_positions_and_values(n):
+    base = (torch.randn(n, device="cuda") * 100).half()
+    assert ps.DynamicLossScaler._has_inf_or_nan(base) is False
+    assert oracle.has_inf_or_nan(base.cpu().numpy()) is False
+    for pos in sorted({0, n - 1, n // 2, max(0, n - 9)}):
+        for bad in (float("inf"), float("-inf"), float("nan")):
+            x = base.clone()
+            x[pos] = bad
+            assert ps.DynamicLossScaler._has_inf_or_nan(x) is True
+            assert oracle.has_inf_or_nan(x.cpu().numpy()) is True
+            if n > 1:  # unaligned view (2-byte offset) must see the same thing
+                assert ps.DynamicLossScaler._has_inf_or_nan(x[1:]) is (pos != 0)
+    # largest finite fp16 values are not an overflow; +inf and -inf together are
+    big = torch.full((n,), 65504.0, dtype=torch.half, device="cuda")
+    assert ps.DynamicLossScaler._has_inf_or_nan(big) is False
+    f32 = base.float()
+    assert ps.DynamicLossScaler._has_inf_or_nan(f32) is False
+    f32[n // 2] = float("nan")
+    assert ps.DynamicLossScaler._has_inf_or_nan(f32) is True
+
+
+def test_overflow_scan_empty_and_sticky_flag():
+    s = ps.DynamicLossScaler(init_scale=2**16)
+    s.scan(torch.zeros(0, dtype=torch.half, device="cuda"))
+    assert s.overflow_flag is False
+    bad = torch.tensor([1.0, float("inf")], dtype=torch.half, device="cuda")
+    good = torch.ones(5000, dtype=torch.half, device="cuda")
+    s.scan(good)
+    assert s.overflow_flag is False
+    s.scan(bad)
+    s.scan(good)  # sticky: a later clean gradient does not clear it
+    assert s.overflow_flag is True
+    s.update_scale(None)  # consumes and clears the device flag
+    assert s.overflow_flag is False and s.loss_scale == 2**16 / 2 and s.last_step_skipped is True
+
+
+# ---------------------------------------------------------------- state machine
+
+CASES = [
+    dict(init_scale=2**16, scale_factor=2, scale_window=3, min_scale=1),
+    dict(init_scale=2**16, scale_factor=2, scale_window=1000, min_scale=1),
+    dict(init_scale=4, scale_factor=2, scale_window=2, min_scale=1),
+    dict(init_scale=2**16, scale_factor=2, scale_window=1000, min_scale=2**10),
+    dict(init_scale=16, scale_factor=2, scale_window=1000, delayed_shift=2),
+    dict(init_scale=16, scale_factor=2, scale_window=2, delayed_shift=2),
+    dict(init_scale=16, scale_factor=2, scale_window=1000, delayed_shift=2, consecutive_hysteresis=True),
+    dict(init_scale=16, scale_factor=2.0, scale_window=5, delayed_shift=3, consecutive_hysteresis=True),
+    dict(init_scale=1000.0, scale_factor=3, scale_window=2),
+    dict(init_scale=2**32, scale_factor=2.0, scale_window=7, min_scale=0.5),
+]
+
+
+@pytest.mark.parametrize("kwargs", CASES)
+def test_device_scaler_matches_oracle_state_machine(kwargs):
+    rng = np.random.default_rng(len(str(kwargs)))
+    for density in (0.0, 0.1, 0.5, 1.0):
+        flags = (rng.random(120) < density).tolist()
+        dev = ps.DynamicLossScaler(**kwargs)
+        dev.enable_log(256)
+        ora = oracle.ScalerOracle(**kwargs)
+        want = []
+        for f in flags:
+            dev.update_scale(bool(f))  # asynchronous: nothing is read back in this loop
+            ora.update_scale(bool(f))
+            want.append(ora.loss_scale)
+        log = dev.read_log()
+        assert [f for f, _ in log] == [bool(f) for f in flags]
+        got = [s for _, s in log]
+        assert same_typed(got, want), (kwargs, density, got[:12], want[:12])
+        assert dev.cur_iter == ora.cur_iter and dev.last_overflow_iter == ora.last_overflow_iter
+        assert dev.cur_hysteresis == ora.cur_hysteresis
+        assert same_typed([dev.loss_scale], [ora.loss_scale])
+
+
+def test_hand_trajectory_on_device():
+    s = ps.DynamicLossScaler(init_scale=2**16, scale_factor=2, scale_window=3, min_scale=1)
+    got = []
+    for f in [0, 0, 0, 1, 0, 0, 0, 1, 1]:
+        s.update_scale(bool(f))
+        got.append(s.loss_scale)
+    assert same_typed(got, [65536, 65536, 131072, 65536.0, 65536.0, 65536.0, 131072.0, 65536.0, 32768.0])
+
+
+# ---------------------------------------------------------------- device-gated step, small, vs oracle
+
+def _inject(h, rng, step_chunks, chunk_size):
+    """Write 1..16 non-finite values into the fp16 gradient payloads at seeded positions."""
+    k = int(rng.integers(1, 17))
+    for _ in range(k):
+        c = int(rng.choice(step_chunks))
+        pos = int(rng.choice([0, chunk_size - 1, int(rng.integers(0, chunk_size))]))
+        val = [float("inf"), float("-inf"), float("nan")][int(rng.integers(0, 3))]
+        h.payloads(c)[3][pos] = val
+
+
+@pytest.mark.parametrize("window,factor,delayed", [(1000, 2, 1), (5, 2, 1), (4, 2, 2)])
+def test_gated_step_small_bit_exact_200_steps(window, factor, delayed):
+    """Config-3 shape at a size the oracle can follow: 8 chunks, 200 steps, 5 % of the steps poisoned.
+    Every step: flags, scale, fp32/m/v/fp16 bit-exact against the oracle's optimizer step."""
+    n_chunks, chunk_size, steps = 8, 2048 * 2 + 300, 200
+    kw = dict(init_scale=2**16, scale_factor=factor, scale_window=window, min_scale=1, delayed_shift=delayed)
+    scaler = ps.DynamicLossScaler(**kw)
+    h = ChunkHarness(n_chunks, chunk_size, scaler, seed=3, lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
+    scaler.enable_log(steps)
+    h.fill_state()
+    oc = h.oracle_chunks()
+    oscaler = oracle.ScalerOracle(**kw)
+    oopt = oracle.OptimizerStepOracle(oc, oscaler, lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
+    rng = np.random.default_rng(0)
+    bad_steps = set(rng.choice(steps, size=steps // 20, replace=False).tolist())
+    want_flags, want_scales = [], []
+    for step in range(steps):
+        h.fill_grads(1e-3, float(oscaler.loss_scale))
+        if step in bad_steps:
+            _inject(h, rng, list(range(n_chunks)), chunk_size)
+        for i, c in enumerate(oc):
+            c["p16"][...] = h.download(i)[3]
+        h.opt.step()
+        oopt.check_overflow()
+        skipped = oopt.step()
+        want_flags.append(skipped)
+        want_scales.append(oscaler.loss_scale)
+        if step in bad_steps or step % 25 == 0 or step == steps - 1:
+            h.compare(oc, what=f"step {step} (skipped={skipped})")
+    log = scaler.read_log()
+    assert [f for f, _ in log] == want_flags
+    assert all(want_flags[s] for s in bad_steps)
+    if window == 1000:  # no growth in 200 steps: only the poisoned steps overflow
+        assert want_flags == [s in bad_steps for s in range(steps)]
+    else:  # a growing scale also drives honest gradients over the fp16 range now and then
+        assert sum(want_flags) > len(bad_steps)
+    assert same_typed([s for _, s in log], want_scales)
+    assert h.opt.state[h.params[0]]["step"] == oopt.step_count == steps - sum(want_flags)
+    assert scaler.skipped_steps == sum(want_flags)
+    h.compare(oc, what="final")
+
+
+def test_gated_step_non_power_of_two_scale_uses_true_division():
+    kw = dict(init_scale=3000.0, scale_factor=3, scale_window=2, min_scale=1)
+    scaler = ps.DynamicLossScaler(**kw)
+    h = ChunkHarness(2, 2048 + 13, scaler, seed=8, lr=1e-3, weight_decay=0.001)
+    h.fill_state()
+    oc = h.oracle_chunks()
+    oscaler = oracle.ScalerOracle(**kw)
+    oopt = oracle.OptimizerStepOracle(oc, oscaler, lr=1e-3, weight_decay=0.001)
+    for step in range(6):
+        h.fill_grads(1e-3, min(float(oscaler.loss_scale), 3e4))
+        if step == 3:
+            h.payloads(1)[3][5] = float("nan")
+        for i, c in enumerate(oc):
+            c["p16"][...] = h.download(i)[3]
+        h.opt.step()
+        oopt.check_overflow()
+        oopt.step()
+        h.compare(oc, what=f"step {step}")
+        assert same_typed([scaler.loss_scale], [oscaler.loss_scale])
+
+
+# ---------------------------------------------------------------- BASELINE config 3 at full size
+
+def test_config3_full_size_flags_and_scale_trajectory():
+    """8 chunks of 64 Mi elements, 200 steps, a seeded 5 % of them poisoned with +-inf/nan at 1..16 positions
+    (first / last element of a chunk included).  Dynamic scaler 2^16, window 1000, "hysteresis" 2 (the engine hands it
+    over as scale_factor), min 1.  Nothing is read back inside the loop.  Checked: flags exactly on the poisoned
+    steps, scale sequence bit-exact with the oracle (ten halvings, no growth), step counter 190, and on a skipped
+    step fp32 param/m/v untouched (checksum) with fp16 == RNE(fp32)."""
+    n_chunks, steps = 8, 200
+    cfg = {"enabled": True, "loss_scale": 0, "initial_scale_power": 16, "loss_scale_window": 1000, "hysteresis": 2, "min_loss_scale": 1}
+    _, _, scaler, _ = ps.parse_config({"fp16": cfg})
+    oscaler = oracle.scaler_from_config(cfg)
+    h = ChunkHarness(n_chunks, N_FULL, scaler, seed=5, lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
+    scaler.enable_log(steps)
+    h.fill_state()
+    rng = np.random.default_rng(0)
+    bad_steps = sorted(rng.choice(steps, size=10, replace=False).tolist())
+    checks = {}
+    sums = torch.zeros(steps, 3, dtype=torch.int64, device="cuda")
+    fp16_ok = torch.ones(steps, dtype=torch.bool, device="cuda")
+
+    def checksum():
+        return torch.stack([sum(h.payloads(i)[k].view(torch.int32).sum(dtype=torch.int64) for i in range(n_chunks)) for k in range(3)])
+
+    # gradients are drawn at a fixed magnitude so that they stay finite in fp16 for every scale on the trajectory
+    grad_pool = [(torch.randn(N_FULL, device="cuda") * 1e-3 * 64).half() for _ in range(2)]
+    for step in range(steps):
+        for i in range(n_chunks):
+            h.payloads(i)[3].copy_(grad_pool[(step + i) % 2])
+        if step in bad_steps:
+            _inject(h, rng, [0, n_chunks - 1, int(rng.integers(0, n_chunks))], N_FULL)
+            before = checksum()
+        h.opt.step()
+        if step in bad_steps:
+            sums[step] = checksum() - before
+            ok = torch.tensor(True, device="cuda")
+            for i in range(n_chunks):
+                p, _, _, hh = h.payloads(i)
+                ok = ok & torch.equal(p.half(), hh)
+            fp16_ok[step] = ok
+    want_scales = []
+    for step in range(steps):
+        oscaler.update_scale(step in bad_steps)
+        want_scales.append(oscaler.loss_scale)
+    log = scaler.read_log()
+    assert [i for i, (f, _) in enumerate(log) if f] == bad_steps
+    assert same_typed([s for _, s in log], want_scales)
+    assert want_scales[-1] == 2.0**6
+    assert h.opt.state[h.params[0]]["step"] == steps - len(bad_steps) == 190
+    assert not sums.any().item(), "a skipped step must leave fp32 param / m / v untouched"
+    assert fp16_ok.all().item(), "a skipped step must restore fp16 == RNE(fp32)"
+
+
+# ---------------------------------------------------------------- checkpoint
+
+def test_state_dict_round_trip_continues_bit_exact():
+    """Semantics of the reference's checkpoint test (unitest/test_checkpoint.py:44-180): save, keep training,
+    reload, replay the same gradients -> identical results, incl. step and (an addition) the scaler state."""
+    kw = dict(init_scale=2**10, scale_factor=2, scale_window=4, min_scale=1)
+    h = ChunkHarness(2, 2048 + 99, ps.DynamicLossScaler(**kw), seed=21, lr=1e-3, weight_decay=0.01, use_adamw=True)
+    h.fill_state()
+    grads = [[(torch.randn(h.chunk_size, device="cuda") * 1e-3 * 512).half() for _ in range(2)] for _ in range(8)]
+    grads[5][1][7] = float("inf")
+
+    def run(lo, hi):
+        for s in range(lo, hi):
+            for i in range(2):
+                h.payloads(i)[3].copy_(grads[s][i])
+            h.opt.step()
+
+    run(0, 3)
+    sd = h.opt.state_dict()
+    master = [h.payloads(i)[0].clone() for i in range(2)]
+    assert sd["state"][0]["step"] == 3 and sd["state"][0]["exp_avg"].device.type == "cpu"
+    run(3, 8)
+    final = [tuple(t.clone() for t in h.payloads(i)) for i in range(2)]
+    final_scale, final_step = h.opt.loss_scaler.loss_scale, h.opt.state[h.params[0]]["step"]
+
+    h2 = ChunkHarness(2, 2048 + 99, ps.DynamicLossScaler(**kw), seed=99, lr=1e-3, weight_decay=0.01, use_adamw=True)
+    for i in range(2):
+        h2.payloads(i)[0].copy_(master[i])  # the model checkpoint restores the fp32 master params
+    h2.opt.load_state_dict(sd)
+    assert h2.opt.state[h2.params[0]]["step"] == 3
+    h, h_old = h2, h
+    run(3, 8)
+    for i in range(2):
+        for a, b in zip(h.payloads(i), final[i]):
+            assert torch.equal(a.view(torch.int16 if a.dtype == torch.half else torch.int32), b.view(torch.int16 if b.dtype == torch.half else torch.int32))
+    assert h.opt.loss_scaler.loss_scale == final_scale and h.opt.state[h.params[0]]["step"] == final_step == 7
