@@ -1,0 +1,192 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused chunk-list Adam step on one MI355X.
+
+A "step" is one optimizer.step() over the whole chunk list: one launch of the fused Adam kernel that
+reads every element's fp16 gradient and fp32 param/m/v once and writes fp32 param/m/v and the fp16 param
+once (28 algorithmic bytes per element).  Inputs are resident in HBM before the timed region.
+
+Workload (default): BASELINE config 4 -- 24 chunks of 64 Mi elements (1.61 G parameters incl. padding),
+g16 = (N(0,1e-3) * 2^12).half(), p ~ N(0,.02), m ~ N(0,1e-4), v = |N(0,1e-6)|, AdamW lr 1e-4
+betas (.9,.999) eps 1e-8 wd .01, static loss scale 2^12, first timed step t=100.
+
+Prints ONE JSON line (see the keys below).  `cpu_baseline` times the CPU oracle (a port of the reference's
+AVX/OpenMP Adam) on this host as a reported baseline only.
+"""
+import argparse
+import json
+import os
+import re
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+N_CHUNK = 64 * 1024 * 1024
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
+BYTES_PER_ELEMENT = 28  # read 2+4+4+4, write 4+4+4+2
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--chunks", type=int, default=24, help="chunk-list length (24 = the 1.5 B-parameter configuration)")
+    ap.add_argument("--chunk-size", type=int, default=N_CHUNK)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-reps", type=int, default=20)
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also launch one plain device-to-device copy of 1 Gi floats (4 GiB read, 4 GiB written) "
+                    "so that a rocprofv3 --pmc run holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
+    return ap.parse_args()
+
+
+def traffic_from_profile():
+    """HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (calibrated against a copy
+    kernel), as recorded in the committed profile summary; None when no such summary exists."""
+    path = os.path.join(ROOT, "profiles", "adam_chunks_config4_pmc.txt")
+    try:
+        m = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", open(path).read(), flags=re.M)
+        return float(m.group(1)) if m else None
+    except OSError:
+        return None
+
+
+def cpu_baseline(reps):
+    """The CPU oracle on one 64 Mi-element chunk with BASELINE config 1 inputs, all host cores of this process."""
+    import numpy as np
+
+    import oracle
+
+    n = N_CHUNK
+    rng = np.random.default_rng(0)
+    p = rng.standard_normal(n, dtype=np.float32) * np.float32(0.02)
+    m = np.zeros(n, np.float32)
+    v = np.zeros(n, np.float32)
+    g = (rng.standard_normal(n, dtype=np.float32) * np.float32(8e-3)).astype(np.float16)
+    o = oracle.AdamOracle(1e-3, 0.9, 0.999, 1e-6, 0.0, False)
+    isa = o.update(1, 1e-3, 0.9, 0.999, 1e-6, 0.0, True, p, g, m, v, 8.0)
+    o.update(2, 1e-3, 0.9, 0.999, 1e-6, 0.0, True, p, g, m, v, 8.0)
+    best = float("inf")
+    for r in range(reps):
+        t0 = time.perf_counter()
+        o.update(3 + r, 1e-3, 0.9, 0.999, 1e-6, 0.0, True, p, g, m, v, 8.0)
+        best = min(best, time.perf_counter() - t0)
+    try:
+        cores = len(os.sched_getaffinity(0))
+    except AttributeError:
+        cores = os.cpu_count()
+    omp = os.environ.get("OMP_NUM_THREADS")
+    if omp and omp.isdigit():
+        cores = min(cores, int(omp))
+    return {
+        "value": n / best,
+        "unit": "params/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"1 chunk of {n} elements (BASELINE config 1 inputs, static scale 8), best of {reps} steps after 2 warm-up; "
+        f"oracle code path {['', 'scalar', 'AVX2', 'AVX-512'][isa]}; 26 B/element -> {26 * n / best / 1e9:.0f} GB/s",
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (every GPU box here has one GPU)")
+    import torch
+
+    import patrickstar_amd as ps
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    C, N = args.chunks, args.chunk_size
+
+    client = ps.PatrickStarClient(0, N)
+    params = client.append_flat_chunks(C)
+    opt = ps.FP16Adam(client, params, loss_scaler=ps.LossScaler(2**12), lr=1e-4, betas=(0.9, 0.999), eps=1e-8,
+                      weight_decay=0.01, use_adamw=True)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(0)
+    cl = client.chunk_list
+    grads = []
+    for pos in client.positions():
+        cl[pos.fp32].payload.normal_(0, 0.02, generator=gen)
+        cl[pos.exp_avg].payload.normal_(0, 1e-4, generator=gen)
+        cl[pos.exp_avg_sq].payload.normal_(0, 1e-6, generator=gen).abs_()
+        tmp = torch.empty(N, device=dev).normal_(0, 1e-3, generator=gen).mul_(2.0**12)
+        cl[pos.fp16].payload.copy_(tmp)
+        del tmp
+    # the step overwrites the fp16 gradients with fp16 parameters; later steps then read those as "gradients" of the
+    # same magnitude class (|p| ~ 0.02 vs |g*scale| ~ 4), which changes values, not the work done per element
+    for p in params:
+        dict.__setitem__(opt.state[p], "step", 99 - args.warmup)
+
+    if args.calibration_copy:
+        src = torch.empty(1 << 30, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    for _ in range(args.warmup):
+        opt.step()
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        starts[i].record()  # on torch's current stream, the stream the kernel is launched on
+        opt.step()
+        ends[i].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kernel_ms = [s.elapsed_time(e) for s, e in zip(starts, ends)]
+    avg_kernel_ms = sum(kernel_ms) / len(kernel_ms)
+    ms_per_step = wall * 1e3 / args.steps
+    elements = C * N
+    algorithmic = BYTES_PER_ELEMENT * elements
+    achieved = algorithmic / (avg_kernel_ms * 1e-3) / 1e9
+
+    out = {
+        "metric": "Adam params/sec, fused chunk-list optimizer step, 1 GPU",
+        "value": elements / (ms_per_step * 1e-3),
+        "unit": "params/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": f"BASELINE config 4: {C} chunks x {N} elements ({elements} parameters incl. padding) resident in HBM, "
+            "AdamW lr 1e-4 betas (0.9,0.999) eps 1e-8 wd 0.01, static loss scale 2^12, fp16 grads -> fp32 p/m/v + fp16 params",
+            "chunks": C,
+            "chunk_numel": N,
+            "kernel": "adam_chunks_kernel<decoupled, exact-reciprocal unscale>",
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": traffic_from_profile() if (C, N) == (24, N_CHUNK) else None,
+            "algorithmic_bytes_per_launch": algorithmic,
+            "avg_kernel_ms": avg_kernel_ms,
+            "min_kernel_ms": min(kernel_ms),
+        },
+    }
+    del opt, client, params, grads
+    torch.cuda.empty_cache()
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(args.cpu_reps)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,212 @@
+"""CPU-only tests of the host side: chunk layout known answers, config parsing, argument checks,
+and that the C-ABI library loads and exports every symbol the header declares (no compute calls)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import patrickstar_amd as ps
+from patrickstar_amd import _lib
+from patrickstar_amd.chunk_layout import AccessType, ChunkTensorIndex, ChunkType, ParamType, register_param
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _param(n, name):
+    p = torch.nn.Parameter(torch.zeros(n))
+    register_param(p, ParamType.CHUNK_BASED, torch.float, name)
+    return p
+
+
+def test_first_fit_known_answers():
+    """The expectations of the reference's unitest/test_chunk_data.py:51-102: sizes 10, 15, 5 in a 40-element chunk
+    land at 0, 10, 25; 100 is rejected; re-inserting is a no-op; a second chunk starts at 0."""
+    idx = ChunkTensorIndex(40)
+    p1 = _param(10, "param1")
+    idx.add_tensor(0, p1.ps_attr.data_id(), 0, p1.numel(), p1, AccessType.DATA)
+    assert idx.tensor_id_to_chunk_id(p1.ps_attr.data_id()) == 0
+    assert idx.get_chunk_id(p1, AccessType.DATA) == 0
+    p2 = _param(15, "param2")
+    assert idx.get_chunk_id(p2, AccessType.DATA) is None
+    assert idx.try_insert_tensor(0, p2, AccessType.DATA)
+    assert idx.get_tensor_info(p2.ps_attr.data_id()).start_offset == 10
+    p3 = _param(5, "param3")
+    assert idx.try_insert_tensor(0, p3, AccessType.DATA)
+    assert idx.get_tensor_info(p3.ps_attr.data_id()).start_offset == 25
+    p4 = _param(100, "param4")
+    assert not idx.try_insert_tensor(0, p4, AccessType.DATA)
+    p5 = _param(13, "param5")
+    assert idx.try_insert_tensor(1, p5, AccessType.DATA)
+    assert idx.get_tensor_info(p5.ps_attr.data_id()).start_offset == 0
+    assert idx.try_insert_tensor(1, p5, AccessType.DATA)
+    assert idx.get_tensor_info(p5.ps_attr.data_id()).start_offset == 0
+    assert not idx.try_insert_tensor(1, _param(1000, "param6"), AccessType.DATA)
+    assert [i.start_offset for i in idx.generate_tensor_info_in_order(0)] == [0, 10, 25]
+    assert idx.used_numel(0) == 30
+
+
+def test_first_fit_fills_gaps_and_list_insert_is_atomic():
+    idx = ChunkTensorIndex(40)
+    a, b, c = _param(10, "a"), _param(10, "b"), _param(10, "c")
+    for p in (a, b, c):
+        assert idx.try_insert_tensor(0, p, AccessType.DATA)
+    idx.delete_tensor(0, b, AccessType.DATA)  # hole at [10, 20)
+    big, small = _param(11, "big"), _param(6, "small")
+    assert idx.try_insert_tensor(0, big, AccessType.DATA) is False or idx.get_tensor_info(big.ps_attr.data_id()).start_offset == 30
+    assert idx.try_insert_tensor(0, small, AccessType.DATA)
+    assert idx.get_tensor_info(small.ps_attr.data_id()).start_offset == 10
+    # atomic list insert: the second member does not fit -> the first is rolled back
+    idx2 = ChunkTensorIndex(20)
+    x, y = _param(15, "x"), _param(10, "y")
+    assert not idx2.try_insert_tensor_list(0, [x, y], AccessType.DATA)
+    assert idx2.get_chunk_id(x, AccessType.DATA) is None and idx2.used_numel(0) == 0
+    assert idx2.try_insert_tensor_list(0, [x], AccessType.DATA)
+
+
+class _Tiny(torch.nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.a = torch.nn.Linear(4, 6)  # 24 + 6
+        self.b = torch.nn.Linear(6, 2)  # 12 + 2
+        self.scale = torch.nn.Parameter(torch.ones(3))
+
+
+def test_client_packs_modules_in_construction_order_and_mirrors_offsets():
+    client = ps.PatrickStarClient(0, 32, device="cpu")
+    model = _Tiny()
+    w0 = model.a.weight.detach().clone()
+    client.register_model(model)
+    idx = client.chunk_tensor_index
+    ids16 = list(client.chunk_ids_generator(ChunkType.PARAM_FP16))
+    ids32 = list(client.chunk_ids_generator(ChunkType.PARAM_FP32))
+    assert len(ids16) == len(ids32) == 2
+    # children first (a: 30 elements fills chunk 0 up to 30; b: 14 does not fit behind it -> chunk 1), then the parent's own (3)
+    info = lambda p: idx.get_tensor_info(p.ps_attr.data_id())
+    assert (info(model.a.weight).chunk_id, info(model.a.weight).start_offset) == (ids16[0], 0)
+    assert (info(model.a.bias).chunk_id, info(model.a.bias).start_offset) == (ids16[0], 24)
+    assert (info(model.b.weight).chunk_id, info(model.b.weight).start_offset) == (ids16[1], 0)
+    assert (info(model.b.bias).chunk_id, info(model.b.bias).start_offset) == (ids16[1], 12)
+    assert (info(model.scale).chunk_id, info(model.scale).start_offset) == (ids16[1], 14)
+    # fp32 shadows share the layout; payloads hold the initial values, the tail is zero
+    sh = client.param_fp16_to_param_fp32_map[model.a.weight]
+    assert (info(sh).chunk_id, info(sh).start_offset) == (ids32[0], 0)
+    assert torch.equal(client.access_data(sh), w0)
+    assert torch.equal(client.access_data(model.a.weight), w0.half())
+    assert not client.chunk_list[ids16[0]].payload[30:].any()
+    assert client.chunk_list[ids16[0]].payload.dtype == torch.half and client.chunk_list[ids32[0]].payload.dtype == torch.float
+
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("HIP library not built")
+    opt = ps.FP16Adam(client, model.parameters(), lr=1e-3)
+    # optimizer() walks parameters in definition order (scale first), yet m/v sit at their parameter's own offset
+    for p in model.parameters():
+        for key, ctype in (("exp_avg", ChunkType.MOMENTUM), ("exp_avg_sq", ChunkType.VARIANCE)):
+            sp = dict.__getitem__(opt.state[p], key)
+            assert info(sp).start_offset == info(p).start_offset
+            assert info(sp).chunk_id == idx.get_optimizer_state_chunk_id(p, AccessType.DATA, ctype)
+            assert not client.access_data(sp).any()
+    pos = client.positions()
+    assert len(pos) == 2 and all(x.exp_avg is not None and x.exp_avg_sq is not None and not x.on_host for x in pos)
+    assert opt.state[model.scale]["step"] == 0 and opt.state[model.scale]["lr"] == 1e-3
+    sd = opt.state_dict()
+    assert set(sd) == {"state", "param_groups"} and sd["state"][0]["exp_avg"].shape == model.scale.shape
+
+
+def test_oversized_module_is_rejected():
+    client = ps.PatrickStarClient(0, 16, device="cpu")
+    with pytest.raises(RuntimeError, match="larger than the default chunk size"):
+        client.register_model(torch.nn.Linear(8, 8))
+
+
+def test_config_parsing_defaults_and_quirks():
+    t, p, scaler, clip = ps.parse_config(None)
+    assert (t, scaler, clip) == ("Adam", None, -1)
+    assert p == {"lr": 0.01, "betas": (0.9, 0.999), "eps": 1e-8, "weight_decay": 0, "use_hybrid_adam": True}
+    t, p, scaler, clip = ps.parse_config({"optimizer": {"type": "AdamW", "params": {"lr": 1e-4}}, "gradient_clipping": 1.0})
+    assert t == "AdamW" and p["lr"] == 1e-4 and p["betas"] == (0.9, 0.999) and scaler is None and clip == 1.0
+    # the README configuration of the reference (README.md:59-92)
+    cfg = {
+        "optimizer": {"type": "Adam", "params": {"lr": 0.001, "betas": (0.9, 0.999), "eps": 1e-6, "weight_decay": 0, "use_hybrid_adam": True}},
+        "fp16": {"enabled": True, "loss_scale": 0, "initial_scale_power": 2**3, "loss_scale_window": 1000, "hysteresis": 2, "min_loss_scale": 1},
+        "default_chunk_size": 64 * 1024 * 1024, "release_after_init": True, "use_cpu_embedding": False,
+    }
+    t, p, scaler, clip = ps.parse_config(cfg)
+    assert isinstance(scaler, ps.DynamicLossScaler)
+    assert scaler.loss_scale == 2**8 and scaler.scale_factor == 2 and scaler.scale_window == 1000
+    assert scaler.delayed_shift == 1 and scaler.consecutive_hysteresis is False and scaler.min_scale == 1
+    # "hysteresis" feeds the scale FACTOR; the window defaults to 2000
+    _, _, s2, _ = ps.parse_config({"fp16": {"enabled": True, "loss_scale": 0, "hysteresis": 4}})
+    assert s2.scale_factor == 4 and s2.delayed_shift == 1 and s2.scale_window == 2000 and s2.loss_scale == 2**16
+    _, _, s3, _ = ps.parse_config({"fp16": {"enabled": True, "loss_scale": 128}})
+    assert isinstance(s3, ps.LossScaler) and s3.loss_scale == 128 and s3.has_overflow(None) is False
+    s3.update_scale(True)
+    assert s3.loss_scale == 128
+    with pytest.raises(ValueError, match="Only support Adam and AdamW"):
+        ps.parse_config({"optimizer": {"type": "SGD"}})
+    with pytest.raises(AssertionError, match="Must enable fp16"):
+        ps.parse_config({"fp16": {"enabled": False, "loss_scale": 0}})
+    with pytest.raises(AssertionError, match="loss_scale"):
+        ps.parse_config({"fp16": {"enabled": True}})
+
+
+@pytest.mark.skipif(not os.path.exists(_lib.LIB_PATH), reason="HIP library not built")
+def test_fp16adam_argument_checks():
+    client = ps.PatrickStarClient(0, 64, device="cpu")
+    params = client.append_flat_chunks(1)
+    for kw, msg in [
+        (dict(lr=-1.0), "Invalid learning rate"),
+        (dict(eps=-1e-8), "Invalid epsilon value"),
+        (dict(betas=(1.0, 0.999)), "Invalid beta parameter at index 0"),
+        (dict(betas=(0.9, -0.1)), "Invalid beta parameter at index 1"),
+        (dict(weight_decay=-0.1), "Invalid weight_decay value"),
+    ]:
+        with pytest.raises(ValueError, match=msg):
+            ps.FP16Adam(client, params, **kw)
+    with pytest.raises(AssertionError, match="one param group"):
+        ps.FP16Adam(client, [{"params": params[:1]}, {"params": [torch.nn.Parameter(torch.zeros(1))]}])
+    first = ps.FP16Adam.optimizer_id
+    a = ps.FP16Adam(client, params)
+    assert a.opt_id == first and ps.FP16Adam.optimizer_id == first + 1
+    assert a.has_overflow is False and a.loss_scaler is None
+    del a
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    """Every function declared in include/ps_adam.h is exported by libps_adam.so and bound by the Python loader."""
+    header = open(os.path.join(ROOT, "include", "ps_adam.h")).read()
+    body = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(ps_[a-z0-9_]+)\s*\(", body))
+    assert len(declared) >= 17
+    assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
+    assert os.path.exists(_lib.LIB_PATH), "build the HIP library first (python -m patrickstar_amd.build)"
+    lib = _lib.load()
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.ps_abi_version() == 1
+    # host-only entry points: registry and argument checks work without a GPU
+    assert lib.ps_adam_create(77, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, 0) == 0
+    assert lib.ps_adam_destroy(77) == 0
+    assert lib.ps_scaler_update(None, 0, None, 0, None) == _lib.PS_ERR_BAD_ARG
+    assert b"d_state" in lib.ps_last_error()
+    assert lib.ps_state_init(None, 1.0, 1, 2.0, 1, 10, 1.0, 1, 1, 0, 0.9, 0.999, None) == _lib.PS_ERR_BAD_ARG
+    assert ctypes.sizeof(_lib.ps_step_state) == 128 and ctypes.sizeof(_lib.ps_chunk) == 32
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(_lib.HipLibraryMissing, match="no CPU fallback"):
+        _lib.load()
+    client = ps.PatrickStarClient(0, 64, device="cpu")
+    with pytest.raises(_lib.HipLibraryMissing):
+        ps.FP16Adam(client, client.append_flat_chunks(1))
+
+
+def test_dynamic_scaler_needs_a_gpu_for_anything_but_its_configuration():
+    s = ps.DynamicLossScaler(init_scale=2**8, scale_window=10)
+    assert s.loss_scale == 2**8 and s.cur_iter == 0 and s.last_overflow_iter == -1 and s.cur_hysteresis == 1
+    if not torch.cuda.is_available():
+        with pytest.raises(RuntimeError, match="GPU"):
+            s.update_scale(True)
