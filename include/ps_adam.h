@@ -11,9 +11,11 @@
  * (loss_scaler.py:158-182).
  *
  * Conventions
- *   - plain C types only; every pointer named d_* (and every pointer inside
- *     ps_chunk) is a DEVICE address unless stated otherwise; the library never
- *     allocates, frees or keeps tensor memory.
+ *   - plain C types only; every pointer named d_* (and every address inside a
+ *     ps_chunk, unless stated otherwise) is a DEVICE address; arrays of
+ *     ps_chunk descriptors themselves are ordinary HOST arrays that the call
+ *     reads before it returns (descriptors reach the kernels as kernel
+ *     arguments); the library never allocates, frees or keeps tensor memory.
  *   - every entry point that takes a stream only ENQUEUES work on it and
  *     returns; nothing here synchronises with the host except ps_state_read.
  *   - return value: 0 on success; a negative value on failure
@@ -133,10 +135,10 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
  * read fp16 grad, fp32 param, m, v once; write fp32 param, m, v and the fp16
  * param (over the grad) once: 28 bytes per element.  Host scalar state is
  * advanced ONCE for the call (the chunk list is one flat tensor for the
- * operator).  d_chunks is a device array of n_chunks descriptors. */
+ * operator).  chunks is a host array of n_chunks descriptors. */
 int ps_adam_step_chunks(int optimizer_id, size_t step, float lr, float beta1, float beta2,
                         float epsilon, float weight_decay, int bias_correction,
-                        const ps_chunk* d_chunks, int n_chunks, size_t chunk_numel,
+                        const ps_chunk* chunks, int n_chunks, size_t chunk_numel,
                         float loss_scale, ps_stream_t stream);
 
 /* Same pass, decided on the device: if d_state->overflow is set, every chunk's
@@ -145,14 +147,47 @@ int ps_adam_step_chunks(int optimizer_id, size_t step, float lr, float beta1, fl
  * loss_scale = (float)d_state->cur_scale and t = d_state->adam_step + 1
  * (beta^t from d_state).  Follow with ps_scaler_update(..., PS_FLAG_FROM_DEVICE). */
 int ps_adam_step_chunks_gated(int optimizer_id, float lr, float epsilon, float weight_decay,
-                              int bias_correction, const ps_chunk* d_chunks, int n_chunks,
+                              int bias_correction, const ps_chunk* chunks, int n_chunks,
                               size_t chunk_numel, const ps_step_state* d_state,
                               ps_stream_t stream);
 
 /* Unconditional restore p16 = RNE(p32) of a chunk list (FP16ChunkWriteBuffer,
  * chunk_io_buff.py:85-151), or only when d_state->overflow is set if d_state != NULL. */
-int ps_restore_fp16_chunks(const ps_chunk* d_chunks, int n_chunks, size_t chunk_numel,
+int ps_restore_fp16_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_numel,
                            const ps_step_state* d_state, ps_stream_t stream);
+
+/* ---- chunks that live in pinned host memory (hybrid placement) ------------
+ *
+ * The reference updates host-resident chunks with the CPU operator after
+ * staging their fp16 gradients (chunk_io_buff.py:214-255) and casts the result
+ * back through a GPU buffer (chunk_io_buff.py:85-151).  Here such chunks are
+ * streamed through HBM instead: for chunk k, slot k % n_slots of `staging`
+ * receives fp16 grad + fp32 param/m/v by hipMemcpyAsync on a side stream
+ * (14 B/element), the fused kernel runs on it, and fp32 param/m/v + fp16 param
+ * go back on another side stream (14 B/element); events order the three, so
+ * with n_slots >= 2 the copies of neighbouring chunks overlap the kernel.
+ *   host_chunks  host array of descriptors whose addresses are PINNED HOST memory
+ *   staging      host array of n_slots (1..8) descriptors of DEVICE buffers of
+ *                chunk_numel elements each, owned by the caller
+ *   advance_state  0 when ps_adam_step_chunks already advanced the operator's
+ *                step scalars for this optimizer step (resident chunks first,
+ *                host chunks second: both halves must see the same beta^t)
+ *   d_state      NULL: host-decided step with loss_scale; else device-gated
+ *                exactly like ps_adam_step_chunks_gated (loss_scale ignored)
+ * Work queued on `stream` before the call is waited for; work queued on it
+ * afterwards waits for the last write-back.  The call itself never blocks.
+ * Calls that overlap in time on one device share the side streams and race. */
+int ps_adam_step_host_chunks(int optimizer_id, size_t step, float lr, float beta1, float beta2,
+                             float epsilon, float weight_decay, int bias_correction,
+                             int advance_state, const ps_chunk* host_chunks, int n_chunks,
+                             size_t chunk_numel, const ps_chunk* staging, int n_slots,
+                             float loss_scale, const ps_step_state* d_state, ps_stream_t stream);
+
+/* The inf/nan probe for host-resident chunks: only the fp16 payloads are
+ * streamed (2 B/element) through staging[i].param_fp16. */
+int ps_overflow_scan_host_chunks(const ps_chunk* host_chunks, int n_chunks, size_t chunk_numel,
+                                 const ps_chunk* staging, int n_slots, ps_step_state* d_state,
+                                 ps_stream_t stream);
 
 /* Whole-buffer RNE cast (payload_fp16.copy_(payload_fp32), chunk_io_buff.py:116-126). */
 int ps_cast_fp32_to_fp16(const float* d_src, uint16_t* d_dst, size_t numel, ps_stream_t stream);
@@ -185,7 +220,7 @@ int ps_overflow_scan(const uint16_t* d_grads_fp16, size_t numel, ps_step_state* 
                      ps_stream_t stream);
 int ps_overflow_scan_f32(const float* d_grads_fp32, size_t numel, ps_step_state* d_state,
                          ps_stream_t stream);
-int ps_overflow_scan_chunks(const ps_chunk* d_chunks, int n_chunks, size_t chunk_numel,
+int ps_overflow_scan_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_numel,
                             ps_step_state* d_state, ps_stream_t stream);
 
 /* Backward-side producer (patrickstar/core/hook.py:200-230): copy one parameter's

@@ -77,6 +77,8 @@ SIGNATURES = {
     "ps_adam_update": (_i, [_i, _sz, _f, _f, _f, _f, _f, _i, _vp, _vp, _i, _vp, _vp, _sz, _f, _vp, _vp]),
     "ps_adam_step_chunks": (_i, [_i, _sz, _f, _f, _f, _f, _f, _i, _vp, _i, _sz, _f, _vp]),
     "ps_adam_step_chunks_gated": (_i, [_i, _f, _f, _f, _i, _vp, _i, _sz, _vp, _vp]),
+    "ps_adam_step_host_chunks": (_i, [_i, _sz, _f, _f, _f, _f, _f, _i, _i, _vp, _i, _sz, _vp, _i, _f, _vp, _vp]),
+    "ps_overflow_scan_host_chunks": (_i, [_vp, _i, _sz, _vp, _i, _vp, _vp]),
     "ps_restore_fp16_chunks": (_i, [_vp, _i, _sz, _vp, _vp]),
     "ps_cast_fp32_to_fp16": (_i, [_vp, _vp, _sz, _vp]),
     "ps_state_init": (_i, [_vp, _d, _i, _d, _i, _i64, _d, _i, _i, _i, _f, _f, _vp]),
@@ -129,3 +131,11 @@ def current_stream_handle():
     import torch
 
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def chunk_array(rows):
+    """Host array of ps_chunk descriptors from rows of (fp32, exp_avg, exp_avg_sq, fp16) addresses."""
+    arr = (ps_chunk * len(rows))()
+    for i, (p32, m, v, p16) in enumerate(rows):
+        arr[i].param_fp32, arr[i].exp_avg, arr[i].exp_avg_sq, arr[i].param_fp16 = p32, m, v, p16
+    return arr

@@ -2,9 +2,20 @@
 //
 // Everything here is HBM-bandwidth bound: 28 bytes move per element per step
 // (read fp16 grad + fp32 param/m/v, write fp32 param/m/v + fp16 param) for
-// ~20 flops, so the kernels are organised around 16-byte per-lane accesses,
-// enough independent loads in flight per lane to cover HBM latency, and
-// exactly one pass over the data.  No matrix cores are involved.
+// ~20 flops.  No matrix cores are involved.  What the kernels are organised
+// around, all of it measured on MI355X:
+//   * one pass over the data, in place; per lane one 16-byte access to each
+//     fp32 array and one 8-byte access to the fp16 array, so that every wave
+//     instruction covers a contiguous span of whole cache lines;
+//   * one small tile (512 elements) per workgroup and a CAP on resident waves
+//     (2 per SIMD): the pass touches four arrays for reading and the same four
+//     for writing, and HBM efficiency drops when the set of in-flight cache
+//     lines gets wide; a narrow, steadily advancing window per array gave
+//     5.95 TB/s where the fully occupied machine gave 5.3 TB/s (a plain
+//     1-read-1-write copy peaks at 6.2 TB/s on the same GPU);
+//   * chunk descriptors travel in the kernel-argument segment (64 per launch),
+//     so a wave's first data load depends on one scalar load, not two;
+//   * plain (temporal) loads/stores: non-temporal hints cost 20-25 %.
 //
 // Arithmetic contract (bit-exact with the explicit-intrinsic body of the
 // reference operator, patrickstar/ops/csrc/adam/cpu_adam.cpp:91-141): every
@@ -25,15 +36,26 @@
 
 #include "ps_adam.h"
 
-// Build-time tuning knobs.
-#ifndef PS_UNROLL
-#define PS_UNROLL 1  // 16-byte vector steps per lane per tile (measured: 1 is best, more in-flight loads per wave do not help)
-#endif
+// Build-time tuning knobs of the fused Adam kernels (defaults = measured best).
 #ifndef PS_BLOCK
-#define PS_BLOCK 256  // threads per workgroup
+#define PS_BLOCK 128  // threads per workgroup
+#endif
+#ifndef PS_LANE_ELEMS
+#define PS_LANE_ELEMS 4  // elements per lane per vector step (4 or 8)
+#endif
+#ifndef PS_UNROLL
+#define PS_UNROLL 1  // vector steps per lane per tile
+#endif
+#ifndef PS_MAX_WAVES_PER_EU
+#define PS_MAX_WAVES_PER_EU 2  // cap on resident waves per SIMD (0: no cap)
 #endif
 #ifndef PS_STREAMING
-#define PS_STREAMING 0  // 1 marks chunk payload accesses non-temporal (measured on MI355X: 20-25 % slower)
+#define PS_STREAMING 0  // 1 marks chunk payload accesses non-temporal (slower on MI355X)
+#endif
+#if PS_MAX_WAVES_PER_EU > 0
+#define PS_OCCUPANCY __attribute__((amdgpu_waves_per_eu(1, PS_MAX_WAVES_PER_EU)))
+#else
+#define PS_OCCUPANCY
 #endif
 
 namespace {
@@ -56,9 +78,9 @@ int hip_fail(hipError_t e, const char* what)
     return fail(-(int)e, "%s: %s", what, hipGetErrorString(e));
 }
 
-#define PS_HIP(call)                                   \
-    do {                                               \
-        hipError_t e_ = (call);                        \
+#define PS_HIP(call)                                      \
+    do {                                                  \
+        hipError_t e_ = (call);                           \
         if (e_ != hipSuccess) return hip_fail(e_, #call); \
     } while (0)
 
@@ -71,7 +93,6 @@ struct HostAdam {
     float alpha, beta1, beta2, eps, weight_decay;
     float beta1_t = 1.0f, beta2_t = 1.0f;
     size_t step = 0;
-    float bc1 = 1.0f, bc2inv = 1.0f;
     bool adamw;
 
     // cpu_adam.h:143-162
@@ -95,18 +116,12 @@ struct HostAdam {
             beta2_t = beta2_t * beta2;
         }
     }
-    // cpu_adam.h:163-175
-    void set(float lr, float epsilon, float wd, bool bias_correction)
+    // cpu_adam.h:163-170 (the bias-correction scalars follow in finish_consts)
+    void set(float lr, float epsilon, float wd)
     {
         alpha = lr;
         eps = epsilon;
         weight_decay = wd;
-        bc1 = 1.0f;
-        bc2inv = 1.0f;
-        if (bias_correction) {
-            bc1 = 1.0f - beta1_t;
-            bc2inv = 1.0f / sqrtf(1.0f - beta2_t);
-        }
     }
 };
 
@@ -124,6 +139,7 @@ std::shared_ptr<HostAdam> find_opt(int id)
 
 enum WdMode { WD_NONE = 0, WD_L2 = 1, WD_DECOUPLED = 2 };
 enum Unscale { UNSCALE_NONE = 0, UNSCALE_DIV = 1, UNSCALE_MUL = 2 };
+constexpr int UNSCALE_RUNTIME = -1;  // template value: look at StepConsts::unscale (uniform branch)
 
 // Per-launch constants (cpu_adam.cpp:39-46 and the SIMD_SET block at :55-77).
 struct StepConsts {
@@ -152,6 +168,7 @@ __host__ __device__ inline void finish_consts(StepConsts& c, float lr, float bet
                                               float beta2_t, bool bias_correction,
                                               float loss_scale)
 {
+    // cpu_adam.h:170-174
     float bc1 = 1.0f, bc2inv = 1.0f;
     if (bias_correction) {
         bc1 = 1.0f - beta1_t;
@@ -199,6 +216,20 @@ __device__ __forceinline__ void adam_element(const StepConsts& c, float g, float
     p = __builtin_fmaf(u, c.step_size, p);
 }
 
+template <int WD, int UNS>
+__device__ __forceinline__ void element_any(const StepConsts& c, float g, float& p, float& m,
+                                            float& v)
+{
+    if (UNS != UNSCALE_RUNTIME)
+        adam_element<WD, UNS>(c, g, p, m, v);
+    else if (c.unscale == UNSCALE_MUL)
+        adam_element<WD, UNSCALE_MUL>(c, g, p, m, v);
+    else if (c.unscale == UNSCALE_DIV)
+        adam_element<WD, UNSCALE_DIV>(c, g, p, m, v);
+    else
+        adam_element<WD, UNSCALE_NONE>(c, g, p, m, v);
+}
+
 __device__ __forceinline__ float half_bits_to_float(uint32_t h)
 {
     return __half2float(__ushort_as_half((unsigned short)h));
@@ -215,70 +246,105 @@ __device__ __forceinline__ uint32_t float_to_half_bits(float f)
     return (uint32_t)__half_as_ushort(__float2half_rn(f));
 }
 
-// 16-byte global accesses.  PS_STREAMING=1 would mark them non-temporal; on
-// MI355X that costs bandwidth (partial-line write-through), so it is off.
+// ------------------------------------------------------- vector accesses
+
 typedef float float4v __attribute__((ext_vector_type(4)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
 
-// Chunk payload addresses are read from a descriptor array in memory, so the
-// compiler cannot tell their address space and would fall back to flat_*
-// instructions.  They are always device-global: say so.
+// Chunk payloads are always device-global memory; saying so keeps the
+// compiler from falling back to flat_* instructions for pointers it did not
+// see being allocated.
 #define PS_GLOBAL __attribute__((address_space(1)))
 typedef PS_GLOBAL float4v gfloat4v;
 typedef PS_GLOBAL uint4v guint4v;
-typedef PS_GLOBAL float gfloat;
-typedef PS_GLOBAL uint16_t ghalf;
+typedef PS_GLOBAL uint2v guint2v;
 
-__device__ __forceinline__ const gfloat4v* gvec(const float* p) { return (const gfloat4v*)(p); }
-__device__ __forceinline__ gfloat4v* gvec(float* p) { return (gfloat4v*)(p); }
-__device__ __forceinline__ const guint4v* gvec(const uint16_t* p) { return (const guint4v*)(p); }
-__device__ __forceinline__ guint4v* gvec(uint16_t* p) { return (guint4v*)(p); }
-
-__device__ __forceinline__ float4v ld_stream(const gfloat4v* p)
+__device__ __forceinline__ float4v ld_f4(const float* p)
 {
 #if PS_STREAMING
-    return __builtin_nontemporal_load(p);
+    return __builtin_nontemporal_load((const gfloat4v*)(p));
 #else
-    return *p;
+    return *(const gfloat4v*)(p);
 #endif
 }
-__device__ __forceinline__ uint4v ld_stream(const guint4v* p)
+__device__ __forceinline__ void st_f4(float* p, float4v v)
 {
 #if PS_STREAMING
-    return __builtin_nontemporal_load(p);
+    __builtin_nontemporal_store(v, (gfloat4v*)(p));
 #else
-    return *p;
+    *(gfloat4v*)(p) = v;
 #endif
 }
-__device__ __forceinline__ void st_stream(gfloat4v* p, float4v v)
+__device__ __forceinline__ uint4v ld_u4(const uint16_t* p)
 {
 #if PS_STREAMING
-    __builtin_nontemporal_store(v, p);
+    return __builtin_nontemporal_load((const guint4v*)(p));
 #else
-    *p = v;
+    return *(const guint4v*)(p);
 #endif
 }
-__device__ __forceinline__ void st_stream(guint4v* p, uint4v v)
+__device__ __forceinline__ void st_u4(uint16_t* p, uint4v v)
 {
 #if PS_STREAMING
-    __builtin_nontemporal_store(v, p);
+    __builtin_nontemporal_store(v, (guint4v*)(p));
 #else
-    *p = v;
+    *(guint4v*)(p) = v;
 #endif
 }
 
-constexpr int kBlock = PS_BLOCK;   // 4 waves at 256
-constexpr int kLaneElems = 8;      // elements per lane per vector step: 16 B of fp16, 2 x 16 B of each fp32 array
-constexpr int kUnroll = PS_UNROLL; // vector steps per lane per tile
-constexpr int kTile = kBlock * kLaneElems * kUnroll;  // 2048 elements = 56 KiB of traffic per tile
+constexpr int kBlock = PS_BLOCK;
+// Elements per lane per vector step.  8: one 16-byte access of fp16 and two
+// 16-byte accesses per fp32 array.  4: an 8-byte access of fp16 and one
+// 16-byte access per fp32 array.
+constexpr int kLaneElems = PS_LANE_ELEMS;
+constexpr int kUnroll = PS_UNROLL;  // vector steps per lane per tile
+constexpr int kTile = kBlock * kLaneElems * kUnroll;
+constexpr int kQuads = kLaneElems / 4;  // float4 accesses per fp32 array per step
+constexpr int kWords = kLaneElems / 2;  // 32-bit words of fp16 pairs per step
+static_assert(kLaneElems == 4 || kLaneElems == 8, "PS_LANE_ELEMS must be 4 or 8");
+static_assert(kBlock % 64 == 0 && kBlock >= 64 && kBlock <= 1024, "PS_BLOCK must be whole waves");
 
-constexpr int UNSCALE_RUNTIME = -1;  // template value: look at StepConsts::unscale (uniform branch)
+// fp16 pairs of one lane and step: 2 or 4 words, moved with one 8- or 16-byte access
+struct HalfWords {
+    uint32_t w[kWords];
+};
+
+__device__ __forceinline__ HalfWords ld_halves(const uint16_t* p)
+{
+    HalfWords r;
+    if (kWords == 4) {
+        uint4v t = ld_u4(p);
+#pragma unroll
+        for (int k = 0; k < kWords; ++k) r.w[k] = t[k];
+    } else {
+        uint2v t = *(const guint2v*)(p);
+#pragma unroll
+        for (int k = 0; k < kWords; ++k) r.w[k] = t[k];
+    }
+    return r;
+}
+
+__device__ __forceinline__ void st_halves(uint16_t* p, const HalfWords& r)
+{
+    if (kWords == 4) {
+        uint4v t;
+#pragma unroll
+        for (int k = 0; k < kWords; ++k) t[k] = r.w[k];
+        st_u4(p, t);
+    } else {
+        uint2v t;
+#pragma unroll
+        for (int k = 0; k < kWords; ++k) t[k] = r.w[k];
+        *(guint2v*)(p) = t;
+    }
+}
 
 // The registers of one lane for one tile.
 struct LaneTile {
-    uint4v g[kUnroll];
-    float4v p[kUnroll][2], m[kUnroll][2], v[kUnroll][2];
-    uint4v h[kUnroll];
+    HalfWords g[kUnroll];
+    float4v p[kUnroll][kQuads], m[kUnroll][kQuads], v[kUnroll][kQuads];
+    HalfWords h[kUnroll];
 };
 
 template <int WD, int UNS>
@@ -287,8 +353,8 @@ __device__ __forceinline__ void lane_math(const StepConsts& c, LaneTile& r)
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            uint32_t word = r.g[u][w];
+        for (int w = 0; w < kWords; ++w) {
+            uint32_t word = r.g[u].w[w];
             float g0 = half_bits_to_float(word & 0xFFFFu);
             float g1 = half_bits_to_float(word >> 16);
             const int e0 = 2 * w, e1 = 2 * w + 1;
@@ -304,15 +370,14 @@ __device__ __forceinline__ void lane_math(const StepConsts& c, LaneTile& r)
             r.p[u][e1 >> 2][e1 & 3] = p1;
             r.m[u][e1 >> 2][e1 & 3] = m1;
             r.v[u][e1 >> 2][e1 & 3] = v1;
-            r.h[u][w] = float_to_half_bits(p0) | (float_to_half_bits(p1) << 16);
+            r.h[u].w[w] = float_to_half_bits(p0) | (float_to_half_bits(p1) << 16);
         }
     }
 }
 
 // One tile of one chunk, fast path: the whole tile is in range and all four
 // bases are 16-byte aligned.  All loads of the tile are issued before the
-// first use so that each lane has 7 * kUnroll independent 16-byte loads in
-// flight.  Loads and stores are written once, outside any branch on the
+// first use.  Loads and stores are written once, outside any branch on the
 // arithmetic variant.
 template <int WD, int UNS>
 __device__ __forceinline__ void adam_tile_vec(const StepConsts& c, float* __restrict__ p32,
@@ -323,13 +388,13 @@ __device__ __forceinline__ void adam_tile_vec(const StepConsts& c, float* __rest
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
         size_t i = base + ((size_t)u * kBlock + threadIdx.x) * kLaneElems;
-        r.g[u] = ld_stream(gvec(h16 + i));
-        r.p[u][0] = ld_stream(gvec(p32 + i));
-        r.p[u][1] = ld_stream(gvec(p32 + i + 4));
-        r.m[u][0] = ld_stream(gvec(m32 + i));
-        r.m[u][1] = ld_stream(gvec(m32 + i + 4));
-        r.v[u][0] = ld_stream(gvec(v32 + i));
-        r.v[u][1] = ld_stream(gvec(v32 + i + 4));
+        r.g[u] = ld_halves(h16 + i);
+#pragma unroll
+        for (int q = 0; q < kQuads; ++q) r.p[u][q] = ld_f4(p32 + i + 4 * q);
+#pragma unroll
+        for (int q = 0; q < kQuads; ++q) r.m[u][q] = ld_f4(m32 + i + 4 * q);
+#pragma unroll
+        for (int q = 0; q < kQuads; ++q) r.v[u][q] = ld_f4(v32 + i + 4 * q);
     }
     if (UNS != UNSCALE_RUNTIME) {
         lane_math<WD, UNS>(c, r);
@@ -343,28 +408,14 @@ __device__ __forceinline__ void adam_tile_vec(const StepConsts& c, float* __rest
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
         size_t i = base + ((size_t)u * kBlock + threadIdx.x) * kLaneElems;
-        st_stream(gvec(p32 + i), r.p[u][0]);
-        st_stream(gvec(p32 + i + 4), r.p[u][1]);
-        st_stream(gvec(m32 + i), r.m[u][0]);
-        st_stream(gvec(m32 + i + 4), r.m[u][1]);
-        st_stream(gvec(v32 + i), r.v[u][0]);
-        st_stream(gvec(v32 + i + 4), r.v[u][1]);
-        st_stream(gvec(h16 + i), r.h[u]);
+#pragma unroll
+        for (int q = 0; q < kQuads; ++q) st_f4(p32 + i + 4 * q, r.p[u][q]);
+#pragma unroll
+        for (int q = 0; q < kQuads; ++q) st_f4(m32 + i + 4 * q, r.m[u][q]);
+#pragma unroll
+        for (int q = 0; q < kQuads; ++q) st_f4(v32 + i + 4 * q, r.v[u][q]);
+        st_halves(h16 + i, r.h[u]);
     }
-}
-
-template <int WD, int UNS>
-__device__ __forceinline__ void element_any(const StepConsts& c, float g, float& p, float& m,
-                                            float& v)
-{
-    if (UNS != UNSCALE_RUNTIME)
-        adam_element<WD, UNS>(c, g, p, m, v);
-    else if (c.unscale == UNSCALE_MUL)
-        adam_element<WD, UNSCALE_MUL>(c, g, p, m, v);
-    else if (c.unscale == UNSCALE_DIV)
-        adam_element<WD, UNSCALE_DIV>(c, g, p, m, v);
-    else
-        adam_element<WD, UNSCALE_NONE>(c, g, p, m, v);
 }
 
 // Same elements, one at a time: ragged tile ends and unaligned bases.
@@ -414,14 +465,15 @@ __device__ __forceinline__ void restore_tile(const float* __restrict__ p32,
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             size_t i = base + ((size_t)u * kBlock + threadIdx.x) * kLaneElems;
-            float4v a = ld_stream(gvec(p32 + i));
-            float4v b = ld_stream(gvec(p32 + i + 4));
-            uint4v out;
-            out[0] = float_to_half_bits(a[0]) | (float_to_half_bits(a[1]) << 16);
-            out[1] = float_to_half_bits(a[2]) | (float_to_half_bits(a[3]) << 16);
-            out[2] = float_to_half_bits(b[0]) | (float_to_half_bits(b[1]) << 16);
-            out[3] = float_to_half_bits(b[2]) | (float_to_half_bits(b[3]) << 16);
-            st_stream(gvec(h16 + i), out);
+            float4v a[kQuads];
+#pragma unroll
+            for (int q = 0; q < kQuads; ++q) a[q] = ld_f4(p32 + i + 4 * q);
+            HalfWords out;
+#pragma unroll
+            for (int w = 0; w < kWords; ++w)
+                out.w[w] = float_to_half_bits(a[w >> 1][(2 * w) & 3]) |
+                           (float_to_half_bits(a[w >> 1][(2 * w + 1) & 3]) << 16);
+            st_halves(h16 + i, out);
         }
     } else {
         if (end > numel) end = numel;
@@ -430,33 +482,23 @@ __device__ __forceinline__ void restore_tile(const float* __restrict__ p32,
     }
 }
 
-// ---------------------------------------------------------------- kernels
+// ------------------------------------------------------- chunk-list kernels
+//
+// Grid: x = tile inside a chunk, y = chunk inside the batch.  Up to kBatch
+// descriptors are passed BY VALUE in the kernel-argument segment.
 
-struct ChunkListArgs {
-    const ps_chunk* chunks;
-    int n_chunks;
-    size_t chunk_numel;
-    size_t tiles_per_chunk;
-    size_t n_tiles;
+constexpr int kBatch = 64;
+struct ChunkBatch {
+    ps_chunk c[kBatch];
 };
-
-template <int WD, int UNS>
-__device__ __forceinline__ void chunk_list_pass(const ChunkListArgs& a, const StepConsts& c)
-{
-    for (size_t t = blockIdx.x; t < a.n_tiles; t += gridDim.x) {
-        size_t ci = t / a.tiles_per_chunk;
-        size_t base = (t - ci * a.tiles_per_chunk) * (size_t)kTile;
-        ps_chunk ch = a.chunks[ci];
-        adam_tile<WD, UNS>(c, ch, base, a.chunk_numel);
-    }
-}
 
 // Host-decided step: all scalars arrive as kernel arguments and the
 // arithmetic variant is a compile-time property of the kernel.
 template <int WD, int UNS>
-__global__ void __launch_bounds__(kBlock) adam_chunks_kernel(ChunkListArgs a, StepConsts c)
+__global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
+    adam_chunks_kernel(ChunkBatch b, size_t chunk_numel, StepConsts c)
 {
-    chunk_list_pass<WD, UNS>(a, c);
+    adam_tile<WD, UNS>(c, b.c[blockIdx.y], (size_t)blockIdx.x * kTile, chunk_numel);
 }
 
 struct GatedArgs {
@@ -470,38 +512,32 @@ struct GatedArgs {
 // The weight-decay form is known to the host; the unscale form depends on
 // the device-resident scale and is a uniform branch around the arithmetic.
 template <int WD>
-__global__ void __launch_bounds__(kBlock)
-    adam_chunks_gated_kernel(ChunkListArgs a, GatedArgs ga, const ps_step_state* __restrict__ st)
+__global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
+    adam_chunks_gated_kernel(ChunkBatch b, size_t chunk_numel, GatedArgs ga,
+                             const ps_step_state* __restrict__ st)
 {
+    const ps_chunk& ch = b.c[blockIdx.y];
+    const size_t base = (size_t)blockIdx.x * kTile;
     if (st->overflow) {
-        for (size_t t = blockIdx.x; t < a.n_tiles; t += gridDim.x) {
-            size_t ci = t / a.tiles_per_chunk;
-            size_t base = (t - ci * a.tiles_per_chunk) * (size_t)kTile;
-            ps_chunk ch = a.chunks[ci];
-            restore_tile(ch.param_fp32, ch.param_fp16, base, a.chunk_numel);
-        }
+        restore_tile(ch.param_fp32, ch.param_fp16, base, chunk_numel);
         return;
     }
     StepConsts c;
     // The operator takes loss_scale as a C float: the Python number narrows (RNE).
     finish_consts(c, ga.lr, st->beta1, st->beta2, ga.eps, ga.wd, ga.adamw != 0, st->beta1_t_next,
                   st->beta2_t_next, ga.bias_correction != 0, (float)st->cur_scale);
-    chunk_list_pass<WD, UNSCALE_RUNTIME>(a, c);
+    adam_tile<WD, UNSCALE_RUNTIME>(c, ch, base, chunk_numel);
 }
 
-__global__ void __launch_bounds__(kBlock)
-    restore_chunks_kernel(ChunkListArgs a, const ps_step_state* __restrict__ st)
+__global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
+    restore_chunks_kernel(ChunkBatch b, size_t chunk_numel, const ps_step_state* __restrict__ st)
 {
     if (st != nullptr && !st->overflow) return;
-    for (size_t t = blockIdx.x; t < a.n_tiles; t += gridDim.x) {
-        size_t ci = t / a.tiles_per_chunk;
-        size_t base = (t - ci * a.tiles_per_chunk) * (size_t)kTile;
-        ps_chunk ch = a.chunks[ci];
-        restore_tile(ch.param_fp32, ch.param_fp16, base, a.chunk_numel);
-    }
+    const ps_chunk& ch = b.c[blockIdx.y];
+    restore_tile(ch.param_fp32, ch.param_fp16, (size_t)blockIdx.x * kTile, chunk_numel);
 }
 
-__global__ void __launch_bounds__(kBlock)
+__global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
     cast_kernel(const float* __restrict__ src, uint16_t* __restrict__ dst, size_t numel,
                 size_t n_tiles)
 {
@@ -509,18 +545,22 @@ __global__ void __launch_bounds__(kBlock)
         restore_tile(src, dst, t * (size_t)kTile, numel);
 }
 
+// ------------------------------------------------- auxiliary (non-hot) kernels
+
+constexpr int kAuxBlock = 256;
+
 // Flat tensor, any grad dtype, optional fp16 output (adam_update of the operator).
 // Element-wise accesses: tensors handed to the operator are views at arbitrary
 // element offsets inside a chunk, so no alignment can be assumed.
 template <int WD, bool GRAD_HALF>
-__global__ void __launch_bounds__(kBlock)
+__global__ void __launch_bounds__(kAuxBlock)
     adam_flat_kernel(StepConsts c, float* p32, const void* grads, float* m32, float* v32,
                      uint16_t* out16, size_t numel)
 {
     const uint16_t* gh = static_cast<const uint16_t*>(grads);
     const float* gf = static_cast<const float*>(grads);
-    size_t stride = (size_t)gridDim.x * kBlock;
-    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < numel; i += stride) {
+    size_t stride = (size_t)gridDim.x * kAuxBlock;
+    for (size_t i = (size_t)blockIdx.x * kAuxBlock + threadIdx.x; i < numel; i += stride) {
         float g = GRAD_HALF ? half_bits_to_float(gh[i]) : gf[i];
         float p = p32[i], m = m32[i], v = v32[i];
         element_any<WD, UNSCALE_RUNTIME>(c, g, p, m, v);
@@ -547,7 +587,7 @@ __device__ __forceinline__ uint32_t nonfinite_halves(uint32_t w)
 // four waves, then at most one atomic per block (none when nothing was seen).
 __device__ __forceinline__ void block_flag_commit(uint32_t hit, uint32_t* flag)
 {
-    __shared__ uint32_t wave_hit[kBlock / 64];
+    __shared__ uint32_t wave_hit[kAuxBlock / 64];
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) hit |= (uint32_t)__shfl_xor((int)hit, off, 64);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -556,72 +596,62 @@ __device__ __forceinline__ void block_flag_commit(uint32_t hit, uint32_t* flag)
     if (threadIdx.x == 0) {
         uint32_t any = 0;
 #pragma unroll
-        for (int w = 0; w < kBlock / 64; ++w) any |= wave_hit[w];
+        for (int w = 0; w < kAuxBlock / 64; ++w) any |= wave_hit[w];
         if (any) atomicOr(flag, 1u);
     }
 }
 
 constexpr int kScanUnroll = 4;
-constexpr int kScanTile = kBlock * kLaneElems * kScanUnroll;  // 8192 halves = 16 KiB
+constexpr int kScanTile = kAuxBlock * 8 * kScanUnroll;  // 16-byte loads of 8 halves: 8192 halves = 16 KiB per tile
 
-__device__ __forceinline__ uint32_t scan_span_f16(const uint16_t* __restrict__ h, size_t numel,
-                                                  size_t first_tile, size_t tile_stride)
+// One scan tile of a fp16 buffer.
+__device__ __forceinline__ uint32_t scan_tile_f16(const uint16_t* __restrict__ h, size_t numel,
+                                                  size_t tile)
 {
     uint32_t hit = 0;
-    const bool aligned = (((uintptr_t)h) & 15u) == 0;
-    size_t n_tiles = (numel + kScanTile - 1) / kScanTile;
-    for (size_t t = first_tile; t < n_tiles; t += tile_stride) {
-        size_t base = t * (size_t)kScanTile;
-        if (aligned && base + kScanTile <= numel) {
-            uint4v w[kScanUnroll];
+    const size_t base = tile * (size_t)kScanTile;
+    if (base >= numel) return 0;
+    if ((((uintptr_t)h) & 15u) == 0 && base + kScanTile <= numel) {
+        uint4v w[kScanUnroll];
 #pragma unroll
-            for (int u = 0; u < kScanUnroll; ++u)
-                w[u] = ld_stream(gvec(
-                    h + base + ((size_t)u * kBlock + threadIdx.x) * kLaneElems));
+        for (int u = 0; u < kScanUnroll; ++u)
+            w[u] = ld_u4(h + base + ((size_t)u * kAuxBlock + threadIdx.x) * 8);
 #pragma unroll
-            for (int u = 0; u < kScanUnroll; ++u)
-                hit |= nonfinite_halves(w[u][0]) | nonfinite_halves(w[u][1]) |
-                       nonfinite_halves(w[u][2]) | nonfinite_halves(w[u][3]);
-        } else {
-            size_t end = base + kScanTile < numel ? base + kScanTile : numel;
-            for (size_t i = base + threadIdx.x; i < end; i += kBlock)
-                hit |= ((h[i] & 0x7C00u) == 0x7C00u) ? 1u : 0u;
-        }
+        for (int u = 0; u < kScanUnroll; ++u)
+            hit |= nonfinite_halves(w[u][0]) | nonfinite_halves(w[u][1]) |
+                   nonfinite_halves(w[u][2]) | nonfinite_halves(w[u][3]);
+    } else {
+        size_t end = base + kScanTile < numel ? base + kScanTile : numel;
+        for (size_t i = base + threadIdx.x; i < end; i += kAuxBlock)
+            hit |= ((h[i] & 0x7C00u) == 0x7C00u) ? 1u : 0u;
     }
     return hit;
 }
 
-__global__ void __launch_bounds__(kBlock)
-    scan_f16_kernel(const uint16_t* __restrict__ h, size_t numel, ps_step_state* st)
+__global__ void __launch_bounds__(kAuxBlock)
+    scan_f16_kernel(const uint16_t* __restrict__ h, size_t numel, size_t n_tiles,
+                    ps_step_state* st)
 {
-    uint32_t hit = scan_span_f16(h, numel, blockIdx.x, gridDim.x);
+    uint32_t hit = 0;
+    for (size_t t = blockIdx.x; t < n_tiles; t += gridDim.x) hit |= scan_tile_f16(h, numel, t);
     block_flag_commit(hit, &st->overflow);
 }
 
-__global__ void __launch_bounds__(kBlock)
+__global__ void __launch_bounds__(kAuxBlock)
     scan_f32_kernel(const float* __restrict__ f, size_t numel, ps_step_state* st)
 {
     uint32_t hit = 0;
     const uint32_t* w = reinterpret_cast<const uint32_t*>(f);
-    size_t stride = (size_t)gridDim.x * kBlock;
-    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < numel; i += stride)
+    size_t stride = (size_t)gridDim.x * kAuxBlock;
+    for (size_t i = (size_t)blockIdx.x * kAuxBlock + threadIdx.x; i < numel; i += stride)
         hit |= ((w[i] & 0x7F800000u) == 0x7F800000u) ? 1u : 0u;
     block_flag_commit(hit, &st->overflow);
 }
 
-__global__ void __launch_bounds__(kBlock)
-    scan_chunks_kernel(ChunkListArgs a, ps_step_state* st)
+__global__ void __launch_bounds__(kAuxBlock)
+    scan_chunks_kernel(ChunkBatch b, size_t chunk_numel, ps_step_state* st)
 {
-    // blocks are dealt over (chunk, tile) pairs of the whole list
-    uint32_t hit = 0;
-    size_t tiles_per_chunk = (a.chunk_numel + kScanTile - 1) / kScanTile;
-    size_t n_tiles = tiles_per_chunk * (size_t)a.n_chunks;
-    for (size_t t = blockIdx.x; t < n_tiles; t += gridDim.x) {
-        size_t ci = t / tiles_per_chunk;
-        size_t tile = t - ci * tiles_per_chunk;
-        // a one-tile span: first_tile = tile, stride large enough to stop after it
-        hit |= scan_span_f16(a.chunks[ci].param_fp16, a.chunk_numel, tile, tiles_per_chunk);
-    }
+    uint32_t hit = scan_tile_f16(b.c[blockIdx.y].param_fp16, chunk_numel, blockIdx.x);
     block_flag_commit(hit, &st->overflow);
 }
 
@@ -632,15 +662,15 @@ __global__ void __launch_bounds__(kBlock)
 // element.  fp32 gradients are rounded to fp16 (RNE); the probe looks at the
 // value that lands in the chunk.
 template <bool SRC_HALF>
-__global__ void __launch_bounds__(kBlock)
+__global__ void __launch_bounds__(kAuxBlock)
     grad_to_chunk_kernel(const void* __restrict__ src, uint16_t* __restrict__ dst, size_t numel,
                          ps_step_state* st)
 {
     const uint16_t* sh = static_cast<const uint16_t*>(src);
     const float* sf = static_cast<const float*>(src);
     uint32_t hit = 0;
-    size_t stride = (size_t)gridDim.x * kBlock;
-    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < numel; i += stride) {
+    size_t stride = (size_t)gridDim.x * kAuxBlock;
+    for (size_t i = (size_t)blockIdx.x * kAuxBlock + threadIdx.x; i < numel; i += stride) {
         uint32_t h = SRC_HALF ? (uint32_t)sh[i] : float_to_half_bits(sf[i]);
         dst[i] = (uint16_t)h;
         hit |= ((h & 0x7C00u) == 0x7C00u) ? 1u : 0u;
@@ -729,54 +759,152 @@ __global__ void scaler_update_kernel(ps_step_state* st, int flag_mode, ps_scale_
     *st = s;
 }
 
-// ------------------------------------------------------------ launch shapes
+// ------------------------------------------------------------ launch helpers
 
-// One workgroup per tile measured fastest on MI355X (the hardware dispatcher
-// keeps the set of in-flight tiles a narrow, advancing window of each array,
-// which is what DRAM page locality wants); a resident grid-stride loop was
-// 3-8 % slower.  The cap only guards the 2^31-1 limit of gridDim.x, beyond
-// which the kernels' stride loops take over.
-int grid_cap() { return 0x7FFFFFFF; }
+constexpr size_t kMaxGridX = 0x7FFFFFFFull;
 
-unsigned grid_for(size_t n_tiles)
+unsigned grid_1d(size_t n_blocks)
 {
-    size_t cap = (size_t)grid_cap();
-    size_t g = n_tiles < cap ? n_tiles : cap;
+    size_t g = n_blocks < kMaxGridX ? n_blocks : kMaxGridX;
     return (unsigned)(g ? g : 1);
 }
 
-int make_chunk_args(ChunkListArgs& a, const ps_chunk* d_chunks, int n_chunks, size_t chunk_numel)
+// Validated view of a host array of chunk descriptors.
+struct ChunkList {
+    const ps_chunk* chunks;
+    int n_chunks;
+    size_t chunk_numel;
+    size_t tiles_per_chunk;  // of kTile elements
+};
+
+int make_chunk_list(ChunkList& a, const ps_chunk* chunks, int n_chunks, size_t chunk_numel,
+                    size_t tile)
 {
-    if (d_chunks == nullptr && n_chunks > 0) return fail(PS_ERR_BAD_ARG, "d_chunks is NULL");
     if (n_chunks < 0) return fail(PS_ERR_BAD_ARG, "n_chunks = %d is negative", n_chunks);
-    a.chunks = d_chunks;
+    if (chunks == nullptr && n_chunks > 0) return fail(PS_ERR_BAD_ARG, "chunks is NULL");
+    a.chunks = chunks;
     a.n_chunks = n_chunks;
     a.chunk_numel = chunk_numel;
-    a.tiles_per_chunk = (chunk_numel + kTile - 1) / kTile;
-    a.n_tiles = a.tiles_per_chunk * (size_t)n_chunks;
+    a.tiles_per_chunk = (chunk_numel + tile - 1) / tile;
+    if (a.tiles_per_chunk > kMaxGridX)
+        return fail(PS_ERR_BAD_ARG, "chunk_numel = %zu is beyond the launch grid", chunk_numel);
+    return 0;
+}
+
+// Calls launch(batch, n_in_batch, grid) for every group of up to kBatch chunks.
+template <typename F>
+int for_each_batch(const ChunkList& a, F launch)
+{
+    if (a.n_chunks == 0 || a.tiles_per_chunk == 0) return 0;
+    for (int first = 0; first < a.n_chunks; first += kBatch) {
+        int n = a.n_chunks - first < kBatch ? a.n_chunks - first : kBatch;
+        ChunkBatch b;
+        memset(&b, 0, sizeof(b));
+        for (int i = 0; i < n; ++i) {
+            const ps_chunk& c = a.chunks[first + i];
+            if (!c.param_fp32 || !c.exp_avg || !c.exp_avg_sq || !c.param_fp16)
+                return fail(PS_ERR_BAD_ARG, "chunk %d has a NULL payload address", first + i);
+            b.c[i] = c;
+        }
+        launch(b, dim3((unsigned)a.tiles_per_chunk, (unsigned)n));
+        PS_HIP(hipGetLastError());
+    }
     return 0;
 }
 
 template <int WD>
-void launch_adam_chunks_wd(const ChunkListArgs& a, const StepConsts& c, hipStream_t s)
+void launch_adam_batch_wd(const ChunkBatch& b, dim3 grid, size_t chunk_numel, const StepConsts& c,
+                          hipStream_t s)
 {
-    dim3 grid(grid_for(a.n_tiles)), block(kBlock);
+    dim3 block(kBlock);
     if (c.unscale == UNSCALE_MUL)
-        hipLaunchKernelGGL((adam_chunks_kernel<WD, UNSCALE_MUL>), grid, block, 0, s, a, c);
+        hipLaunchKernelGGL((adam_chunks_kernel<WD, UNSCALE_MUL>), grid, block, 0, s, b, chunk_numel, c);
     else if (c.unscale == UNSCALE_DIV)
-        hipLaunchKernelGGL((adam_chunks_kernel<WD, UNSCALE_DIV>), grid, block, 0, s, a, c);
+        hipLaunchKernelGGL((adam_chunks_kernel<WD, UNSCALE_DIV>), grid, block, 0, s, b, chunk_numel, c);
     else
-        hipLaunchKernelGGL((adam_chunks_kernel<WD, UNSCALE_NONE>), grid, block, 0, s, a, c);
+        hipLaunchKernelGGL((adam_chunks_kernel<WD, UNSCALE_NONE>), grid, block, 0, s, b, chunk_numel, c);
 }
 
-void launch_adam_chunks(const ChunkListArgs& a, const StepConsts& c, hipStream_t s)
+void launch_adam_batch(const ChunkBatch& b, dim3 grid, size_t chunk_numel, const StepConsts& c,
+                       hipStream_t s)
 {
     if (c.wd_mode == WD_DECOUPLED)
-        launch_adam_chunks_wd<WD_DECOUPLED>(a, c, s);
+        launch_adam_batch_wd<WD_DECOUPLED>(b, grid, chunk_numel, c, s);
     else if (c.wd_mode == WD_L2)
-        launch_adam_chunks_wd<WD_L2>(a, c, s);
+        launch_adam_batch_wd<WD_L2>(b, grid, chunk_numel, c, s);
     else
-        launch_adam_chunks_wd<WD_NONE>(a, c, s);
+        launch_adam_batch_wd<WD_NONE>(b, grid, chunk_numel, c, s);
+}
+
+void launch_gated_batch(const ChunkBatch& b, dim3 grid, size_t chunk_numel, const GatedArgs& ga,
+                        const ps_step_state* d_state, hipStream_t s)
+{
+    dim3 block(kBlock);
+    const bool decay = ga.wd > 0.0f;
+    if (decay && ga.adamw)
+        hipLaunchKernelGGL(adam_chunks_gated_kernel<WD_DECOUPLED>, grid, block, 0, s, b, chunk_numel, ga, d_state);
+    else if (decay)
+        hipLaunchKernelGGL(adam_chunks_gated_kernel<WD_L2>, grid, block, 0, s, b, chunk_numel, ga, d_state);
+    else
+        hipLaunchKernelGGL(adam_chunks_gated_kernel<WD_NONE>, grid, block, 0, s, b, chunk_numel, ga, d_state);
+}
+
+// ------------------------------------------- host-resident chunks: streaming
+//
+// Chunks that live in pinned host memory are streamed through caller-owned
+// staging buffers in HBM: H2D copies on one side stream, the fused kernel on a
+// compute side stream, D2H copies on another side stream, tied together with
+// events, so that with two or more staging slots the copy of chunk k+1 and the
+// write-back of chunk k-1 overlap the kernel on chunk k.  Nothing blocks the
+// host.  The streams and events are created once per device and kept.
+
+constexpr int kMaxSlots = 8;
+
+struct Pipeline {
+    bool ready = false;
+    hipStream_t h2d = nullptr, compute = nullptr, d2h = nullptr;
+    hipEvent_t entry = nullptr;
+    hipEvent_t h2d_done[kMaxSlots] = {}, compute_done[kMaxSlots] = {}, d2h_done[kMaxSlots] = {};
+    bool slot_used[kMaxSlots] = {};
+};
+
+std::mutex g_pipeline_mutex;
+std::unordered_map<int, Pipeline> g_pipelines;
+
+int get_pipeline(Pipeline** out)
+{
+    int dev = 0;
+    PS_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(g_pipeline_mutex);
+    Pipeline& p = g_pipelines[dev];
+    if (!p.ready) {
+        // default priority on purpose
+        PS_HIP(hipStreamCreateWithFlags(&p.h2d, hipStreamNonBlocking));
+        PS_HIP(hipStreamCreateWithFlags(&p.compute, hipStreamNonBlocking));
+        PS_HIP(hipStreamCreateWithFlags(&p.d2h, hipStreamNonBlocking));
+        PS_HIP(hipEventCreateWithFlags(&p.entry, hipEventDisableTiming));
+        for (int i = 0; i < kMaxSlots; ++i) {
+            PS_HIP(hipEventCreateWithFlags(&p.h2d_done[i], hipEventDisableTiming));
+            PS_HIP(hipEventCreateWithFlags(&p.compute_done[i], hipEventDisableTiming));
+            PS_HIP(hipEventCreateWithFlags(&p.d2h_done[i], hipEventDisableTiming));
+        }
+        p.ready = true;
+    }
+    *out = &p;
+    return 0;
+}
+
+int check_slots(const ps_chunk* staging, int n_slots, bool fp16_only)
+{
+    if (n_slots < 1 || n_slots > kMaxSlots)
+        return fail(PS_ERR_BAD_ARG, "n_slots = %d must be in 1..%d", n_slots, kMaxSlots);
+    if (!staging) return fail(PS_ERR_BAD_ARG, "staging is NULL");
+    for (int i = 0; i < n_slots; ++i) {
+        if (!staging[i].param_fp16 ||
+            (!fp16_only && (!staging[i].param_fp32 || !staging[i].exp_avg || !staging[i].exp_avg_sq)))
+            return fail(PS_ERR_BAD_ARG, "staging slot %d has a NULL buffer", i);
+    }
+    return 0;
 }
 
 }  // namespace
@@ -829,17 +957,16 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
     if (numel > 0 && (!d_params || !d_grads || !d_exp_avg || !d_exp_avg_sq))
         return fail(PS_ERR_BAD_ARG, "ps_adam_update: NULL tensor pointer");
     o->advance(step, beta1, beta2);
-    o->set(lr, epsilon, weight_decay, bias_correction != 0);
+    o->set(lr, epsilon, weight_decay);
     if (numel == 0) return 0;
     StepConsts c;
     finish_consts(c, o->alpha, o->beta1, o->beta2, o->eps, o->weight_decay, o->adamw, o->beta1_t,
                   o->beta2_t, bias_correction != 0, loss_scale);
-    size_t blocks = (numel + kBlock - 1) / kBlock;
-    unsigned grid = grid_for(blocks);
+    unsigned grid = grid_1d((numel + kAuxBlock - 1) / kAuxBlock);
     hipStream_t s = static_cast<hipStream_t>(stream);
-#define PS_FLAT(WD, HALF)                                                                     \
-    hipLaunchKernelGGL((adam_flat_kernel<WD, HALF>), dim3(grid), dim3(kBlock), 0, s, c, d_params, \
-                       d_grads, d_exp_avg, d_exp_avg_sq, d_param_fp16_out, numel)
+#define PS_FLAT(WD, HALF)                                                                  \
+    hipLaunchKernelGGL((adam_flat_kernel<WD, HALF>), dim3(grid), dim3(kAuxBlock), 0, s, c, \
+                       d_params, d_grads, d_exp_avg, d_exp_avg_sq, d_param_fp16_out, numel)
     if (grads_are_half) {
         if (c.wd_mode == WD_DECOUPLED) PS_FLAT(WD_DECOUPLED, true);
         else if (c.wd_mode == WD_L2) PS_FLAT(WD_L2, true);
@@ -856,66 +983,55 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
 
 int ps_adam_step_chunks(int optimizer_id, size_t step, float lr, float beta1, float beta2,
                         float epsilon, float weight_decay, int bias_correction,
-                        const ps_chunk* d_chunks, int n_chunks, size_t chunk_numel,
+                        const ps_chunk* chunks, int n_chunks, size_t chunk_numel,
                         float loss_scale, ps_stream_t stream)
 {
     auto o = find_opt(optimizer_id);
     if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
-    ChunkListArgs a;
-    if (int rc = make_chunk_args(a, d_chunks, n_chunks, chunk_numel)) return rc;
+    ChunkList a;
+    if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, kTile)) return rc;
     o->advance(step, beta1, beta2);
-    o->set(lr, epsilon, weight_decay, bias_correction != 0);
-    if (a.n_tiles == 0) return 0;
+    o->set(lr, epsilon, weight_decay);
     StepConsts c;
     finish_consts(c, o->alpha, o->beta1, o->beta2, o->eps, o->weight_decay, o->adamw, o->beta1_t,
                   o->beta2_t, bias_correction != 0, loss_scale);
-    launch_adam_chunks(a, c, static_cast<hipStream_t>(stream));
-    PS_HIP(hipGetLastError());
-    return 0;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid) {
+        launch_adam_batch(b, grid, chunk_numel, c, s);
+    });
 }
 
 int ps_adam_step_chunks_gated(int optimizer_id, float lr, float epsilon, float weight_decay,
-                              int bias_correction, const ps_chunk* d_chunks, int n_chunks,
+                              int bias_correction, const ps_chunk* chunks, int n_chunks,
                               size_t chunk_numel, const ps_step_state* d_state,
                               ps_stream_t stream)
 {
     auto o = find_opt(optimizer_id);
     if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
     if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
-    ChunkListArgs a;
-    if (int rc = make_chunk_args(a, d_chunks, n_chunks, chunk_numel)) return rc;
-    if (a.n_tiles == 0) return 0;
+    ChunkList a;
+    if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, kTile)) return rc;
     GatedArgs ga;
     ga.lr = lr;
     ga.eps = epsilon;
     ga.wd = weight_decay;
     ga.adamw = o->adamw ? 1 : 0;
     ga.bias_correction = bias_correction;
-    {
-        dim3 grid(grid_for(a.n_tiles)), block(kBlock);
-        hipStream_t s = static_cast<hipStream_t>(stream);
-        const bool decay = weight_decay > 0.0f;
-        if (decay && o->adamw)
-            hipLaunchKernelGGL(adam_chunks_gated_kernel<WD_DECOUPLED>, grid, block, 0, s, a, ga, d_state);
-        else if (decay)
-            hipLaunchKernelGGL(adam_chunks_gated_kernel<WD_L2>, grid, block, 0, s, a, ga, d_state);
-        else
-            hipLaunchKernelGGL(adam_chunks_gated_kernel<WD_NONE>, grid, block, 0, s, a, ga, d_state);
-    }
-    PS_HIP(hipGetLastError());
-    return 0;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid) {
+        launch_gated_batch(b, grid, chunk_numel, ga, d_state, s);
+    });
 }
 
-int ps_restore_fp16_chunks(const ps_chunk* d_chunks, int n_chunks, size_t chunk_numel,
+int ps_restore_fp16_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_numel,
                            const ps_step_state* d_state, ps_stream_t stream)
 {
-    ChunkListArgs a;
-    if (int rc = make_chunk_args(a, d_chunks, n_chunks, chunk_numel)) return rc;
-    if (a.n_tiles == 0) return 0;
-    hipLaunchKernelGGL(restore_chunks_kernel, dim3(grid_for(a.n_tiles)), dim3(kBlock), 0,
-                       static_cast<hipStream_t>(stream), a, d_state);
-    PS_HIP(hipGetLastError());
-    return 0;
+    ChunkList a;
+    if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, kTile)) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid) {
+        hipLaunchKernelGGL(restore_chunks_kernel, grid, dim3(kBlock), 0, s, b, chunk_numel, d_state);
+    });
 }
 
 int ps_cast_fp32_to_fp16(const float* d_src, uint16_t* d_dst, size_t numel, ps_stream_t stream)
@@ -923,9 +1039,129 @@ int ps_cast_fp32_to_fp16(const float* d_src, uint16_t* d_dst, size_t numel, ps_s
     if (numel == 0) return 0;
     if (!d_src || !d_dst) return fail(PS_ERR_BAD_ARG, "ps_cast_fp32_to_fp16: NULL pointer");
     size_t n_tiles = (numel + kTile - 1) / kTile;
-    hipLaunchKernelGGL(cast_kernel, dim3(grid_for(n_tiles)), dim3(kBlock), 0,
+    hipLaunchKernelGGL(cast_kernel, dim3(grid_1d(n_tiles)), dim3(kBlock), 0,
                        static_cast<hipStream_t>(stream), d_src, d_dst, numel, n_tiles);
     PS_HIP(hipGetLastError());
+    return 0;
+}
+
+int ps_adam_step_host_chunks(int optimizer_id, size_t step, float lr, float beta1, float beta2,
+                             float epsilon, float weight_decay, int bias_correction,
+                             int advance_state, const ps_chunk* host_chunks, int n_chunks,
+                             size_t chunk_numel, const ps_chunk* staging, int n_slots,
+                             float loss_scale, const ps_step_state* d_state, ps_stream_t stream)
+{
+    auto o = find_opt(optimizer_id);
+    if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
+    ChunkList a;
+    if (int rc = make_chunk_list(a, host_chunks, n_chunks, chunk_numel, kTile)) return rc;
+    if (int rc = check_slots(staging, n_slots, false)) return rc;
+    for (int i = 0; i < n_chunks; ++i) {
+        const ps_chunk& c = host_chunks[i];
+        if (!c.param_fp32 || !c.exp_avg || !c.exp_avg_sq || !c.param_fp16)
+            return fail(PS_ERR_BAD_ARG, "host chunk %d has a NULL payload address", i);
+    }
+    StepConsts c;
+    GatedArgs ga;
+    if (d_state == nullptr) {
+        if (advance_state) o->advance(step, beta1, beta2);
+        o->set(lr, epsilon, weight_decay);
+        finish_consts(c, o->alpha, o->beta1, o->beta2, o->eps, o->weight_decay, o->adamw,
+                      o->beta1_t, o->beta2_t, bias_correction != 0, loss_scale);
+    } else {
+        ga.lr = lr;
+        ga.eps = epsilon;
+        ga.wd = weight_decay;
+        ga.adamw = o->adamw ? 1 : 0;
+        ga.bias_correction = bias_correction;
+    }
+    if (n_chunks == 0 || chunk_numel == 0) return 0;
+    Pipeline* p = nullptr;
+    if (int rc = get_pipeline(&p)) return rc;
+    hipStream_t caller = static_cast<hipStream_t>(stream);
+    const size_t b32 = chunk_numel * sizeof(float), b16 = chunk_numel * sizeof(uint16_t);
+
+    // everything the caller queued so far (gradients written, the device flag set) comes first
+    PS_HIP(hipEventRecord(p->entry, caller));
+    PS_HIP(hipStreamWaitEvent(p->h2d, p->entry, 0));
+    PS_HIP(hipStreamWaitEvent(p->compute, p->entry, 0));
+    for (int i = 0; i < kMaxSlots; ++i) p->slot_used[i] = false;
+
+    for (int k = 0; k < n_chunks; ++k) {
+        const int s = k % n_slots;
+        const ps_chunk& h = host_chunks[k];
+        const ps_chunk& d = staging[s];
+        // the slot is free once its previous occupant has been written back
+        if (p->slot_used[s]) PS_HIP(hipStreamWaitEvent(p->h2d, p->d2h_done[s], 0));
+        PS_HIP(hipMemcpyAsync(d.param_fp16, h.param_fp16, b16, hipMemcpyHostToDevice, p->h2d));
+        PS_HIP(hipMemcpyAsync(d.param_fp32, h.param_fp32, b32, hipMemcpyHostToDevice, p->h2d));
+        PS_HIP(hipMemcpyAsync(d.exp_avg, h.exp_avg, b32, hipMemcpyHostToDevice, p->h2d));
+        PS_HIP(hipMemcpyAsync(d.exp_avg_sq, h.exp_avg_sq, b32, hipMemcpyHostToDevice, p->h2d));
+        PS_HIP(hipEventRecord(p->h2d_done[s], p->h2d));
+
+        PS_HIP(hipStreamWaitEvent(p->compute, p->h2d_done[s], 0));
+        ChunkBatch b;
+        memset(&b, 0, sizeof(b));
+        b.c[0] = d;
+        dim3 grid((unsigned)a.tiles_per_chunk, 1);
+        if (d_state == nullptr)
+            launch_adam_batch(b, grid, chunk_numel, c, p->compute);
+        else
+            launch_gated_batch(b, grid, chunk_numel, ga, d_state, p->compute);
+        PS_HIP(hipGetLastError());
+        PS_HIP(hipEventRecord(p->compute_done[s], p->compute));
+
+        PS_HIP(hipStreamWaitEvent(p->d2h, p->compute_done[s], 0));
+        PS_HIP(hipMemcpyAsync(h.param_fp16, d.param_fp16, b16, hipMemcpyDeviceToHost, p->d2h));
+        // (on a device-skipped step these three come back unchanged; copying them anyway
+        // keeps the host free of any knowledge of the flag)
+        PS_HIP(hipMemcpyAsync(h.param_fp32, d.param_fp32, b32, hipMemcpyDeviceToHost, p->d2h));
+        PS_HIP(hipMemcpyAsync(h.exp_avg, d.exp_avg, b32, hipMemcpyDeviceToHost, p->d2h));
+        PS_HIP(hipMemcpyAsync(h.exp_avg_sq, d.exp_avg_sq, b32, hipMemcpyDeviceToHost, p->d2h));
+        PS_HIP(hipEventRecord(p->d2h_done[s], p->d2h));
+        p->slot_used[s] = true;
+    }
+    // later work on the caller's stream sees every chunk written back
+    for (int s = 0; s < n_slots; ++s)
+        if (p->slot_used[s]) PS_HIP(hipStreamWaitEvent(caller, p->d2h_done[s], 0));
+    return 0;
+}
+
+int ps_overflow_scan_host_chunks(const ps_chunk* host_chunks, int n_chunks, size_t chunk_numel,
+                                 const ps_chunk* staging, int n_slots, ps_step_state* d_state,
+                                 ps_stream_t stream)
+{
+    if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
+    ChunkList a;
+    if (int rc = make_chunk_list(a, host_chunks, n_chunks, chunk_numel, kScanTile)) return rc;
+    if (int rc = check_slots(staging, n_slots, true)) return rc;
+    if (n_chunks == 0 || chunk_numel == 0) return 0;
+    Pipeline* p = nullptr;
+    if (int rc = get_pipeline(&p)) return rc;
+    hipStream_t caller = static_cast<hipStream_t>(stream);
+    const size_t b16 = chunk_numel * sizeof(uint16_t);
+    const size_t n_tiles = a.tiles_per_chunk;
+    PS_HIP(hipEventRecord(p->entry, caller));
+    PS_HIP(hipStreamWaitEvent(p->h2d, p->entry, 0));
+    PS_HIP(hipStreamWaitEvent(p->compute, p->entry, 0));
+    for (int i = 0; i < kMaxSlots; ++i) p->slot_used[i] = false;
+    for (int k = 0; k < n_chunks; ++k) {
+        const int s = k % n_slots;
+        if (!host_chunks[k].param_fp16)
+            return fail(PS_ERR_BAD_ARG, "host chunk %d has a NULL fp16 payload address", k);
+        if (p->slot_used[s]) PS_HIP(hipStreamWaitEvent(p->h2d, p->compute_done[s], 0));
+        PS_HIP(hipMemcpyAsync(staging[s].param_fp16, host_chunks[k].param_fp16, b16,
+                              hipMemcpyHostToDevice, p->h2d));
+        PS_HIP(hipEventRecord(p->h2d_done[s], p->h2d));
+        PS_HIP(hipStreamWaitEvent(p->compute, p->h2d_done[s], 0));
+        hipLaunchKernelGGL(scan_f16_kernel, dim3(grid_1d(n_tiles)), dim3(kAuxBlock), 0, p->compute,
+                           staging[s].param_fp16, chunk_numel, n_tiles, d_state);
+        PS_HIP(hipGetLastError());
+        PS_HIP(hipEventRecord(p->compute_done[s], p->compute));
+        p->slot_used[s] = true;
+    }
+    for (int s = 0; s < n_slots; ++s)
+        if (p->slot_used[s]) PS_HIP(hipStreamWaitEvent(caller, p->compute_done[s], 0));
     return 0;
 }
 
@@ -1001,8 +1237,8 @@ int ps_overflow_scan(const uint16_t* d_grads_fp16, size_t numel, ps_step_state* 
     if (numel == 0) return 0;
     if (!d_grads_fp16) return fail(PS_ERR_BAD_ARG, "d_grads_fp16 is NULL");
     size_t n_tiles = (numel + kScanTile - 1) / kScanTile;
-    hipLaunchKernelGGL(scan_f16_kernel, dim3(grid_for(n_tiles)), dim3(kBlock), 0,
-                       static_cast<hipStream_t>(stream), d_grads_fp16, numel, d_state);
+    hipLaunchKernelGGL(scan_f16_kernel, dim3(grid_1d(n_tiles)), dim3(kAuxBlock), 0,
+                       static_cast<hipStream_t>(stream), d_grads_fp16, numel, n_tiles, d_state);
     PS_HIP(hipGetLastError());
     return 0;
 }
@@ -1013,25 +1249,23 @@ int ps_overflow_scan_f32(const float* d_grads_fp32, size_t numel, ps_step_state*
     if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
     if (numel == 0) return 0;
     if (!d_grads_fp32) return fail(PS_ERR_BAD_ARG, "d_grads_fp32 is NULL");
-    size_t blocks = (numel + (size_t)kBlock * 16 - 1) / ((size_t)kBlock * 16);
-    hipLaunchKernelGGL(scan_f32_kernel, dim3(grid_for(blocks)), dim3(kBlock), 0,
+    size_t blocks = (numel + (size_t)kAuxBlock * 16 - 1) / ((size_t)kAuxBlock * 16);
+    hipLaunchKernelGGL(scan_f32_kernel, dim3(grid_1d(blocks)), dim3(kAuxBlock), 0,
                        static_cast<hipStream_t>(stream), d_grads_fp32, numel, d_state);
     PS_HIP(hipGetLastError());
     return 0;
 }
 
-int ps_overflow_scan_chunks(const ps_chunk* d_chunks, int n_chunks, size_t chunk_numel,
+int ps_overflow_scan_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_numel,
                             ps_step_state* d_state, ps_stream_t stream)
 {
     if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
-    ChunkListArgs a;
-    if (int rc = make_chunk_args(a, d_chunks, n_chunks, chunk_numel)) return rc;
-    if (a.n_tiles == 0) return 0;
-    size_t scan_tiles = ((chunk_numel + kScanTile - 1) / kScanTile) * (size_t)n_chunks;
-    hipLaunchKernelGGL(scan_chunks_kernel, dim3(grid_for(scan_tiles)), dim3(kBlock), 0,
-                       static_cast<hipStream_t>(stream), a, d_state);
-    PS_HIP(hipGetLastError());
-    return 0;
+    ChunkList a;
+    if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, kScanTile)) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid) {
+        hipLaunchKernelGGL(scan_chunks_kernel, grid, dim3(kAuxBlock), 0, s, b, chunk_numel, d_state);
+    });
 }
 
 int ps_grad_to_chunk(const void* d_grad, int grad_is_half, uint16_t* d_slot_fp16, size_t numel,
@@ -1039,8 +1273,8 @@ int ps_grad_to_chunk(const void* d_grad, int grad_is_half, uint16_t* d_slot_fp16
 {
     if (numel == 0) return 0;
     if (!d_grad || !d_slot_fp16) return fail(PS_ERR_BAD_ARG, "ps_grad_to_chunk: NULL pointer");
-    size_t blocks = (numel + (size_t)kBlock * 4 - 1) / ((size_t)kBlock * 4);
-    dim3 grid(grid_for(blocks)), block(kBlock);
+    size_t blocks = (numel + (size_t)kAuxBlock * 4 - 1) / ((size_t)kAuxBlock * 4);
+    dim3 grid(grid_1d(blocks)), block(kAuxBlock);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (grad_is_half)
         hipLaunchKernelGGL(grad_to_chunk_kernel<true>, grid, block, 0, s, d_grad, d_slot_fp16, numel,

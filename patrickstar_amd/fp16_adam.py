@@ -152,7 +152,7 @@ class FP16Adam(torch.optim.Optimizer):
 
     # -- chunk descriptor tables -------------------------------------------------
     def _build_tables(self):
-        """Device array of ps_chunk descriptors for HBM-resident positions; list of host-resident ones."""
+        """Array of ps_chunk descriptors for HBM-resident positions; list of host-resident ones."""
         dev_rows, host_positions = [], []
         cl = self.client.chunk_list
         for pos in self.client.positions():
@@ -169,9 +169,7 @@ class FP16Adam(torch.optim.Optimizer):
                         cl[pos.fp16].payload.data_ptr(),
                     ]
                 )
-        table = None
-        if dev_rows:
-            table = torch.tensor(dev_rows, dtype=torch.int64).to(self.client.device)
+        table = _lib.chunk_array(dev_rows) if dev_rows else None
         self._tables = (table, len(dev_rows), host_positions)
         if host_positions:
             from .hybrid import HostChunkStreamer
@@ -214,7 +212,7 @@ class FP16Adam(torch.optim.Optimizer):
         if n_dev:
             _lib.check(
                 self._lib.ps_overflow_scan_chunks(
-                    table.data_ptr(), n_dev, self.client.default_chunk_size, self.loss_scaler.state_ptr, stream
+                    table, n_dev, self.client.default_chunk_size, self.loss_scaler.state_ptr, stream
                 ),
                 "ps_overflow_scan_chunks",
             )
@@ -263,7 +261,7 @@ class FP16Adam(torch.optim.Optimizer):
                 if n_dev:
                     _lib.check(
                         self._lib.ps_adam_step_chunks_gated(
-                            self.opt_id, lr, eps, weight_decay, 1, table.data_ptr(), n_dev, chunk_numel,
+                            self.opt_id, lr, eps, weight_decay, 1, table, n_dev, chunk_numel,
                             scaler.state_ptr, stream,
                         ),
                         "ps_adam_step_chunks_gated",
@@ -286,7 +284,7 @@ class FP16Adam(torch.optim.Optimizer):
             if n_dev:
                 _lib.check(
                     self._lib.ps_adam_step_chunks(
-                        self.opt_id, step_no, lr, beta1, beta2, eps, weight_decay, 1, table.data_ptr(), n_dev,
+                        self.opt_id, step_no, lr, beta1, beta2, eps, weight_decay, 1, table, n_dev,
                         chunk_numel, float(loss_scale), stream,
                     ),
                     "ps_adam_step_chunks",

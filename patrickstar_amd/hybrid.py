@@ -1,0 +1,72 @@
+"""Host-resident chunk positions: streamed through HBM staging slots by the C ABI.
+
+The reference's hybrid Adam keeps some chunks' optimizer state in host memory and
+updates them with the CPU operator (``patrickstar/ops/fp16_cpu_adam.py:415-428``,
+``patrickstar/ops/chunk_io_buff.py:214-255``).  On MI355X those chunks are instead
+copied into double-buffered HBM staging by ``hipMemcpyAsync`` on side streams,
+updated by the same fused kernel as resident chunks, and copied back, all ordered
+by events inside ``ps_adam_step_host_chunks``; the Python side only owns the
+staging buffers.
+"""
+import torch
+
+from . import _lib
+
+
+class HostChunkStreamer:
+    def __init__(self, client, host_positions, n_slots=2):
+        self.client = client
+        self.n_slots = n_slots
+        self.chunk_numel = client.default_chunk_size
+        cl = client.chunk_list
+        rows = []
+        for pos in host_positions:
+            payloads = [cl[c].payload for c in (pos.fp32, pos.exp_avg, pos.exp_avg_sq, pos.fp16)]
+            for t in payloads:
+                if t.device.type != "cpu" or not t.is_pinned():
+                    raise RuntimeError("host-resident chunk payloads must be pinned host memory")
+            rows.append([t.data_ptr() for t in payloads])
+        self.host_table = _lib.chunk_array(rows)
+        self.n_host = len(rows)
+        dev = client.device
+        n = self.chunk_numel
+        # staging lives for the life of the optimizer: allocating it per step (as the reference does with
+        # its per-step buffers, fp16_cpu_adam.py:530-547) would serialise against the streams that use it
+        self._slots = [
+            (
+                torch.empty(n, dtype=torch.float, device=dev),
+                torch.empty(n, dtype=torch.float, device=dev),
+                torch.empty(n, dtype=torch.float, device=dev),
+                torch.empty(n, dtype=torch.half, device=dev),
+            )
+            for _ in range(n_slots)
+        ]
+        self.staging = _lib.chunk_array([[t.data_ptr() for t in slot] for slot in self._slots])
+        self._lib = _lib.load()
+
+    def step_static(self, opt_id, step_no, lr, beta1, beta2, eps, weight_decay, loss_scale, advance):
+        _lib.check(
+            self._lib.ps_adam_step_host_chunks(
+                opt_id, step_no, lr, beta1, beta2, eps, weight_decay, 1, int(advance), self.host_table, self.n_host,
+                self.chunk_numel, self.staging, self.n_slots, float(loss_scale), None, _lib.current_stream_handle(),
+            ),
+            "ps_adam_step_host_chunks",
+        )
+
+    def step_gated(self, opt_id, lr, eps, weight_decay, scaler):
+        _lib.check(
+            self._lib.ps_adam_step_host_chunks(
+                opt_id, 0, lr, 0.0, 0.0, eps, weight_decay, 1, 0, self.host_table, self.n_host, self.chunk_numel,
+                self.staging, self.n_slots, -1.0, scaler.state_ptr, _lib.current_stream_handle(),
+            ),
+            "ps_adam_step_host_chunks",
+        )
+
+    def scan_gradients(self, scaler):
+        _lib.check(
+            self._lib.ps_overflow_scan_host_chunks(
+                self.host_table, self.n_host, self.chunk_numel, self.staging, self.n_slots, scaler.state_ptr,
+                _lib.current_stream_handle(),
+            ),
+            "ps_overflow_scan_host_chunks",
+        )

@@ -169,13 +169,35 @@ def test_empty_and_zero_sized_chunk_lists():
     s = _lib.current_stream_handle()
     lib.ps_adam_create(902, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, 0)
     assert lib.ps_adam_step_chunks(902, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, 1024, -1.0, s) == 0
-    table = torch.zeros(4, dtype=torch.int64, device="cuda")
-    assert lib.ps_adam_step_chunks(902, 2, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, table.data_ptr(), 1, 0, -1.0, s) == 0
+    buf = torch.zeros(64, dtype=torch.float, device="cuda")
+    one = _lib.chunk_array([[buf.data_ptr()] * 4])
+    assert lib.ps_adam_step_chunks(902, 2, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, one, 1, 0, -1.0, s) == 0
     assert lib.ps_adam_step_chunks(902, 3, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 2, 16, -1.0, s) == _lib.PS_ERR_BAD_ARG
-    assert lib.ps_adam_step_chunks(902, 3, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, table.data_ptr(), -1, 16, -1.0, s) == _lib.PS_ERR_BAD_ARG
+    assert lib.ps_adam_step_chunks(902, 3, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, one, -1, 16, -1.0, s) == _lib.PS_ERR_BAD_ARG
+    null_payload = _lib.chunk_array([[buf.data_ptr(), 0, buf.data_ptr(), buf.data_ptr()]])
+    assert lib.ps_adam_step_chunks(902, 3, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, null_payload, 1, 16, -1.0, s) == _lib.PS_ERR_BAD_ARG
+    assert b"NULL payload" in lib.ps_last_error()
     assert lib.ps_cast_fp32_to_fp16(None, None, 0, s) == 0
     lib.ps_adam_destroy(902)
     torch.cuda.synchronize()
+    assert not buf.any()
+
+
+def test_more_chunks_than_one_launch_carries():
+    """Descriptors travel 64 per launch: a 150-chunk list takes three launches and every chunk is updated."""
+    n = 2048 + 5
+    h = ChunkHarness(150, n, ps.LossScaler(16), seed=6, lr=1e-3, weight_decay=0.01, use_adamw=True)
+    h.fill_state()
+    h.fill_grads(1e-3, 16)
+    idx = [0, 63, 64, 127, 128, 149]
+    oc = h.oracle_chunks(idx)
+    oopt = oracle.OptimizerStepOracle(oc, oracle.StaticScalerOracle(16), lr=1e-3, weight_decay=0.01, use_adamw=True)
+    before = [h.payloads(i)[1].abs().sum().item() for i in range(150)]
+    h.opt.step()
+    oopt.step()
+    h.compare(oc, idx, what="150 chunks")
+    after = [h.payloads(i)[1].abs().sum().item() for i in range(150)]
+    assert all(a != b for a, b in zip(after, before))
 
 
 def test_nonfinite_gradients_with_static_scale_propagate_like_the_oracle():
