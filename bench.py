@@ -36,6 +36,10 @@ def parse_args():
     ap.add_argument("--chunk-size", type=int, default=N_CHUNK)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-reps", type=int, default=20)
+    ap.add_argument("--mode", choices=["static", "dynamic"], default="static",
+                    help="static: BASELINE config 4 as specified (static loss scale, one fused kernel per step). "
+                    "dynamic: same data with a DynamicLossScaler: inf/nan scan (2 B/element) + device-gated kernel + "
+                    "scaler update per step, no host sync")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also launch one plain device-to-device copy of 1 Gi floats (4 GiB read, 4 GiB written) "
                     "so that a rocprofv3 --pmc run holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -106,7 +110,11 @@ def main():
 
     client = ps.PatrickStarClient(0, N)
     params = client.append_flat_chunks(C)
-    opt = ps.FP16Adam(client, params, loss_scaler=ps.LossScaler(2**12), lr=1e-4, betas=(0.9, 0.999), eps=1e-8,
+    if args.mode == "static":
+        scaler = ps.LossScaler(2**12)
+    else:
+        scaler = ps.DynamicLossScaler(init_scale=2**12, scale_factor=2, scale_window=1000, min_scale=1)
+    opt = ps.FP16Adam(client, params, loss_scaler=scaler, lr=1e-4, betas=(0.9, 0.999), eps=1e-8,
                       weight_decay=0.01, use_adamw=True)
     gen = torch.Generator(device=dev)
     gen.manual_seed(0)
@@ -121,8 +129,11 @@ def main():
         del tmp
     # the step overwrites the fp16 gradients with fp16 parameters; later steps then read those as "gradients" of the
     # same magnitude class (|p| ~ 0.02 vs |g*scale| ~ 4), which changes values, not the work done per element
-    for p in params:
-        dict.__setitem__(opt.state[p], "step", 99 - args.warmup)
+    if args.mode == "static":
+        for p in params:
+            dict.__setitem__(opt.state[p], "step", 99 - args.warmup)
+    else:
+        scaler._seed_step(99 - args.warmup)
 
     if args.calibration_copy:
         src = torch.empty(1 << 30, dtype=torch.float32, device=dev).normal_()
@@ -146,7 +157,8 @@ def main():
     avg_kernel_ms = sum(kernel_ms) / len(kernel_ms)
     ms_per_step = wall * 1e3 / args.steps
     elements = C * N
-    algorithmic = BYTES_PER_ELEMENT * elements
+    # the dynamic mode adds the 2 B/element probe pass to the step
+    algorithmic = (BYTES_PER_ELEMENT + (2 if args.mode == "dynamic" else 0)) * elements
     achieved = algorithmic / (avg_kernel_ms * 1e-3) / 1e9
 
     out = {
@@ -167,7 +179,9 @@ def main():
             "AdamW lr 1e-4 betas (0.9,0.999) eps 1e-8 wd 0.01, static loss scale 2^12, fp16 grads -> fp32 p/m/v + fp16 params",
             "chunks": C,
             "chunk_numel": N,
-            "kernel": "adam_chunks_kernel<decoupled, exact-reciprocal unscale>",
+            "kernel": "adam_chunks_kernel<decoupled, exact-reciprocal unscale>" if args.mode == "static"
+            else "scan_chunks_kernel + adam_chunks_gated_kernel<decoupled> + scaler_update_kernel",
+            "mode": args.mode,
         },
         "roofline": {
             "bound": "hbm",
@@ -175,7 +189,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": traffic_from_profile() if (C, N) == (24, N_CHUNK) else None,
+            "traffic": traffic_from_profile() if (C, N, args.mode) == (24, N_CHUNK, "static") else None,
             "algorithmic_bytes_per_launch": algorithmic,
             "avg_kernel_ms": avg_kernel_ms,
             "min_kernel_ms": min(kernel_ms),
