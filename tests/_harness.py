@@ -61,7 +61,8 @@ class ChunkHarness:
             h[n:].zero_()
 
     def download(self, i):
-        return tuple(t.cpu().numpy() for t in self.payloads(i))
+        # always a private copy: a host-resident payload would otherwise be aliased by ".cpu()"
+        return tuple(t.detach().to("cpu", copy=True).numpy() for t in self.payloads(i))
 
     def oracle_chunks(self, indices=None):
         """Host mirror of the current device state, as the oracle's chunk dicts."""

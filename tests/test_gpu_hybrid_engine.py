@@ -1,0 +1,157 @@
+"""GPU tests of (a) host-resident chunk positions streamed through HBM staging and (b) the engine front-end.
+
+Bar as everywhere: bit-exact against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import patrickstar_amd as ps
+from _harness import ChunkHarness, assert_bits_equal
+
+pytestmark = pytest.mark.gpu
+
+
+class HybridHarness(ChunkHarness):
+    """Like ChunkHarness, with some positions kept in pinned host memory."""
+
+    def __init__(self, n_chunks, chunk_size, host_positions, loss_scaler=None, seed=0, **adam_kwargs):
+        self.device = torch.device("cuda:0")
+        self.n_chunks, self.chunk_size = n_chunks, chunk_size
+        host = set(host_positions)
+        self.client = ps.PatrickStarClient(0, chunk_size, config={"host_chunk_policy": lambda pos: pos in host})
+        self.params = self.client.append_flat_chunks(n_chunks)
+        self.opt = ps.FP16Adam(self.client, self.params, loss_scaler=loss_scaler, **adam_kwargs)
+        self.gen = torch.Generator(device=self.device)
+        self.gen.manual_seed(seed)
+        self.used = [p.ps_attr.numel for p in self.params]
+
+    def fill_state(self):
+        for i in range(self.n_chunks):
+            p, m, v, h = self.payloads(i)
+            n = self.chunk_size
+            p.copy_(torch.empty(n, device=self.device).normal_(0, 0.02, generator=self.gen))
+            m.copy_(torch.empty(n, device=self.device).normal_(0, 1e-4, generator=self.gen))
+            v.copy_(torch.empty(n, device=self.device).normal_(0, 1e-6, generator=self.gen).abs_())
+            h.copy_(p)
+        torch.cuda.synchronize()
+
+    def fill_grads(self, std, scale):
+        for i in range(self.n_chunks):
+            h = self.payloads(i)[3]
+            tmp = torch.empty(self.chunk_size, device=self.device).normal_(0, std, generator=self.gen).mul_(scale).half()
+            h.copy_(tmp)
+        torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("host_positions", [[1, 3, 4], [0, 1, 2, 3, 4], [4]])
+@pytest.mark.parametrize("chunk_size", [2048 * 3, 2048 + 77])
+def test_hybrid_static_bit_exact(host_positions, chunk_size):
+    h = HybridHarness(5, chunk_size, host_positions, ps.LossScaler(2**12), seed=chunk_size + len(host_positions),
+                      lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
+    for i in range(5):
+        on_host = h.payloads(i)[0].device.type == "cpu"
+        assert on_host == (i in host_positions)
+        assert (not on_host) or all(t.is_pinned() for t in h.payloads(i))
+    h.fill_state()
+    oc = h.oracle_chunks()
+    oopt = oracle.OptimizerStepOracle(oc, oracle.StaticScalerOracle(2**12), lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
+    for step in range(3):  # consecutive steps: resident and host halves must see the same running-product beta^t
+        h.fill_grads(1e-3, 2**12)
+        for i, c in enumerate(oc):
+            c["p16"][...] = h.download(i)[3]
+        h.opt.step()
+        torch.cuda.synchronize()
+        oopt.step()
+        h.compare(oc, what=f"hybrid step {step}")
+
+
+def test_hybrid_dynamic_skips_and_restores_host_chunks_too():
+    kw = dict(init_scale=2**10, scale_factor=2, scale_window=3, min_scale=1)
+    scaler = ps.DynamicLossScaler(**kw)
+    h = HybridHarness(4, 2048 * 2 + 9, [1, 2], scaler, seed=12, lr=1e-3, weight_decay=0.01)
+    h.fill_state()
+    oc = h.oracle_chunks()
+    oscaler = oracle.ScalerOracle(**kw)
+    oopt = oracle.OptimizerStepOracle(oc, oscaler, lr=1e-3, weight_decay=0.01)
+    skipped = []
+    for step in range(7):
+        h.fill_grads(1e-3, float(oscaler.loss_scale))
+        if step == 2:
+            h.payloads(2)[3][5] = float("inf")  # in a HOST-resident chunk: only the streamed probe can see it
+        if step == 5:
+            h.payloads(0)[3][0] = float("nan")  # in a resident chunk
+        for i, c in enumerate(oc):
+            c["p16"][...] = h.download(i)[3]
+        h.opt.step()
+        torch.cuda.synchronize()
+        oopt.check_overflow()
+        skipped.append(oopt.step())
+        h.compare(oc, what=f"hybrid dynamic step {step}")
+        assert scaler.loss_scale == oscaler.loss_scale and type(scaler.loss_scale) is type(oscaler.loss_scale)
+    assert skipped == [False, False, True, False, False, True, False]
+    assert h.opt.state[h.params[0]]["step"] == 5
+
+
+class _MLP(torch.nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.fc1 = torch.nn.Linear(24, 40)
+        self.fc2 = torch.nn.Linear(40, 8)
+        self.gain = torch.nn.Parameter(torch.ones(8))
+
+    def forward(self, x):
+        return (self.fc2(torch.tanh(self.fc1(x))) * self.gain).float().pow(2).mean()
+
+
+@pytest.mark.parametrize("loss_scale", [0, 128])
+def test_engine_end_to_end_against_oracle(loss_scale):
+    """initialize_engine -> forward -> backward -> step on a small fp16 model.  After backward the fp16 chunk payloads
+    hold the gradients; the oracle is fed exactly those and must agree bit for bit with what step() leaves behind."""
+    torch.manual_seed(0)
+    config = {
+        "optimizer": {"type": "AdamW", "params": {"lr": 1e-3, "betas": (0.9, 0.999), "eps": 1e-8, "weight_decay": 0.01}},
+        "fp16": {"enabled": True, "loss_scale": loss_scale, "initial_scale_power": 7, "loss_scale_window": 4, "hysteresis": 2, "min_loss_scale": 1},
+        "default_chunk_size": 1100,
+    }
+    engine, optimizer = ps.initialize_engine(model_func=_MLP, local_rank=0, config=config)
+    client = engine.client
+    assert engine.optimizer is optimizer and isinstance(optimizer, ps.FP16Adam)
+    assert all(p.dtype == torch.half and p.is_cuda for p in engine.module.parameters())
+    pos = client.positions()
+    assert len(pos) == 2  # fc1 fills 1000 of 1100; fc2 (328) does not fit behind it -> second chunk, which also takes gain
+    cl = client.chunk_list
+    mirror = [{"p32": cl[q.fp32].payload.cpu().numpy(), "m": cl[q.exp_avg].payload.cpu().numpy(),
+               "v": cl[q.exp_avg_sq].payload.cpu().numpy(), "p16": cl[q.fp16].payload.cpu().numpy()} for q in pos]
+    oscaler = oracle.scaler_from_config(config["fp16"])
+    oopt = oracle.OptimizerStepOracle(mirror, oscaler, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
+    x = torch.randn(16, 24, device="cuda").half()
+    losses = []
+    for it in range(6):
+        loss = engine(x * (1.0 if it != 3 else 3e4))  # iteration 3 overflows fp16 activations -> inf/nan gradients
+        engine.backward(loss)
+        assert all(p.grad is None for p in engine.module.parameters())
+        for q, c in zip(pos, mirror):
+            c["p16"][...] = cl[q.fp16].payload.cpu().numpy()  # the gradients, as backward left them in the chunks
+        optimizer.step()
+        oopt.check_overflow()
+        skipped = oopt.step()
+        if loss_scale == 0:
+            assert skipped == (it == 3)
+        for q, c in zip(pos, mirror):
+            for key, cid in (("p32", q.fp32), ("m", q.exp_avg), ("v", q.exp_avg_sq), ("p16", q.fp16)):
+                got = cl[cid].payload.cpu().numpy()
+                if loss_scale != 0 and it >= 3:
+                    assert np.array_equal(np.isnan(got), np.isnan(c[key]))  # static scale: the poison spreads, same places
+                else:
+                    assert_bits_equal(got, c[key], f"iteration {it} {key}")
+        losses.append(float(loss))
+        if loss_scale == 0:
+            assert optimizer.loss_scaler.loss_scale == oscaler.loss_scale
+    if loss_scale == 0:
+        assert optimizer.state[next(engine.module.parameters())]["step"] == 5
+        assert losses[5] < losses[0]  # it trains
+    # parameters are views of the chunk payloads: the model sees what the optimizer wrote
+    w = engine.module.fc1.weight
+    info = client.chunk_tensor_index.get_tensor_info(w.ps_attr.data_id())
+    assert w.data_ptr() == cl[info.chunk_id].payload.data_ptr() + 2 * info.start_offset
