@@ -166,22 +166,22 @@ int ps_restore_fp16_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_nu
  * (14 B/element), the fused kernel runs on it, and fp32 param/m/v + fp16 param
  * go back on another side stream (14 B/element); events order the three, so
  * with n_slots >= 2 the copies of neighbouring chunks overlap the kernel.
+ *   chunks       host array of descriptors of HBM-resident chunks (may be empty): updated
+ *                by the same kernels on `stream`, concurrently with the first copies
  *   host_chunks  host array of descriptors whose addresses are PINNED HOST memory
  *   staging      host array of n_slots (1..8) descriptors of DEVICE buffers of
  *                chunk_numel elements each, owned by the caller
- *   advance_state  0 when ps_adam_step_chunks already advanced the operator's
- *                step scalars for this optimizer step (resident chunks first,
- *                host chunks second: both halves must see the same beta^t)
- *   d_state      NULL: host-decided step with loss_scale; else device-gated
- *                exactly like ps_adam_step_chunks_gated (loss_scale ignored)
+ *   d_state      NULL: host-decided step with loss_scale, the operator's step scalars
+ *                advanced ONCE for both lists; else device-gated exactly like
+ *                ps_adam_step_chunks_gated (step, betas and loss_scale ignored)
  * Work queued on `stream` before the call is waited for; work queued on it
  * afterwards waits for the last write-back.  The call itself never blocks.
  * Calls that overlap in time on one device share the side streams and race. */
-int ps_adam_step_host_chunks(int optimizer_id, size_t step, float lr, float beta1, float beta2,
-                             float epsilon, float weight_decay, int bias_correction,
-                             int advance_state, const ps_chunk* host_chunks, int n_chunks,
-                             size_t chunk_numel, const ps_chunk* staging, int n_slots,
-                             float loss_scale, const ps_step_state* d_state, ps_stream_t stream);
+int ps_adam_step_hybrid(int optimizer_id, size_t step, float lr, float beta1, float beta2,
+                        float epsilon, float weight_decay, int bias_correction,
+                        const ps_chunk* chunks, int n_chunks, const ps_chunk* host_chunks,
+                        int n_host_chunks, size_t chunk_numel, const ps_chunk* staging, int n_slots,
+                        float loss_scale, const ps_step_state* d_state, ps_stream_t stream);
 
 /* The inf/nan probe for host-resident chunks: only the fp16 payloads are
  * streamed (2 B/element) through staging[i].param_fp16. */

@@ -77,7 +77,7 @@ SIGNATURES = {
     "ps_adam_update": (_i, [_i, _sz, _f, _f, _f, _f, _f, _i, _vp, _vp, _i, _vp, _vp, _sz, _f, _vp, _vp]),
     "ps_adam_step_chunks": (_i, [_i, _sz, _f, _f, _f, _f, _f, _i, _vp, _i, _sz, _f, _vp]),
     "ps_adam_step_chunks_gated": (_i, [_i, _f, _f, _f, _i, _vp, _i, _sz, _vp, _vp]),
-    "ps_adam_step_host_chunks": (_i, [_i, _sz, _f, _f, _f, _f, _f, _i, _i, _vp, _i, _sz, _vp, _i, _f, _vp, _vp]),
+    "ps_adam_step_hybrid": (_i, [_i, _sz, _f, _f, _f, _f, _f, _i, _vp, _i, _vp, _i, _sz, _vp, _i, _f, _vp, _vp]),
     "ps_overflow_scan_host_chunks": (_i, [_vp, _i, _sz, _vp, _i, _vp, _vp]),
     "ps_restore_fp16_chunks": (_i, [_vp, _i, _sz, _vp, _vp]),
     "ps_cast_fp32_to_fp16": (_i, [_vp, _vp, _sz, _vp]),

@@ -1045,26 +1045,29 @@ int ps_cast_fp32_to_fp16(const float* d_src, uint16_t* d_dst, size_t numel, ps_s
     return 0;
 }
 
-int ps_adam_step_host_chunks(int optimizer_id, size_t step, float lr, float beta1, float beta2,
-                             float epsilon, float weight_decay, int bias_correction,
-                             int advance_state, const ps_chunk* host_chunks, int n_chunks,
-                             size_t chunk_numel, const ps_chunk* staging, int n_slots,
-                             float loss_scale, const ps_step_state* d_state, ps_stream_t stream)
+int ps_adam_step_hybrid(int optimizer_id, size_t step, float lr, float beta1, float beta2,
+                        float epsilon, float weight_decay, int bias_correction,
+                        const ps_chunk* chunks, int n_chunks, const ps_chunk* host_chunks,
+                        int n_host_chunks, size_t chunk_numel, const ps_chunk* staging, int n_slots,
+                        float loss_scale, const ps_step_state* d_state, ps_stream_t stream)
 {
     auto o = find_opt(optimizer_id);
     if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
-    ChunkList a;
-    if (int rc = make_chunk_list(a, host_chunks, n_chunks, chunk_numel, kTile)) return rc;
-    if (int rc = check_slots(staging, n_slots, false)) return rc;
-    for (int i = 0; i < n_chunks; ++i) {
+    ChunkList resident, host;
+    if (int rc = make_chunk_list(resident, chunks, n_chunks, chunk_numel, kTile)) return rc;
+    if (int rc = make_chunk_list(host, host_chunks, n_host_chunks, chunk_numel, kTile)) return rc;
+    if (n_host_chunks > 0)
+        if (int rc = check_slots(staging, n_slots, false)) return rc;
+    for (int i = 0; i < n_host_chunks; ++i) {
         const ps_chunk& c = host_chunks[i];
         if (!c.param_fp32 || !c.exp_avg || !c.exp_avg_sq || !c.param_fp16)
             return fail(PS_ERR_BAD_ARG, "host chunk %d has a NULL payload address", i);
     }
+    // one advance of the operator's step scalars for the whole list, resident and host alike
     StepConsts c;
     GatedArgs ga;
     if (d_state == nullptr) {
-        if (advance_state) o->advance(step, beta1, beta2);
+        o->advance(step, beta1, beta2);
         o->set(lr, epsilon, weight_decay);
         finish_consts(c, o->alpha, o->beta1, o->beta2, o->eps, o->weight_decay, o->adamw,
                       o->beta1_t, o->beta2_t, bias_correction != 0, loss_scale);
@@ -1075,19 +1078,29 @@ int ps_adam_step_host_chunks(int optimizer_id, size_t step, float lr, float beta
         ga.adamw = o->adamw ? 1 : 0;
         ga.bias_correction = bias_correction;
     }
-    if (n_chunks == 0 || chunk_numel == 0) return 0;
-    Pipeline* p = nullptr;
-    if (int rc = get_pipeline(&p)) return rc;
     hipStream_t caller = static_cast<hipStream_t>(stream);
+    const bool stream_host = n_host_chunks > 0 && chunk_numel > 0;
+    Pipeline* p = nullptr;
+    if (stream_host) {
+        if (int rc = get_pipeline(&p)) return rc;
+        // Everything the caller queued so far (gradients written, the device flag set) comes
+        // first; the resident chunks' kernels, queued next, do NOT hold the copies back.
+        PS_HIP(hipEventRecord(p->entry, caller));
+        PS_HIP(hipStreamWaitEvent(p->h2d, p->entry, 0));
+        PS_HIP(hipStreamWaitEvent(p->compute, p->entry, 0));
+    }
+    int rc = for_each_batch(resident, [&](const ChunkBatch& b, dim3 grid) {
+        if (d_state == nullptr)
+            launch_adam_batch(b, grid, chunk_numel, c, caller);
+        else
+            launch_gated_batch(b, grid, chunk_numel, ga, d_state, caller);
+    });
+    if (rc) return rc;
+    if (!stream_host) return 0;
+
     const size_t b32 = chunk_numel * sizeof(float), b16 = chunk_numel * sizeof(uint16_t);
-
-    // everything the caller queued so far (gradients written, the device flag set) comes first
-    PS_HIP(hipEventRecord(p->entry, caller));
-    PS_HIP(hipStreamWaitEvent(p->h2d, p->entry, 0));
-    PS_HIP(hipStreamWaitEvent(p->compute, p->entry, 0));
     for (int i = 0; i < kMaxSlots; ++i) p->slot_used[i] = false;
-
-    for (int k = 0; k < n_chunks; ++k) {
+    for (int k = 0; k < n_host_chunks; ++k) {
         const int s = k % n_slots;
         const ps_chunk& h = host_chunks[k];
         const ps_chunk& d = staging[s];
@@ -1103,7 +1116,7 @@ int ps_adam_step_host_chunks(int optimizer_id, size_t step, float lr, float beta
         ChunkBatch b;
         memset(&b, 0, sizeof(b));
         b.c[0] = d;
-        dim3 grid((unsigned)a.tiles_per_chunk, 1);
+        dim3 grid((unsigned)host.tiles_per_chunk, 1);
         if (d_state == nullptr)
             launch_adam_batch(b, grid, chunk_numel, c, p->compute);
         else
@@ -1112,9 +1125,9 @@ int ps_adam_step_host_chunks(int optimizer_id, size_t step, float lr, float beta
         PS_HIP(hipEventRecord(p->compute_done[s], p->compute));
 
         PS_HIP(hipStreamWaitEvent(p->d2h, p->compute_done[s], 0));
-        PS_HIP(hipMemcpyAsync(h.param_fp16, d.param_fp16, b16, hipMemcpyDeviceToHost, p->d2h));
-        // (on a device-skipped step these three come back unchanged; copying them anyway
+        // (on a device-skipped step fp32 param / m / v come back unchanged; copying them anyway
         // keeps the host free of any knowledge of the flag)
+        PS_HIP(hipMemcpyAsync(h.param_fp16, d.param_fp16, b16, hipMemcpyDeviceToHost, p->d2h));
         PS_HIP(hipMemcpyAsync(h.param_fp32, d.param_fp32, b32, hipMemcpyDeviceToHost, p->d2h));
         PS_HIP(hipMemcpyAsync(h.exp_avg, d.exp_avg, b32, hipMemcpyDeviceToHost, p->d2h));
         PS_HIP(hipMemcpyAsync(h.exp_avg_sq, d.exp_avg_sq, b32, hipMemcpyDeviceToHost, p->d2h));

@@ -101,6 +101,7 @@ class FP16Adam(torch.optim.Optimizer):
         self._dynamic = isinstance(loss_scaler, DynamicLossScaler)
         self._host_overflow = False
         self._steps_dirty = False
+        self.staging_slots = 2  # HBM staging slots for host-resident chunks (double buffering)
 
         assert len(self.param_groups) == 1, "Only support one param group at the moment."
         # Eager state initialisation: m and v are chunk tensors shadowing the fp16 parameter chunks.
@@ -174,7 +175,7 @@ class FP16Adam(torch.optim.Optimizer):
         if host_positions:
             from .hybrid import HostChunkStreamer
 
-            self._streamer = HostChunkStreamer(self.client, host_positions)
+            self._streamer = HostChunkStreamer(self.client, host_positions, n_slots=self.staging_slots)
         return self._tables
 
     def invalidate_tables(self):
@@ -258,7 +259,9 @@ class FP16Adam(torch.optim.Optimizer):
                 scaler = self.loss_scaler
                 if self.scan_in_step:
                     self.check_overflow_chunks()
-                if n_dev:
+                if host_positions:
+                    self._streamer.step(self.opt_id, 0, lr, beta1, beta2, eps, weight_decay, -1.0, table, n_dev, scaler)
+                elif n_dev:
                     _lib.check(
                         self._lib.ps_adam_step_chunks_gated(
                             self.opt_id, lr, eps, weight_decay, 1, table, n_dev, chunk_numel,
@@ -266,8 +269,6 @@ class FP16Adam(torch.optim.Optimizer):
                         ),
                         "ps_adam_step_chunks_gated",
                     )
-                if host_positions:
-                    self._streamer.step_gated(self.opt_id, lr, eps, weight_decay, scaler)
                 scaler.update_scale(None)  # consume the device flag; advances state["step"] on a clean step
                 self._steps_dirty = True
                 return loss
@@ -281,17 +282,15 @@ class FP16Adam(torch.optim.Optimizer):
                         step_no = dict.__getitem__(st, "step") + 1
                         dict.__setitem__(st, "step", step_no)
             loss_scale = self.loss_scaler.loss_scale if self.loss_scaler is not None else -1
-            if n_dev:
+            if host_positions:
+                self._streamer.step(self.opt_id, step_no, lr, beta1, beta2, eps, weight_decay, loss_scale, table, n_dev)
+            elif n_dev:
                 _lib.check(
                     self._lib.ps_adam_step_chunks(
                         self.opt_id, step_no, lr, beta1, beta2, eps, weight_decay, 1, table, n_dev,
                         chunk_numel, float(loss_scale), stream,
                     ),
                     "ps_adam_step_chunks",
-                )
-            if host_positions:
-                self._streamer.step_static(
-                    self.opt_id, step_no, lr, beta1, beta2, eps, weight_decay, float(loss_scale), advance=(n_dev == 0)
                 )
             if self.loss_scaler:
                 self.loss_scaler.update_scale(False)

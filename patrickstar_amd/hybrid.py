@@ -5,7 +5,7 @@ updates them with the CPU operator (``patrickstar/ops/fp16_cpu_adam.py:415-428``
 ``patrickstar/ops/chunk_io_buff.py:214-255``).  On MI355X those chunks are instead
 copied into double-buffered HBM staging by ``hipMemcpyAsync`` on side streams,
 updated by the same fused kernel as resident chunks, and copied back, all ordered
-by events inside ``ps_adam_step_host_chunks``; the Python side only owns the
+by events inside ``ps_adam_step_hybrid``; the Python side only owns the
 staging buffers.
 """
 import torch
@@ -44,22 +44,16 @@ class HostChunkStreamer:
         self.staging = _lib.chunk_array([[t.data_ptr() for t in slot] for slot in self._slots])
         self._lib = _lib.load()
 
-    def step_static(self, opt_id, step_no, lr, beta1, beta2, eps, weight_decay, loss_scale, advance):
+    def step(self, opt_id, step_no, lr, beta1, beta2, eps, weight_decay, loss_scale, resident, n_resident, scaler=None):
+        """One optimizer step over the resident chunk array AND the host-resident chunks.
+        ``scaler`` (a device-resident DynamicLossScaler) selects the device-gated form."""
         _lib.check(
-            self._lib.ps_adam_step_host_chunks(
-                opt_id, step_no, lr, beta1, beta2, eps, weight_decay, 1, int(advance), self.host_table, self.n_host,
-                self.chunk_numel, self.staging, self.n_slots, float(loss_scale), None, _lib.current_stream_handle(),
+            self._lib.ps_adam_step_hybrid(
+                opt_id, step_no, lr, beta1, beta2, eps, weight_decay, 1, resident, n_resident, self.host_table,
+                self.n_host, self.chunk_numel, self.staging, self.n_slots, float(loss_scale),
+                scaler.state_ptr if scaler is not None else None, _lib.current_stream_handle(),
             ),
-            "ps_adam_step_host_chunks",
-        )
-
-    def step_gated(self, opt_id, lr, eps, weight_decay, scaler):
-        _lib.check(
-            self._lib.ps_adam_step_host_chunks(
-                opt_id, 0, lr, 0.0, 0.0, eps, weight_decay, 1, 0, self.host_table, self.n_host, self.chunk_numel,
-                self.staging, self.n_slots, -1.0, scaler.state_ptr, _lib.current_stream_handle(),
-            ),
-            "ps_adam_step_host_chunks",
+            "ps_adam_step_hybrid",
         )
 
     def scan_gradients(self, scaler):
