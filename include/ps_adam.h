@@ -112,6 +112,14 @@ const char* ps_last_error(void); /* text of the calling thread's latest failure 
 int ps_adam_create(int optimizer_id, float alpha, float beta1, float beta2, float eps,
                    float weight_decay, int adamw_mode, int should_log);
 
+/* FP16Adam's element-wise "gradient clipping" (patrickstar/ops/fp16_cpu_adam.py:364-379, the
+ * GPU branch): fp16 gradients are clamped to +-min(65504, gradient_clipping * loss_scale),
+ * the bound narrowed double -> float -> half as Tensor.clamp_ does.  Applied inside the
+ * chunk-list kernels (ps_adam_step_chunks, _gated, _hybrid) at no extra memory traffic; the
+ * device-gated form uses the device-resident scale.  ps_adam_update does not clamp (the
+ * reference clamps in Python before it calls the operator).  <= 0 switches it off (default). */
+int ps_adam_set_grad_clamp(int optimizer_id, double gradient_clipping);
+
 /* destroy_adam (cpu_adam.cpp:744-749).  Unknown ids are ignored, as there. */
 int ps_adam_destroy(int optimizer_id);
 

@@ -288,7 +288,7 @@ class OptimizerStepOracle:
     """
 
     def __init__(self, chunks, loss_scaler=None, lr=1e-3, betas=(0.9, 0.999), eps=1e-8,
-                 weight_decay=0.0, use_adamw=False, isa=ISA_AUTO):
+                 weight_decay=0.0, use_adamw=False, isa=ISA_AUTO, gradient_clipping=-1):
         self.chunks = chunks
         self.loss_scaler = loss_scaler
         self.lr, self.betas, self.eps, self.weight_decay = lr, betas, eps, weight_decay
@@ -296,6 +296,7 @@ class OptimizerStepOracle:
         self.step_count = 0
         self.has_overflow = False
         self.isa = isa
+        self.gradient_clipping = gradient_clipping
         self.native = AdamOracle(lr, betas[0], betas[1], eps, weight_decay, use_adamw)
 
     def check_overflow(self):
@@ -321,6 +322,18 @@ class OptimizerStepOracle:
         self.native.advance(self.step_count, self.betas[0], self.betas[1])
         self.native.set(self.lr, self.eps, self.weight_decay, True)
         L = lib()
+        if self.gradient_clipping > 0:
+            # fp16_cpu_adam.py:364-379, GPU branch: clamp_ of the fp16 gradient tensor to
+            # +-min(65504, clipping * loss_scale); the Python float bound narrows to float, then to half
+            bound = self.gradient_clipping
+            if self.loss_scaler is not None:
+                bound = bound * self.loss_scaler.loss_scale
+            bound = min(65504.0, bound)
+            b16 = np.float16(np.float32(bound))
+            for c in self.chunks:
+                g = c["p16"]
+                g[g < -b16] = -b16
+                g[g > b16] = b16
         for c in self.chunks:
             took = L.oracle_adam_span(
                 self.native._buf, _ptr(c["p32"]), _ptr(c["p16"]), 1, _ptr(c["m"]), _ptr(c["v"]),

@@ -73,6 +73,7 @@ SIGNATURES = {
     "ps_abi_version": (_i, []),
     "ps_last_error": (ctypes.c_char_p, []),
     "ps_adam_create": (_i, [_i, _f, _f, _f, _f, _f, _i, _i]),
+    "ps_adam_set_grad_clamp": (_i, [_i, _d]),
     "ps_adam_destroy": (_i, [_i]),
     "ps_adam_update": (_i, [_i, _sz, _f, _f, _f, _f, _f, _i, _vp, _vp, _i, _vp, _vp, _sz, _f, _vp, _vp]),
     "ps_adam_step_chunks": (_i, [_i, _sz, _f, _f, _f, _f, _f, _i, _vp, _i, _sz, _f, _vp]),

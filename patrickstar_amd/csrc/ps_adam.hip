@@ -94,6 +94,7 @@ struct HostAdam {
     float beta1_t = 1.0f, beta2_t = 1.0f;
     size_t step = 0;
     bool adamw;
+    double grad_clamp = -1.0;  // FP16Adam.gradient_clipping; <= 0: off
 
     // cpu_adam.h:143-162
     void advance(size_t s, float b1, float b2)
@@ -145,9 +146,47 @@ constexpr int UNSCALE_RUNTIME = -1;  // template value: look at StepConsts::unsc
 struct StepConsts {
     float beta1, beta2, b1m, b2m, bc2inv, eps, step_size, wd_term;
     float scale;  // loss scale (UNSCALE_DIV) or its exact reciprocal (UNSCALE_MUL)
+    float clip;   // element-wise clamp bound of the fp16 gradients (an fp16-representable value); 0 = off
     int wd_mode;
     int unscale;
 };
+
+// binary32 -> nearest binary16 (ties to even), returned as binary32.  Bit-level so that host and
+// device agree; inputs here are positive and at most 65504.
+__host__ __device__ inline float round_to_half_precision(float f)
+{
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    uint32_t e = (x >> 23) & 0xFFu;
+    if (e >= 255 || f == 0.0f) return f;
+    // bits of the float mantissa that do not fit: 13 for a normal half, more below 2^-14
+    int drop = e >= 113 ? 13 : (13 + (113 - (int)e));
+    if (drop >= 25) return 0.0f;
+    uint32_t m = (x & 0x7FFFFFu) | 0x800000u;
+    uint32_t rem = m & ((1u << drop) - 1u), half = 1u << (drop - 1);
+    m >>= drop;
+    if (rem > half || (rem == half && (m & 1u))) m += 1;
+    // value = m * 2^(e - 150 + drop)
+    float r = (float)m;
+    int shift = (int)e - 150 + drop;
+    uint32_t sbits = (uint32_t)(shift + 127) << 23;
+    float scale2;
+    memcpy(&scale2, &sbits, 4);
+    r = r * scale2;
+    return (x >> 31) ? -r : r;
+}
+
+// The bound of the reference's element-wise "gradient clipping" (fp16_cpu_adam.py:364-379, GPU
+// branch): min(65504, clipping * loss_scale) as a Python float, handed to Tensor.clamp_ on an fp16
+// tensor, i.e. narrowed double -> float -> half.  0 when clipping is off.
+__host__ __device__ inline float clamp_bound(double clipping, double loss_scale)
+{
+    if (!(clipping > 0.0)) return 0.0f;
+    double c = clipping;
+    if (loss_scale > 0.0) c = c * loss_scale;
+    if (65504.0 < c) c = 65504.0;
+    return round_to_half_precision((float)c);
+}
 
 // A power-of-two scale 2^k with 2^-k a normal float: g/scale == g*(1/scale)
 // bit for bit (the quotient is the same exact real number before the single
@@ -166,8 +205,9 @@ __host__ __device__ inline bool exact_reciprocal(float s, float* inv)
 __host__ __device__ inline void finish_consts(StepConsts& c, float lr, float beta1, float beta2,
                                               float eps, float wd, bool adamw, float beta1_t,
                                               float beta2_t, bool bias_correction,
-                                              float loss_scale)
+                                              float loss_scale, float clip)
 {
+    c.clip = clip;
     // cpu_adam.h:170-174
     float bc1 = 1.0f, bc2inv = 1.0f;
     if (bias_correction) {
@@ -201,6 +241,8 @@ template <int WD, int UNS>
 __device__ __forceinline__ void adam_element(const StepConsts& c, float g, float& p, float& m,
                                              float& v)
 {
+    // element-wise clamp of the fp16 gradient (comparisons, so a NaN stays a NaN like Tensor.clamp_)
+    if (c.clip > 0.0f) g = g < -c.clip ? -c.clip : (g > c.clip ? c.clip : g);
     if (UNS == UNSCALE_DIV) g = g / c.scale;
     if (UNS == UNSCALE_MUL) g = g * c.scale;
     if (WD == WD_L2) g = __builtin_fmaf(p, c.wd_term, g);
@@ -505,6 +547,7 @@ struct GatedArgs {
     float lr, eps, wd;
     int adamw;
     int bias_correction;
+    double grad_clamp;
 };
 
 // Device-decided step: overflow flag, loss scale and beta^t come from the
@@ -525,7 +568,8 @@ __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
     StepConsts c;
     // The operator takes loss_scale as a C float: the Python number narrows (RNE).
     finish_consts(c, ga.lr, st->beta1, st->beta2, ga.eps, ga.wd, ga.adamw != 0, st->beta1_t_next,
-                  st->beta2_t_next, ga.bias_correction != 0, (float)st->cur_scale);
+                  st->beta2_t_next, ga.bias_correction != 0, (float)st->cur_scale,
+                  clamp_bound(ga.grad_clamp, st->cur_scale));
     adam_tile<WD, UNSCALE_RUNTIME>(c, ch, base, chunk_numel);
 }
 
@@ -940,6 +984,14 @@ int ps_adam_create(int optimizer_id, float alpha, float beta1, float beta2, floa
     return 0;
 }
 
+int ps_adam_set_grad_clamp(int optimizer_id, double gradient_clipping)
+{
+    auto o = find_opt(optimizer_id);
+    if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
+    o->grad_clamp = gradient_clipping;
+    return 0;
+}
+
 int ps_adam_destroy(int optimizer_id)
 {
     std::lock_guard<std::mutex> lock(g_registry_mutex);
@@ -960,8 +1012,9 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
     o->set(lr, epsilon, weight_decay);
     if (numel == 0) return 0;
     StepConsts c;
+    // the reference clamps gradients in Python before it calls the operator: not here
     finish_consts(c, o->alpha, o->beta1, o->beta2, o->eps, o->weight_decay, o->adamw, o->beta1_t,
-                  o->beta2_t, bias_correction != 0, loss_scale);
+                  o->beta2_t, bias_correction != 0, loss_scale, 0.0f);
     unsigned grid = grid_1d((numel + kAuxBlock - 1) / kAuxBlock);
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define PS_FLAT(WD, HALF)                                                                  \
@@ -994,7 +1047,8 @@ int ps_adam_step_chunks(int optimizer_id, size_t step, float lr, float beta1, fl
     o->set(lr, epsilon, weight_decay);
     StepConsts c;
     finish_consts(c, o->alpha, o->beta1, o->beta2, o->eps, o->weight_decay, o->adamw, o->beta1_t,
-                  o->beta2_t, bias_correction != 0, loss_scale);
+                  o->beta2_t, bias_correction != 0, loss_scale,
+                  clamp_bound(o->grad_clamp, (double)loss_scale));
     hipStream_t s = static_cast<hipStream_t>(stream);
     return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid) {
         launch_adam_batch(b, grid, chunk_numel, c, s);
@@ -1017,6 +1071,7 @@ int ps_adam_step_chunks_gated(int optimizer_id, float lr, float epsilon, float w
     ga.wd = weight_decay;
     ga.adamw = o->adamw ? 1 : 0;
     ga.bias_correction = bias_correction;
+    ga.grad_clamp = o->grad_clamp;
     hipStream_t s = static_cast<hipStream_t>(stream);
     return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid) {
         launch_gated_batch(b, grid, chunk_numel, ga, d_state, s);
@@ -1070,13 +1125,15 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, float lr, float beta1, fl
         o->advance(step, beta1, beta2);
         o->set(lr, epsilon, weight_decay);
         finish_consts(c, o->alpha, o->beta1, o->beta2, o->eps, o->weight_decay, o->adamw,
-                      o->beta1_t, o->beta2_t, bias_correction != 0, loss_scale);
+                      o->beta1_t, o->beta2_t, bias_correction != 0, loss_scale,
+                      clamp_bound(o->grad_clamp, (double)loss_scale));
     } else {
         ga.lr = lr;
         ga.eps = epsilon;
         ga.wd = weight_decay;
         ga.adamw = o->adamw ? 1 : 0;
         ga.bias_correction = bias_correction;
+        ga.grad_clamp = o->grad_clamp;
     }
     hipStream_t caller = static_cast<hipStream_t>(stream);
     const bool stream_host = n_host_chunks > 0 && chunk_numel > 0;

@@ -82,10 +82,6 @@ class FP16Adam(torch.optim.Optimizer):
             raise ValueError("Invalid beta parameter at index 1: {}".format(betas[1]))
         if not 0.0 <= weight_decay:
             raise ValueError("Invalid weight_decay value: {}".format(weight_decay))
-        if gradient_clipping is not None and gradient_clipping > 0:
-            raise NotImplementedError(
-                "element-wise gradient clamping (gradient_clipping > 0) is not part of the fused step yet"
-            )
         # fail now, not at the first step, if the HIP library was never built
         self._lib = _lib.load()
         defaults = dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay, amsgrad=amsgrad)
@@ -136,6 +132,9 @@ class FP16Adam(torch.optim.Optimizer):
             "ps_adam_create",
         )
         self._created = True
+        if gradient_clipping is not None and gradient_clipping > 0:
+            # element-wise clamp of the fp16 gradients to +-min(65504, clipping * loss_scale), fused into the kernels
+            _lib.check(self._lib.ps_adam_set_grad_clamp(self.opt_id, float(gradient_clipping)), "ps_adam_set_grad_clamp")
         self._tables = None
         if self._dynamic and torch.cuda.is_available():
             self.loss_scaler.materialize(self.client.device, betas=betas)

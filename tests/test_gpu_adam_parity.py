@@ -285,3 +285,44 @@ def test_config4_first_and_last_chunk_of_24():
     for i in range(24):
         p, _, _, hh = h.payloads(i)
         assert torch.equal(p.half(), hh)
+
+
+# ---------------------------------------------------------------- element-wise gradient clamp
+
+@pytest.mark.parametrize("clipping,scale", [(1.0, 8), (0.3, 1000.0), (0.1, None), (5.0, 2**16), (1.0001, 8), (1e-3, 2**12)])
+def test_fused_gradient_clamp_matches_oracle_and_torch_clamp(clipping, scale):
+    """FP16Adam's "gradient clipping" is an element-wise clamp of the fp16 gradients to +-min(65504, clipping*scale)
+    (fp16_cpu_adam.py:364-379).  The fused form must equal (a) the oracle's restatement and (b) the library call the
+    reference itself makes: Tensor.clamp_ on the fp16 gradient tensor followed by an unclamped step."""
+    n = 2048 * 2 + 31
+    kw = dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
+    mk = lambda: None if scale is None else ps.LossScaler(scale)
+    a = ChunkHarness(2, n, mk(), seed=77, gradient_clipping=clipping, **kw)
+    b = ChunkHarness(2, n, mk(), seed=77, **kw)  # same seed -> same state and gradients
+    for h in (a, b):
+        h.fill_state()
+    oc = a.oracle_chunks()
+    oopt = oracle.OptimizerStepOracle(oc, None if scale is None else oracle.StaticScalerOracle(scale), gradient_clipping=clipping, **kw)
+    bound = min(65504.0, clipping * (scale if scale is not None else 1))
+    for step in range(2):
+        for h in (a, b):
+            h.fill_grads(bound / (scale or 1.0), scale or 1.0)  # scaled gradients ~ N(0, bound): about a third is clamped
+            g = h.payloads(1)[3]
+            g[3], g[4], g[5] = float("inf"), float("-inf"), float("nan")  # static scale: nothing is skipped
+        for i, c in enumerate(oc):
+            c["p16"][...] = a.download(i)[3]
+        clipped_fraction = float((a.payloads(0)[3].float().abs() > bound).float().mean())
+        assert 0.0 < clipped_fraction < 1.0, "the case must actually clamp something, and not everything"
+        for i in range(2):
+            b.payloads(i)[3].clamp_(-bound, bound)  # what the reference calls
+        a.opt.step()
+        b.opt.step()
+        oopt.step()
+        for i in range(2):
+            for x, y, key in zip(a.download(i), b.download(i), ("p32", "m", "v", "p16")):
+                nan = np.isnan(x.astype(np.float32))
+                assert np.array_equal(nan, np.isnan(y.astype(np.float32))) and np.array_equal(nan, np.isnan(oc[i][key].astype(np.float32)))
+                assert_bits_equal(x[~nan], y[~nan], f"step {step} chunk {i} {key}: fused clamp vs Tensor.clamp_")
+                assert_bits_equal(x[~nan], oc[i][key][~nan], f"step {step} chunk {i} {key}: fused clamp vs oracle")
+        # +-inf were clamped to the bound (finite), the NaN stayed a NaN
+        assert np.isfinite(a.download(1)[0][[3, 4]]).all() and np.isnan(a.download(1)[0][5])

@@ -269,3 +269,26 @@ def test_state_dict_round_trip_continues_bit_exact():
         for a, b in zip(h.payloads(i), final[i]):
             assert torch.equal(a.view(torch.int16 if a.dtype == torch.half else torch.int32), b.view(torch.int16 if b.dtype == torch.half else torch.int32))
     assert h.opt.loss_scaler.loss_scale == final_scale and h.opt.state[h.params[0]]["step"] == final_step == 7
+
+
+def test_fused_gradient_clamp_follows_the_device_resident_scale():
+    """With a dynamic scaler the clamp bound min(65504, clipping * loss_scale) moves with the scale, on the device."""
+    kw = dict(init_scale=2**8, scale_factor=2, scale_window=2, min_scale=1)
+    scaler = ps.DynamicLossScaler(**kw)
+    akw = dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0)
+    h = ChunkHarness(2, 2048 + 17, scaler, seed=31, gradient_clipping=0.002, **akw)
+    h.fill_state()
+    oc = h.oracle_chunks()
+    oscaler = oracle.ScalerOracle(**kw)
+    oopt = oracle.OptimizerStepOracle(oc, oscaler, gradient_clipping=0.002, **akw)
+    for step in range(7):
+        h.fill_grads(2e-3, float(oscaler.loss_scale))  # sigma == the clamp bound before scaling
+        if step == 4:
+            h.payloads(0)[3][9] = float("inf")
+        for i, c in enumerate(oc):
+            c["p16"][...] = h.download(i)[3]
+        h.opt.step()
+        oopt.check_overflow()
+        oopt.step()
+        h.compare(oc, what=f"clamp, dynamic scale, step {step}")
+    assert same_typed([scaler.loss_scale], [oscaler.loss_scale])
