@@ -56,6 +56,7 @@ class PatrickStarClient:
         self._param_idx = 0
         # fp16 chunk ids kept in pinned host memory together with their fp32 / m / v chunks
         self.host_fp16_chunk_ids = set()
+        self._slabs = []  # the allocations HBM-resident payloads are views of
         # called with (position index among fp16 chunks) -> True to keep that position in host memory
         self.host_chunk_policy: Optional[Callable[[int], bool]] = None
         default_opts = {"with_mem_saving_comm": False, "with_mem_cache": False, "with_async_move": False}
@@ -187,21 +188,39 @@ class PatrickStarClient:
         raise KeyError(chunk_id)
 
     def allocate_payloads(self):
-        """Give every chunk that has none a zero-filled payload (HBM, or pinned host memory
-        for positions the host-chunk policy selects).  Safe to call repeatedly."""
+        """Give every chunk that has none a zero-filled payload.  Safe to call repeatedly.
+
+        HBM-resident chunks of one list are carved out of ONE allocation per call (a slab): a few large
+        allocations are backed by large physical fragments, which the streaming kernels need when few waves
+        are in flight (measured: 6.30 TB/s from slabs vs 6.01 TB/s from one allocation per chunk; skewing the
+        slabs' start addresses against each other by a few KiB made no measurable difference).
+        Positions selected by the host-chunk policy get their own pinned host allocations instead.
+        """
         ids16 = self.chunk_tensor_index.chunk_type_to_chunk_id_list_map.get(ChunkType.PARAM_FP16, [])
         if self.host_chunk_policy is not None:
             for pos, cid in enumerate(ids16):
                 if self.host_chunk_policy(pos):
                     self.host_fp16_chunk_ids.add(cid)
+        pending = {}
         for chunk_id, chunk in self.chunk_list.generate_chunk():
             if chunk.payload is not None:
                 continue
-            on_host = self._fp16_chunk_of_position(chunk_id) in self.host_fp16_chunk_ids
-            if on_host:
+            if self._fp16_chunk_of_position(chunk_id) in self.host_fp16_chunk_ids:
                 chunk.allocate_payload("cpu", pin_memory=True)
             else:
-                chunk.allocate_payload(self.device)
+                pending.setdefault(chunk.chunk_type, []).append(chunk)
+        for chunk_type, chunks in pending.items():
+            if self.device.type == "cpu":
+                for chunk in chunks:
+                    chunk.allocate_payload(self.device)
+                continue
+            total = sum(c.capacity for c in chunks)
+            slab = torch.zeros(total, dtype=chunks[0].data_type, device=self.device)
+            self._slabs.append(slab)
+            cursor = 0
+            for chunk in chunks:
+                chunk.payload = slab.narrow(0, cursor, chunk.capacity)
+                cursor += chunk.capacity
 
     def chunk_ids_generator(self, chunk_type):
         for cid in self.chunk_tensor_index.chunk_type_to_chunk_id_list_map.get(chunk_type, []):

@@ -7,12 +7,13 @@
 //   * one pass over the data, in place; per lane one 16-byte access to each
 //     fp32 array and one 8-byte access to the fp16 array, so that every wave
 //     instruction covers a contiguous span of whole cache lines;
-//   * one small tile (512 elements) per workgroup and a CAP on resident waves
-//     (2 per SIMD): the pass touches four arrays for reading and the same four
+//   * one small tile (256 elements) per single-wave workgroup and a CAP on
+//     resident workgroups (9 per CU, enforced by requesting 17 KiB of unused
+//     dynamic LDS): the pass touches four arrays for reading and the same four
 //     for writing, and HBM efficiency drops when the set of in-flight cache
 //     lines gets wide; a narrow, steadily advancing window per array gave
-//     5.95 TB/s where the fully occupied machine gave 5.3 TB/s (a plain
-//     1-read-1-write copy peaks at 6.2 TB/s on the same GPU);
+//     6.3 TB/s where the fully occupied machine gave 5.3 TB/s (a plain
+//     1-read-1-write copy peaks at 6.2-6.3 TB/s on the same GPU);
 //   * chunk descriptors travel in the kernel-argument segment (64 per launch),
 //     so a wave's first data load depends on one scalar load, not two;
 //   * plain (temporal) loads/stores: non-temporal hints cost 20-25 %.
@@ -38,7 +39,7 @@
 
 // Build-time tuning knobs of the fused Adam kernels (defaults = measured best).
 #ifndef PS_BLOCK
-#define PS_BLOCK 128  // threads per workgroup
+#define PS_BLOCK 64  // threads per workgroup
 #endif
 #ifndef PS_LANE_ELEMS
 #define PS_LANE_ELEMS 4  // elements per lane per vector step (4 or 8)
@@ -47,7 +48,10 @@
 #define PS_UNROLL 1  // vector steps per lane per tile
 #endif
 #ifndef PS_MAX_WAVES_PER_EU
-#define PS_MAX_WAVES_PER_EU 2  // cap on resident waves per SIMD (0: no cap)
+#define PS_MAX_WAVES_PER_EU 0  // cap on resident waves per SIMD (0: no cap; the LDS request below does the capping)
+#endif
+#ifndef PS_LDS_KB
+#define PS_LDS_KB 17  // KiB of (unused) dynamic LDS requested per workgroup: caps resident workgroups per CU at floor(160 / PS_LDS_KB) = 9
 #endif
 #ifndef PS_STREAMING
 #define PS_STREAMING 0  // 1 marks chunk payload accesses non-temporal (slower on MI355X)
@@ -336,6 +340,7 @@ __device__ __forceinline__ void st_u4(uint16_t* p, uint4v v)
 }
 
 constexpr int kBlock = PS_BLOCK;
+constexpr unsigned kLdsBytes = PS_LDS_KB * 1024u;
 // Elements per lane per vector step.  8: one 16-byte access of fp16 and two
 // 16-byte accesses per fp32 array.  4: an 8-byte access of fp16 and one
 // 16-byte access per fp32 array.
@@ -862,11 +867,11 @@ void launch_adam_batch_wd(const ChunkBatch& b, dim3 grid, size_t chunk_numel, co
 {
     dim3 block(kBlock);
     if (c.unscale == UNSCALE_MUL)
-        hipLaunchKernelGGL((adam_chunks_kernel<WD, UNSCALE_MUL>), grid, block, 0, s, b, chunk_numel, c);
+        hipLaunchKernelGGL((adam_chunks_kernel<WD, UNSCALE_MUL>), grid, block, kLdsBytes, s, b, chunk_numel, c);
     else if (c.unscale == UNSCALE_DIV)
-        hipLaunchKernelGGL((adam_chunks_kernel<WD, UNSCALE_DIV>), grid, block, 0, s, b, chunk_numel, c);
+        hipLaunchKernelGGL((adam_chunks_kernel<WD, UNSCALE_DIV>), grid, block, kLdsBytes, s, b, chunk_numel, c);
     else
-        hipLaunchKernelGGL((adam_chunks_kernel<WD, UNSCALE_NONE>), grid, block, 0, s, b, chunk_numel, c);
+        hipLaunchKernelGGL((adam_chunks_kernel<WD, UNSCALE_NONE>), grid, block, kLdsBytes, s, b, chunk_numel, c);
 }
 
 void launch_adam_batch(const ChunkBatch& b, dim3 grid, size_t chunk_numel, const StepConsts& c,
@@ -886,11 +891,11 @@ void launch_gated_batch(const ChunkBatch& b, dim3 grid, size_t chunk_numel, cons
     dim3 block(kBlock);
     const bool decay = ga.wd > 0.0f;
     if (decay && ga.adamw)
-        hipLaunchKernelGGL(adam_chunks_gated_kernel<WD_DECOUPLED>, grid, block, 0, s, b, chunk_numel, ga, d_state);
+        hipLaunchKernelGGL(adam_chunks_gated_kernel<WD_DECOUPLED>, grid, block, kLdsBytes, s, b, chunk_numel, ga, d_state);
     else if (decay)
-        hipLaunchKernelGGL(adam_chunks_gated_kernel<WD_L2>, grid, block, 0, s, b, chunk_numel, ga, d_state);
+        hipLaunchKernelGGL(adam_chunks_gated_kernel<WD_L2>, grid, block, kLdsBytes, s, b, chunk_numel, ga, d_state);
     else
-        hipLaunchKernelGGL(adam_chunks_gated_kernel<WD_NONE>, grid, block, 0, s, b, chunk_numel, ga, d_state);
+        hipLaunchKernelGGL(adam_chunks_gated_kernel<WD_NONE>, grid, block, kLdsBytes, s, b, chunk_numel, ga, d_state);
 }
 
 // ------------------------------------------- host-resident chunks: streaming
