@@ -5,7 +5,7 @@ A "step" is one optimizer.step() over the whole chunk list: one launch of the fu
 reads every element's fp16 gradient and fp32 param/m/v once and writes fp32 param/m/v and the fp16 param
 once (28 algorithmic bytes per element).  Inputs are resident in HBM before the timed region.
 
-Workload (default): BASELINE config 4 -- 24 chunks of 64 Mi elements (1.61 G parameters incl. padding),
+Workload (default): the 1.5 B-parameter configuration -- 24 chunks of 64 Mi elements (1.61 G parameters incl. padding),
 g16 = (N(0,1e-3) * 2^12).half(), p ~ N(0,.02), m ~ N(0,1e-4), v = |N(0,1e-6)|, AdamW lr 1e-4
 betas (.9,.999) eps 1e-8 wd .01, static loss scale 2^12, first timed step t=100.
 
@@ -40,7 +40,7 @@ def parse_args():
                     help="with --mode hybrid: how many of --chunks live in pinned host memory (the LAST ones)")
     ap.add_argument("--slots", type=int, default=2, help="with --mode hybrid: HBM staging slots")
     ap.add_argument("--mode", choices=["static", "dynamic", "hybrid"], default="static",
-                    help="static: BASELINE config 4 as specified (static loss scale, one fused kernel per step). "
+                    help="static: the 1.5 B-parameter configuration as specified (static loss scale, one fused kernel per step). "
                     "dynamic: same data with a DynamicLossScaler: inf/nan scan (2 B/element) + device-gated kernel + "
                     "scaler update per step, no host sync")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -61,7 +61,7 @@ def traffic_from_profile():
 
 
 def cpu_baseline(reps):
-    """The CPU oracle on one 64 Mi-element chunk with BASELINE config 1 inputs, all host cores of this process."""
+    """The CPU oracle on one 64 Mi-element chunk with the one-chunk reference-CPU-path inputs (p~N(0,.02), m=v=0, g16=(N(0,1e-3)*8).half(), static scale 8), all host cores of this process."""
     import numpy as np
 
     import oracle
@@ -80,6 +80,10 @@ def cpu_baseline(reps):
         t0 = time.perf_counter()
         o.update(3 + r, 1e-3, 0.9, 0.999, 1e-6, 0.0, True, p, g, m, v, 8.0)
         best = min(best, time.perf_counter() - t0)
+    # the un-vectorised code path as well (what the reference's own builder selects on a non-Intel host)
+    t0 = time.perf_counter()
+    o.update(3 + reps, 1e-3, 0.9, 0.999, 1e-6, 0.0, True, p, g, m, v, 8.0, oracle.ISA_SCALAR)
+    scalar_s = time.perf_counter() - t0
     try:
         cores = len(os.sched_getaffinity(0))
     except AttributeError:
@@ -92,13 +96,14 @@ def cpu_baseline(reps):
         "unit": "params/s",
         "cores": cores,
         "kind": "port",
-        "sample": f"1 chunk of {n} elements (BASELINE config 1 inputs, static scale 8), best of {reps} steps after 2 warm-up; "
-        f"oracle code path {['', 'scalar', 'AVX2', 'AVX-512'][isa]}; 26 B/element -> {26 * n / best / 1e9:.0f} GB/s",
+        "sample": f"1 chunk of {n} elements (one-chunk CPU-path inputs, static scale 8), best of {reps} steps after 2 warm-up; "
+        f"oracle code path {['', 'scalar', 'AVX2', 'AVX-512'][isa]}; 26 B/element -> {26 * n / best / 1e9:.0f} GB/s; "
+        f"scalar code path of the same oracle, 1 step: {n / scalar_s / 1e9:.2f} G params/s",
     }
 
 
 def run_hybrid(args):
-    """BASELINE config 5 shape: C chunks, the last H of them in pinned host memory, streamed through HBM staging.
+    """The hybrid-placement configuration: C chunks, the last H of them in pinned host memory, streamed through HBM staging.
     Reports effective params/s over the whole list and the overlap efficiency
     max(kernel total, H2D total, D2H total) / wall."""
     import torch
@@ -193,7 +198,7 @@ def run_hybrid(args):
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": f"BASELINE config 5 shape: {C} chunks x {N} elements, {C - H} resident in HBM, {H} in pinned host memory "
+            "workload": f"hybrid placement: {C} chunks x {N} elements, {C - H} resident in HBM, {H} in pinned host memory "
             f"streamed through {args.slots} HBM staging slots (14 B/element each way over the host link)",
             "chunks": C, "host_chunks": H, "chunk_numel": N, "slots": args.slots,
         },
@@ -291,7 +296,7 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": f"BASELINE config 4: {C} chunks x {N} elements ({elements} parameters incl. padding) resident in HBM, "
+            "workload": f"1.5B-parameter chunk list: {C} chunks x {N} elements ({elements} parameters incl. padding) resident in HBM, "
             "AdamW lr 1e-4 betas (0.9,0.999) eps 1e-8 wd 0.01, static loss scale 2^12, fp16 grads -> fp32 p/m/v + fp16 params",
             "chunks": C,
             "chunk_numel": N,

@@ -221,10 +221,10 @@ def test_nonfinite_gradients_with_static_scale_propagate_like_the_oracle():
     assert np.isnan(p[[5, 9, 100]]).all() and h.opt.has_overflow is False
 
 
-# ---------------------------------------------------------------- BASELINE configurations
+# ---------------------------------------------------------------- the benchmark's named configurations
 
 def test_config1_one_full_chunk_ten_steps():
-    """BASELINE config 1: one 64 Mi-element chunk, p~N(0,.02), m=v=0, g16=(N(0,1e-3)*8).half(), static scale 8,
+    """Configuration "one chunk on the reference CPU path": one 64 Mi-element chunk, p~N(0,.02), m=v=0, g16=(N(0,1e-3)*8).half(), static scale 8,
     Adam lr 1e-3 betas (.9,.999) eps 1e-6 wd 0, steps 1..10.  Bit-exact against the oracle after every step."""
     h = ChunkHarness(1, N_FULL, ps.LossScaler(8), seed=0, lr=1e-3, betas=(0.9, 0.999), eps=1e-6, weight_decay=0)
     h.fill_state(m_std=0, v_std=0)
@@ -242,7 +242,7 @@ def test_config1_one_full_chunk_ten_steps():
 
 
 def test_config2_padded_two_chunks_cold_t100():
-    """BASELINE config 2: 124,439,808 parameters in 2 chunks of 64 Mi, zero tail; m~N(0,1e-4), v=|N(0,1e-6)|,
+    """Configuration "GPT-2-small-sized": 124,439,808 parameters in 2 chunks of 64 Mi, zero tail; m~N(0,1e-4), v=|N(0,1e-6)|,
     g16=(N(0,1e-3)*2^16).half(), AdamW wd .01 lr 1e-4, t=100 cold."""
     real = 124_439_808
     h = ChunkHarness(2, N_FULL, ps.LossScaler(2**16), used_numel_last=real - N_FULL, seed=1,
@@ -264,7 +264,7 @@ def test_config2_padded_two_chunks_cold_t100():
 
 
 def test_config4_first_and_last_chunk_of_24():
-    """BASELINE config 4 (the timed one): 24 chunks resident in HBM, AdamW lr 1e-4 eps 1e-8 wd .01, static scale 2^12,
+    """Configuration "GPT-2-1.5B-sized" (the timed one): 24 chunks resident in HBM, AdamW lr 1e-4 eps 1e-8 wd .01, static scale 2^12,
     t=100.  The oracle checks the first and the last chunk; a checksum guards the ones in between against being skipped."""
     h = ChunkHarness(24, N_FULL, ps.LossScaler(2**12), seed=4, lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
     h.fill_state()

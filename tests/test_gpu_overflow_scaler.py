@@ -180,7 +180,7 @@ def test_gated_step_non_power_of_two_scale_uses_true_division():
         assert same_typed([scaler.loss_scale], [oscaler.loss_scale])
 
 
-# ---------------------------------------------------------------- BASELINE config 3 at full size
+# ---------------------------------------------------------------- the overflow / loss-scale configuration at full size
 
 def test_config3_full_size_flags_and_scale_trajectory():
     """8 chunks of 64 Mi elements, 200 steps, a seeded 5 % of them poisoned with +-inf/nan at 1..16 positions

@@ -102,7 +102,7 @@ def test_scale_is_init_times_power_of_factor_property():
 
 
 def test_config3_expectation():
-    """BASELINE config 3: 10 overflows in 200 steps, window 1000 -> ten halvings, no growth."""
+    """The overflow / loss-scale configuration: 10 overflows in 200 steps, window 1000 -> ten halvings, no growth."""
     rng = np.random.default_rng(0)
     bad = set(rng.choice(200, size=10, replace=False).tolist())
     s = scaler_from_config({"enabled": True, "loss_scale": 0, "initial_scale_power": 16, "loss_scale_window": 1000, "hysteresis": 2, "min_loss_scale": 1})
