@@ -620,6 +620,52 @@ __global__ void __launch_bounds__(kAuxBlock)
     }
 }
 
+// The same operator on a span whose four (five) addresses share one 16-byte phase: single-wave
+// workgroups over 256-element tiles with 16-byte accesses, resident-workgroup cap as for the chunk
+// kernels.  Gradients are read only; the fp16 output is optional.
+template <int WD, bool GRAD_HALF>
+__global__ void __launch_bounds__(64)
+    adam_flat_vec_kernel(StepConsts c, float* p32, const void* grads, float* m32, float* v32,
+                         uint16_t* out16,  // may alias grads (fp16 gradients overwritten by fp16 parameters)
+                         size_t n_tiles)
+{
+    for (size_t t = blockIdx.x; t < n_tiles; t += gridDim.x) {
+        const size_t i = (t * 64 + threadIdx.x) * 4;
+        float g[4];
+        if (GRAD_HALF) {
+            uint2v w = *(const guint2v*)(static_cast<const uint16_t*>(grads) + i);
+            g[0] = half_bits_to_float(w[0] & 0xFFFFu);
+            g[1] = half_bits_to_float(w[0] >> 16);
+            g[2] = half_bits_to_float(w[1] & 0xFFFFu);
+            g[3] = half_bits_to_float(w[1] >> 16);
+        } else {
+            float4v gv = ld_f4(static_cast<const float*>(grads) + i);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) g[e] = gv[e];
+        }
+        float4v p = ld_f4(p32 + i), m = ld_f4(m32 + i), v = ld_f4(v32 + i);
+        uint32_t h[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float pe = p[e], me = m[e], ve = v[e];
+            element_any<WD, UNSCALE_RUNTIME>(c, g[e], pe, me, ve);
+            p[e] = pe;
+            m[e] = me;
+            v[e] = ve;
+            h[e] = float_to_half_bits(pe);
+        }
+        st_f4(p32 + i, p);
+        st_f4(m32 + i, m);
+        st_f4(v32 + i, v);
+        if (out16 != nullptr) {
+            uint2v o;
+            o[0] = h[0] | (h[1] << 16);
+            o[1] = h[2] | (h[3] << 16);
+            *(guint2v*)(out16 + i) = o;
+        }
+    }
+}
+
 // ----------------------------------------------------------- overflow scan
 //
 // A binary16 value is inf or nan iff its five exponent bits are all set.
@@ -723,6 +769,81 @@ __global__ void __launch_bounds__(kAuxBlock)
         uint32_t h = SRC_HALF ? (uint32_t)sh[i] : float_to_half_bits(sf[i]);
         dst[i] = (uint16_t)h;
         hit |= ((h & 0x7C00u) == 0x7C00u) ? 1u : 0u;
+    }
+    if (st != nullptr) block_flag_commit(hit, &st->overflow);
+}
+
+// Vector form of the same copy for long gradients.  The chunk slot sets the grid: 16-byte stores to
+// 16-byte aligned addresses of the slot.  A fp16 source is generally at a different phase, so each lane
+// loads the two ALIGNED 16-byte source blocks that straddle its output vector and funnel-shifts them by
+// S halves in registers; no misaligned memory access is made.  Every 16-byte block that is loaded holds
+// at least one element of the gradient, so it lies inside the gradient's allocation.
+template <int S>
+__device__ __forceinline__ uint4v shift_halves(const uint4v& a, const uint4v& b)
+{
+    const uint32_t w[8] = {a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+    constexpr int d = (2 * S) / 4, r = (2 * S) % 4;
+    uint4v o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = r ? ((w[i + d] >> 16) | (w[i + d + 1] << 16)) : w[i + d];
+    return o;
+}
+
+template <int S>
+__device__ __forceinline__ uint32_t copy_shifted_f16(const uint16_t* src_al, uint16_t* dst_al,
+                                                      size_t n_vec)
+{
+    uint32_t hit = 0;
+    size_t stride = (size_t)gridDim.x * kAuxBlock;
+    for (size_t j = (size_t)blockIdx.x * kAuxBlock + threadIdx.x; j < n_vec; j += stride) {
+        uint4v a = ld_u4(src_al + 8 * j);
+        uint4v b = a;
+        if (S != 0) b = ld_u4(src_al + 8 * j + 8);
+        uint4v o = shift_halves<S>(a, b);
+        hit |= nonfinite_halves(o[0]) | nonfinite_halves(o[1]) | nonfinite_halves(o[2]) |
+               nonfinite_halves(o[3]);
+        st_u4(dst_al + 8 * j, o);
+    }
+    return hit;
+}
+
+__global__ void __launch_bounds__(kAuxBlock)
+    grad_to_chunk_f16_vec_kernel(const uint16_t* __restrict__ src_al, int shift,
+                                 uint16_t* __restrict__ dst_al, size_t n_vec, ps_step_state* st)
+{
+    uint32_t hit = 0;
+    switch (shift) {
+        case 0: hit = copy_shifted_f16<0>(src_al, dst_al, n_vec); break;
+        case 1: hit = copy_shifted_f16<1>(src_al, dst_al, n_vec); break;
+        case 2: hit = copy_shifted_f16<2>(src_al, dst_al, n_vec); break;
+        case 3: hit = copy_shifted_f16<3>(src_al, dst_al, n_vec); break;
+        case 4: hit = copy_shifted_f16<4>(src_al, dst_al, n_vec); break;
+        case 5: hit = copy_shifted_f16<5>(src_al, dst_al, n_vec); break;
+        case 6: hit = copy_shifted_f16<6>(src_al, dst_al, n_vec); break;
+        default: hit = copy_shifted_f16<7>(src_al, dst_al, n_vec); break;
+    }
+    if (st != nullptr) block_flag_commit(hit, &st->overflow);
+}
+
+// fp32 gradients: eight dword-aligned floats per output vector (multi-dword loads need dword alignment only).
+typedef float4v __attribute__((aligned(4))) float4v_dword_aligned;
+__global__ void __launch_bounds__(kAuxBlock)
+    grad_to_chunk_f32_vec_kernel(const float* __restrict__ src, uint16_t* __restrict__ dst_al,
+                                 size_t n_vec, ps_step_state* st)
+{
+    uint32_t hit = 0;
+    size_t stride = (size_t)gridDim.x * kAuxBlock;
+    for (size_t j = (size_t)blockIdx.x * kAuxBlock + threadIdx.x; j < n_vec; j += stride) {
+        float4v x = *(const PS_GLOBAL float4v_dword_aligned*)(src + 8 * j);
+        float4v y = *(const PS_GLOBAL float4v_dword_aligned*)(src + 8 * j + 4);
+        uint4v o;
+        o[0] = float_to_half_bits(x[0]) | (float_to_half_bits(x[1]) << 16);
+        o[1] = float_to_half_bits(x[2]) | (float_to_half_bits(x[3]) << 16);
+        o[2] = float_to_half_bits(y[0]) | (float_to_half_bits(y[1]) << 16);
+        o[3] = float_to_half_bits(y[2]) | (float_to_half_bits(y[3]) << 16);
+        hit |= nonfinite_halves(o[0]) | nonfinite_halves(o[1]) | nonfinite_halves(o[2]) |
+               nonfinite_halves(o[3]);
+        st_u4(dst_al + 8 * j, o);
     }
     if (st != nullptr) block_flag_commit(hit, &st->overflow);
 }
@@ -1020,21 +1141,70 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
     // the reference clamps gradients in Python before it calls the operator: not here
     finish_consts(c, o->alpha, o->beta1, o->beta2, o->eps, o->weight_decay, o->adamw, o->beta1_t,
                   o->beta2_t, bias_correction != 0, loss_scale, 0.0f);
-    unsigned grid = grid_1d((numel + kAuxBlock - 1) / kAuxBlock);
     hipStream_t s = static_cast<hipStream_t>(stream);
-#define PS_FLAT(WD, HALF)                                                                  \
-    hipLaunchKernelGGL((adam_flat_kernel<WD, HALF>), dim3(grid), dim3(kAuxBlock), 0, s, c, \
-                       d_params, d_grads, d_exp_avg, d_exp_avg_sq, d_param_fp16_out, numel)
-    if (grads_are_half) {
-        if (c.wd_mode == WD_DECOUPLED) PS_FLAT(WD_DECOUPLED, true);
-        else if (c.wd_mode == WD_L2) PS_FLAT(WD_L2, true);
-        else PS_FLAT(WD_NONE, true);
-    } else {
-        if (c.wd_mode == WD_DECOUPLED) PS_FLAT(WD_DECOUPLED, false);
-        else if (c.wd_mode == WD_L2) PS_FLAT(WD_L2, false);
-        else PS_FLAT(WD_NONE, false);
-    }
+    const size_t gsz = grads_are_half ? 2 : 4;
+    const char* gbytes = static_cast<const char*>(d_grads);
+
+    // element-wise pass over [lo, hi)
+    auto scalar_span = [&](size_t lo, size_t hi) {
+        if (hi <= lo) return;
+        const size_t n = hi - lo;
+        dim3 grid(grid_1d((n + kAuxBlock - 1) / kAuxBlock)), block(kAuxBlock);
+        uint16_t* out = d_param_fp16_out ? d_param_fp16_out + lo : nullptr;
+#define PS_FLAT(WD, HALF)                                                                      \
+    hipLaunchKernelGGL((adam_flat_kernel<WD, HALF>), grid, block, 0, s, c, d_params + lo,      \
+                       static_cast<const void*>(gbytes + lo * gsz), d_exp_avg + lo,            \
+                       d_exp_avg_sq + lo, out, n)
+        if (grads_are_half) {
+            if (c.wd_mode == WD_DECOUPLED) PS_FLAT(WD_DECOUPLED, true);
+            else if (c.wd_mode == WD_L2) PS_FLAT(WD_L2, true);
+            else PS_FLAT(WD_NONE, true);
+        } else {
+            if (c.wd_mode == WD_DECOUPLED) PS_FLAT(WD_DECOUPLED, false);
+            else if (c.wd_mode == WD_L2) PS_FLAT(WD_L2, false);
+            else PS_FLAT(WD_NONE, false);
+        }
 #undef PS_FLAT
+    };
+
+    // Tensors handed to the operator are views at one element offset into the four chunk
+    // payloads, so their addresses normally share a phase relative to 16-byte (4-element)
+    // boundaries: peel up to 3 leading elements, run whole 256-element tiles with vector
+    // accesses, finish the remainder element-wise.
+    auto elem_phase = [](const void* a, size_t elem_size) -> int {
+        uintptr_t u = reinterpret_cast<uintptr_t>(a);
+        if (u % elem_size) return -1;
+        return (int)((u / elem_size) & 3u);
+    };
+    const int ph = elem_phase(d_params, 4);
+    bool vec_ok = ph >= 0 && numel >= 4096 && elem_phase(d_exp_avg, 4) == ph &&
+                  elem_phase(d_exp_avg_sq, 4) == ph && elem_phase(d_grads, gsz) == ph &&
+                  (d_param_fp16_out == nullptr || elem_phase(d_param_fp16_out, 2) == ph);
+    if (!vec_ok) {
+        scalar_span(0, numel);
+    } else {
+        const size_t head = (size_t)((4 - ph) & 3);
+        const size_t n_tiles = (numel - head) / 256;
+        const size_t body_end = head + n_tiles * 256;
+        scalar_span(0, head);
+        dim3 grid(grid_1d(n_tiles)), block(64);
+        uint16_t* out = d_param_fp16_out ? d_param_fp16_out + head : nullptr;
+#define PS_FLAT_VEC(WD, HALF)                                                                     \
+    hipLaunchKernelGGL((adam_flat_vec_kernel<WD, HALF>), grid, block, kLdsBytes, s, c,            \
+                       d_params + head, static_cast<const void*>(gbytes + head * gsz),            \
+                       d_exp_avg + head, d_exp_avg_sq + head, out, n_tiles)
+        if (grads_are_half) {
+            if (c.wd_mode == WD_DECOUPLED) PS_FLAT_VEC(WD_DECOUPLED, true);
+            else if (c.wd_mode == WD_L2) PS_FLAT_VEC(WD_L2, true);
+            else PS_FLAT_VEC(WD_NONE, true);
+        } else {
+            if (c.wd_mode == WD_DECOUPLED) PS_FLAT_VEC(WD_DECOUPLED, false);
+            else if (c.wd_mode == WD_L2) PS_FLAT_VEC(WD_L2, false);
+            else PS_FLAT_VEC(WD_NONE, false);
+        }
+#undef PS_FLAT_VEC
+        scalar_span(body_end, numel);
+    }
     PS_HIP(hipGetLastError());
     return 0;
 }
@@ -1348,15 +1518,47 @@ int ps_grad_to_chunk(const void* d_grad, int grad_is_half, uint16_t* d_slot_fp16
 {
     if (numel == 0) return 0;
     if (!d_grad || !d_slot_fp16) return fail(PS_ERR_BAD_ARG, "ps_grad_to_chunk: NULL pointer");
-    size_t blocks = (numel + (size_t)kAuxBlock * 4 - 1) / ((size_t)kAuxBlock * 4);
-    dim3 grid(grid_1d(blocks)), block(kAuxBlock);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (grad_is_half)
-        hipLaunchKernelGGL(grad_to_chunk_kernel<true>, grid, block, 0, s, d_grad, d_slot_fp16, numel,
-                           d_state);
-    else
-        hipLaunchKernelGGL(grad_to_chunk_kernel<false>, grid, block, 0, s, d_grad, d_slot_fp16,
-                           numel, d_state);
+    const size_t esz = grad_is_half ? 2 : 4;
+    const char* gbytes = static_cast<const char*>(d_grad);
+
+    auto scalar_span = [&](size_t lo, size_t hi) {
+        if (hi <= lo) return;
+        const size_t n = hi - lo;
+        size_t blocks = (n + (size_t)kAuxBlock * 4 - 1) / ((size_t)kAuxBlock * 4);
+        dim3 grid(grid_1d(blocks)), block(kAuxBlock);
+        const void* src = gbytes + lo * esz;
+        if (grad_is_half)
+            hipLaunchKernelGGL(grad_to_chunk_kernel<true>, grid, block, 0, s, src, d_slot_fp16 + lo, n, d_state);
+        else
+            hipLaunchKernelGGL(grad_to_chunk_kernel<false>, grid, block, 0, s, src, d_slot_fp16 + lo, n, d_state);
+    };
+
+    const uintptr_t dst = reinterpret_cast<uintptr_t>(d_slot_fp16);
+    const uintptr_t src = reinterpret_cast<uintptr_t>(d_grad);
+    const bool addressable = (dst % 2 == 0) && (src % esz == 0);
+    if (!addressable || numel < 4096) {
+        scalar_span(0, numel);
+    } else {
+        // elements before the slot's first 16-byte boundary, whole 8-element vectors, remainder
+        const size_t head = (size_t)(((16 - dst % 16) % 16) / 2);
+        const size_t n_vec = (numel - head) / 8;
+        const size_t body_end = head + n_vec * 8;
+        scalar_span(0, head);
+        size_t blocks = (n_vec + kAuxBlock - 1) / kAuxBlock;
+        dim3 grid(grid_1d(blocks)), block(kAuxBlock);
+        uint16_t* dst_al = d_slot_fp16 + head;
+        if (grad_is_half) {
+            const uintptr_t first = src + head * 2;
+            const int shift = (int)((first % 16) / 2);
+            const uint16_t* src_al = reinterpret_cast<const uint16_t*>(first - (uintptr_t)shift * 2);
+            hipLaunchKernelGGL(grad_to_chunk_f16_vec_kernel, grid, block, 0, s, src_al, shift, dst_al, n_vec, d_state);
+        } else {
+            hipLaunchKernelGGL(grad_to_chunk_f32_vec_kernel, grid, block, 0, s,
+                               static_cast<const float*>(d_grad) + head, dst_al, n_vec, d_state);
+        }
+        scalar_span(body_end, numel);
+    }
     PS_HIP(hipGetLastError());
     return 0;
 }

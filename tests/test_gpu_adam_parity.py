@@ -326,3 +326,63 @@ def test_fused_gradient_clamp_matches_oracle_and_torch_clamp(clipping, scale):
                 assert_bits_equal(x[~nan], oc[i][key][~nan], f"step {step} chunk {i} {key}: fused clamp vs oracle")
         # +-inf were clamped to the bound (finite), the NaN stayed a NaN
         assert np.isfinite(a.download(1)[0][[3, 4]]).all() and np.isnan(a.download(1)[0][5])
+
+
+@pytest.mark.parametrize("phase", [0, 1, 2, 3])
+@pytest.mark.parametrize("grad_dtype", [np.float16, np.float32])
+def test_adam_update_vector_path_all_phases(phase, grad_dtype):
+    """Large tensors take the operator's vector path: views starting 0..3 elements into their buffers (the phase a
+    tensor has inside its chunks), fp16 and fp32 gradients, fp16 output aliasing the fp16 gradients or absent."""
+    lib = _lib.load()
+    rng = np.random.default_rng(100 + phase)
+    n = 256 * 40 + 131  # 40 whole tiles + a remainder, beyond the 4096-element threshold
+    tot = n + phase
+    p = rng.normal(0, 0.02, tot).astype(np.float32)
+    m = rng.normal(0, 1e-4, tot).astype(np.float32)
+    v = np.abs(rng.normal(0, 1e-6, tot)).astype(np.float32)
+    g = (rng.normal(0, 1e-3, tot) * 64).astype(grad_dtype)
+    dp, dm, dv, dg = _dev(p.copy()), _dev(m.copy()), _dev(v.copy()), _dev(g.copy())
+    half = grad_dtype == np.float16
+    out = dg if half else None  # fp16 parameters overwrite the fp16 gradients, as in the chunk layout
+    oid = 903
+    lib.ps_adam_create(oid, 1e-3, 0.9, 0.999, 1e-8, 0.01, 1, 0)
+    rc = lib.ps_adam_update(oid, 5, 1e-3, 0.9, 0.999, 1e-8, 0.01, 1, dp[phase:].data_ptr(), dg[phase:].data_ptr(), int(half),
+                            dm[phase:].data_ptr(), dv[phase:].data_ptr(), n, 64.0, out[phase:].data_ptr() if out is not None else None,
+                            _lib.current_stream_handle())
+    assert rc == 0
+    torch.cuda.synchronize()
+    lib.ps_adam_destroy(oid)
+    po, mo, vo = p[phase:].copy(), m[phase:].copy(), v[phase:].copy()
+    oracle.AdamOracle(1e-3, 0.9, 0.999, 1e-8, 0.01, True).update(5, 1e-3, 0.9, 0.999, 1e-8, 0.01, True, po, g[phase:].copy(), mo, vo, 64.0)
+    assert_bits_equal(dp.cpu().numpy()[phase:], po, "param")
+    assert_bits_equal(dm.cpu().numpy()[phase:], mo, "exp_avg")
+    assert_bits_equal(dv.cpu().numpy()[phase:], vo, "exp_avg_sq")
+    if half:
+        assert_bits_equal(dg.cpu().numpy()[phase:], oracle.cast_fp32_to_fp16(po), "fp16 params over the gradients")
+    else:
+        assert_bits_equal(dg.cpu().numpy(), g, "fp32 gradients untouched")
+    for t, ref in ((dp, p), (dm, m), (dv, v)):
+        assert_bits_equal(t.cpu().numpy()[:phase], ref[:phase], "elements before the view")
+
+
+def test_adam_update_mismatched_phases_fall_back_to_elementwise():
+    lib = _lib.load()
+    rng = np.random.default_rng(9)
+    n = 9000
+    p = rng.normal(0, 0.02, n + 3).astype(np.float32)
+    m = rng.normal(0, 1e-4, n + 3).astype(np.float32)
+    v = np.abs(rng.normal(0, 1e-6, n + 3)).astype(np.float32)
+    g = (rng.normal(0, 1e-3, n + 3)).astype(np.float16)
+    dp, dm, dv, dg = _dev(p.copy()), _dev(m.copy()), _dev(v.copy()), _dev(g.copy())
+    oid = 904
+    lib.ps_adam_create(oid, 1e-3, 0.9, 0.999, 1e-8, 0.0, 0, 0)
+    rc = lib.ps_adam_update(oid, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, dp[1:].data_ptr(), dg[3:].data_ptr(), 1, dm[2:].data_ptr(),
+                            dv.data_ptr(), n, -1.0, None, _lib.current_stream_handle())
+    assert rc == 0
+    torch.cuda.synchronize()
+    lib.ps_adam_destroy(oid)
+    po, mo, vo = p[1:1 + n].copy(), m[2:2 + n].copy(), v[:n].copy()
+    oracle.AdamOracle(1e-3, 0.9, 0.999, 1e-8, 0.0, False).update(1, 1e-3, 0.9, 0.999, 1e-8, 0.0, True, po, g[3:3 + n].copy(), mo, vo, -1.0)
+    assert_bits_equal(dp.cpu().numpy()[1:1 + n], po, "param")
+    assert_bits_equal(dm.cpu().numpy()[2:2 + n], mo, "exp_avg")
+    assert_bits_equal(dv.cpu().numpy()[:n], vo, "exp_avg_sq")

@@ -292,3 +292,50 @@ def test_fused_gradient_clamp_follows_the_device_resident_scale():
         oopt.step()
         h.compare(oc, what=f"clamp, dynamic scale, step {step}")
     assert same_typed([scaler.loss_scale], [oscaler.loss_scale])
+
+
+# ---------------------------------------------------------------- backward-side producer
+
+@pytest.mark.parametrize("src_dtype", [torch.half, torch.float])
+def test_grad_to_chunk_all_alignments_and_probe(src_dtype):
+    """ps_grad_to_chunk == slot.copy_(grad) (RNE for fp32 sources) for every relative alignment of gradient and chunk
+    slot, short (element-wise) and long (vector) gradients; the fused probe sees a non-finite value wherever it sits."""
+    lib = _lib.load()
+    stream = _lib.current_stream_handle()
+    for n in (1, 37, 4095, 4096, 4096 + 8 * 300 + 5):
+        for src_off in range(0, 9):
+            for dst_off in (0, 1, 3, 7, 8, 13):
+                if n < 4096 and (src_off > 2 or dst_off > 3):
+                    continue
+                g_all = (torch.randn(n + 16, device="cuda") * 50).to(src_dtype)
+                slot_all = torch.full((n + 32,), 7.0, dtype=torch.half, device="cuda")
+                g, slot = g_all[src_off:src_off + n], slot_all[dst_off:dst_off + n]
+                scaler = ps.DynamicLossScaler(init_scale=2**4)
+                rc = lib.ps_grad_to_chunk(g.data_ptr(), int(src_dtype == torch.half), slot.data_ptr(), n, scaler.state_ptr, stream)
+                assert rc == 0
+                want = torch.full_like(slot_all, 7.0)
+                want[dst_off:dst_off + n].copy_(g)
+                assert torch.equal(slot_all.view(torch.int16), want.view(torch.int16)), (n, src_off, dst_off)
+                assert scaler.overflow_flag is False
+    # the probe: positions in the head, the vector body and the tail, for a misaligned pair
+    n = 4096 + 8 * 300 + 5
+    for pos in (0, 2, 9, n // 2, n - 9, n - 1):
+        for bad in (float("inf"), float("nan")):
+            g_all = (torch.randn(n + 16, device="cuda") * 50).to(src_dtype)
+            slot_all = torch.zeros(n + 32, dtype=torch.half, device="cuda")
+            g, slot = g_all[3:3 + n], slot_all[5:5 + n]
+            g[pos] = bad
+            scaler = ps.DynamicLossScaler(init_scale=2**4)
+            assert lib.ps_grad_to_chunk(g.data_ptr(), int(src_dtype == torch.half), slot.data_ptr(), n, scaler.state_ptr, stream) == 0
+            assert scaler.overflow_flag is True, (pos, bad)
+    if src_dtype == torch.float:  # a finite fp32 gradient beyond the fp16 range lands as inf in the chunk: flagged
+        g = torch.full((5000,), 1e6, device="cuda")
+        slot = torch.zeros(5000, dtype=torch.half, device="cuda")
+        scaler = ps.DynamicLossScaler(init_scale=2**4)
+        assert lib.ps_grad_to_chunk(g.data_ptr(), 0, slot.data_ptr(), 5000, scaler.state_ptr, stream) == 0
+        assert scaler.overflow_flag is True and torch.isinf(slot).all()
+    # without a state pointer it is a plain copy
+    g = torch.randn(6000, device="cuda").half()
+    slot = torch.zeros(6001, dtype=torch.half, device="cuda")
+    assert lib.ps_grad_to_chunk(g.data_ptr(), 1, slot[1:].data_ptr(), 6000, None, stream) == 0
+    assert torch.equal(slot[1:], g)
