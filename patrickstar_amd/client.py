@@ -129,6 +129,10 @@ class PatrickStarClient:
         constructing before their parent does), copy the initial values into the fp16 and fp32
         payloads and re-point each parameter at its fp16 chunk slot."""
         self.module = model
+        if self.host_chunk_policy is not None:
+            # a module's parameters must be views of fp16 payloads in HBM; host-resident positions are for
+            # chunk lists that are driven directly (append_flat_chunks / explicit payload access)
+            raise NotImplementedError("host_chunk_policy cannot be combined with register_model")
 
         def visit(m):
             for child in m.children():
@@ -143,10 +147,7 @@ class PatrickStarClient:
             slot32 = self.access_data(self.param_fp16_to_param_fp32_map[p16])
             slot32.copy_(init.to(slot32.device, torch.float))
             slot16.copy_(slot32)
-            if slot16.device.type != "cpu":
-                p16.data = slot16
-            else:
-                p16.data = init.to(torch.half)
+            p16.data = slot16  # the module now computes with the chunk's own memory
         return model
 
     def append_flat_chunks(self, n_chunks: int, used_numel_last: Optional[int] = None):

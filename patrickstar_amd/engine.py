@@ -72,6 +72,9 @@ class PatrickStarEngine(torch.nn.Module):
         self.module.train()
         self.client = client
         optim_type, optim_params, self.loss_scaler, self.gradient_clipping = parse_config(config)
+        # parameters already live in the fp16 chunks on the device; buffers follow them (runtime/engine.py:134-138)
+        for buffer in model.buffers():
+            buffer.data = buffer.data.to(self.client.device)
         self.optimizer = FP16Adam(
             self.client,
             self.module.parameters(),

@@ -1,0 +1,57 @@
+"""The reference's optimizer-construction smoke test (unitest/test_optimizer_init.py:45-60: FP16Adam over a BERT built
+from a local config) restated against this engine, extended by a few training iterations."""
+import pytest
+import torch
+
+import patrickstar_amd as ps
+from patrickstar_amd.chunk_layout import AccessType, ChunkType
+
+pytestmark = pytest.mark.gpu
+
+
+def test_engine_trains_a_small_bert():
+    transformers = pytest.importorskip("transformers")
+    cfg = transformers.BertConfig(
+        vocab_size=512, hidden_size=64, num_hidden_layers=2, num_attention_heads=4, intermediate_size=128,
+        max_position_embeddings=64, num_labels=2, hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0,
+    )
+    torch.manual_seed(0)
+    config = {
+        "optimizer": {"type": "Adam", "params": {"lr": 1e-3, "betas": (0.9, 0.999), "eps": 1e-6, "weight_decay": 0, "use_hybrid_adam": True}},
+        "fp16": {"enabled": True, "loss_scale": 0, "initial_scale_power": 10, "loss_scale_window": 1000, "hysteresis": 2, "min_loss_scale": 1},
+        "default_chunk_size": 32 * 1024,
+        "release_after_init": False,
+        "use_cpu_embedding": False,
+    }
+    engine, optimizer = ps.initialize_engine(
+        model_func=lambda: transformers.BertForSequenceClassification(cfg), local_rank=0, config=config
+    )
+    client = engine.client
+    n_params = sum(p.numel() for p in engine.module.parameters())
+    pos = client.positions()
+    assert len(pos) >= 3 and all(q.exp_avg is not None and q.exp_avg_sq is not None for q in pos)
+    assert sum(client.chunk_tensor_index.used_numel(q.fp16) for q in pos) == n_params
+    idx = client.chunk_tensor_index
+    for p in engine.module.parameters():
+        assert p.dtype == torch.half and p.is_cuda
+        info = idx.get_tensor_info(p.ps_attr.data_id())
+        for key in ("exp_avg", "exp_avg_sq"):
+            sp = dict.__getitem__(optimizer.state[p], key)
+            assert idx.get_tensor_info(sp.ps_attr.data_id()).start_offset == info.start_offset
+        assert p.data_ptr() == client.chunk_list[info.chunk_id].payload.data_ptr() + 2 * info.start_offset
+
+    ids = torch.randint(0, 512, (8, 32), device="cuda")
+    labels = torch.randint(0, 2, (8,), device="cuda")
+    losses = []
+    for it in range(12):
+        out = engine(input_ids=ids, labels=labels)
+        loss = out.loss
+        engine.backward(loss)
+        optimizer.step()
+        losses.append(float(loss.detach()))
+    assert all(l == l for l in losses)  # finite
+    assert losses[-1] < losses[0] * 0.8, losses  # it learns the 8 fixed examples
+    steps = optimizer.state[next(engine.module.parameters())]["step"]
+    assert steps + optimizer.loss_scaler.skipped_steps == 12
+    sd = optimizer.state_dict()
+    assert len(sd["state"]) == len(list(engine.module.parameters())) and "loss_scaler" in sd

@@ -210,3 +210,17 @@ def test_dynamic_scaler_needs_a_gpu_for_anything_but_its_configuration():
     if not torch.cuda.is_available():
         with pytest.raises(RuntimeError, match="GPU"):
             s.update_scale(True)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
+
+
+def test_host_chunk_policy_is_for_directly_driven_chunk_lists():
+    client = ps.PatrickStarClient(0, 64, device="cpu", config={"host_chunk_policy": lambda pos: True})
+    with pytest.raises(NotImplementedError, match="register_model"):
+        client.register_model(torch.nn.Linear(4, 4))
