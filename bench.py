@@ -35,6 +35,8 @@ def parse_args():
     ap.add_argument("--chunks", type=int, default=24, help="chunk-list length (24 = the 1.5 B-parameter configuration)")
     ap.add_argument("--chunk-size", type=int, default=N_CHUNK)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-unfused-baseline", action="store_true",
+                    help="skip timing the reference's un-fused GPU branch (a sequence of torch element-wise kernels)")
     ap.add_argument("--cpu-reps", type=int, default=20)
     ap.add_argument("--host-chunks", type=int, default=0,
                     help="with --mode hybrid: how many of --chunks live in pinned host memory (the LAST ones)")
@@ -212,6 +214,49 @@ def run_hybrid(args):
     print(json.dumps(out))
 
 
+def unfused_gpu_branch(C, N, steps=3):
+    """The reference's GPU branch of one step, restated op for op with torch kernels on fresh buffers of the same
+    shape (patrickstar/ops/fp16_cpu_adam.py:245-277,430 per tensor -- here per chunk -- followed by the whole-chunk
+    fp32->fp16 copy_ of patrickstar/ops/chunk_io_buff.py:116-126).  A same-GPU baseline for the fused kernel, reported
+    beside it; not part of `value`."""
+    import math
+
+    import torch
+
+    dev = torch.device("cuda:0")
+    lr, b1, b2, eps, wd, scale, t = 1e-4, 0.9, 0.999, 1e-8, 0.01, 4096.0, 100
+    p = [torch.randn(N, device=dev) * 0.02 for _ in range(C)]
+    m = [torch.randn(N, device=dev) * 1e-4 for _ in range(C)]
+    v = [(torch.randn(N, device=dev) * 1e-6).abs_() for _ in range(C)]
+    h = [(torch.randn(N, device=dev) * 4).half() for _ in range(C)]
+
+    def one_step(step):
+        bc1, bc2 = 1 - b1**step, 1 - b2**step
+        for c in range(C):
+            g = h[c].float()
+            g.div_(scale)
+            p[c].mul_(1 - lr * wd)
+            m[c].mul_(b1).add_(g, alpha=1 - b1)
+            v[c].mul_(b2).addcmul_(g, g, value=1 - b2)
+            denom = (v[c].sqrt() / math.sqrt(bc2)).add_(eps)
+            p[c].addcdiv_(m[c], denom, value=-(lr / bc1))
+            h[c].copy_(p[c])
+
+    one_step(t)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(steps):
+        one_step(t + 1 + k)
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / steps
+    return {
+        "value": C * N / sec,
+        "unit": "params/s",
+        "ms_per_step": sec * 1e3,
+        "kind": "port of the reference's un-fused GPU branch (12 torch kernels per chunk), same GPU, same shapes",
+    }
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -318,6 +363,9 @@ def main():
     }
     del opt, client, params, grads
     torch.cuda.empty_cache()
+    if not args.no_unfused_baseline and args.mode == "static":
+        out["unfused_gpu_baseline"] = unfused_gpu_branch(C, N)
+        torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.cpu_reps)
     print(json.dumps(out))
