@@ -25,14 +25,6 @@ from .chunk_layout import (
     register_param,
 )
 
-_DTYPE_OF_LIST = {
-    ChunkType.PARAM_FP16: torch.half,
-    ChunkType.PARAM_FP32: torch.float,
-    ChunkType.MOMENTUM: torch.float,
-    ChunkType.VARIANCE: torch.float,
-}
-
-
 class ChunkPosition:
     """The four chunks that sit at the same place of the four lists."""
 
@@ -104,7 +96,7 @@ class PatrickStarClient:
             index.add_tensor(chunk_id, tensor_id, ref_info.start_offset, ref_info.numel, param, access_type)
         index.register_optimizer_state_chunk_id(ref_param, access_type, chunk_type, chunk_id)
 
-    def register_module_params(self, module, init_values=True):
+    def register_module_params(self, module):
         """Register the parameters a module owns directly as fp16 chunk tensors with fp32 shadows."""
         fp16_list, fp32_list = [], []
         for name, param in module.named_parameters(recurse=False):

@@ -142,8 +142,11 @@ class FP16Adam(torch.optim.Optimizer):
     def __del__(self):
         # the native object is per id and process-global: drop it with the optimizer
         if getattr(self, "_created", False):
-            self._lib.ps_adam_destroy(self.opt_id)
             self._created = False
+            try:
+                self._lib.ps_adam_destroy(self.opt_id)
+            except Exception:  # interpreter shutdown: the library handle may already be gone
+                pass
 
     def __setstate__(self, state):
         super().__setstate__(state)

@@ -3,7 +3,6 @@ product (FP16Adam over the C ABI) and mirrored on the CPU oracle."""
 import numpy as np
 import torch
 
-import oracle
 import patrickstar_amd as ps
 
 N_FULL = 64 * 1024 * 1024

@@ -4,7 +4,6 @@ Bar: fp32 param / exp_avg / exp_avg_sq and the fp16 param copy BIT-EXACT against
 oracle (the stated tolerance of 1e-6 relative / 1 fp16 ulp is met with zero slack),
 because the kernel performs the same IEEE binary32 operations in the same order.
 """
-import ctypes
 import math
 
 import numpy as np
@@ -14,7 +13,7 @@ import torch
 import oracle
 import patrickstar_amd as ps
 from patrickstar_amd import _lib
-from _harness import N_FULL, ChunkHarness, assert_bits_equal, bits
+from _harness import N_FULL, ChunkHarness, assert_bits_equal
 
 pytestmark = pytest.mark.gpu
 

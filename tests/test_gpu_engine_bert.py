@@ -4,7 +4,6 @@ import pytest
 import torch
 
 import patrickstar_amd as ps
-from patrickstar_amd.chunk_layout import AccessType, ChunkType
 
 pytestmark = pytest.mark.gpu
 

@@ -10,7 +10,7 @@ import torch
 import oracle
 import patrickstar_amd as ps
 from patrickstar_amd import _lib
-from _harness import N_FULL, ChunkHarness, assert_bits_equal
+from _harness import N_FULL, ChunkHarness
 
 pytestmark = pytest.mark.gpu
 
