@@ -15,7 +15,7 @@ from .chunk_layout import (  # noqa: F401
     is_param_registered,
     register_param,
 )
-from .client import PatrickStarClient  # noqa: F401
+from .client import PatrickStarClient, plan_host_positions  # noqa: F401
 from .engine import PatrickStarEngine, initialize_engine, parse_config  # noqa: F401
 from .fp16_adam import FP16Adam  # noqa: F401
 from .loss_scaler import DynamicLossScaler, LossScaler  # noqa: F401

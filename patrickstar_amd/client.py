@@ -34,6 +34,25 @@ class ChunkPosition:
         self.fp16, self.fp32, self.exp_avg, self.exp_avg_sq, self.on_host = fp16, fp32, exp_avg, exp_avg_sq, on_host
 
 
+def plan_host_positions(n_positions, chunk_size, free_bytes, staging_slots=2, margin_use_ratio=0.8):
+    """Which chunk positions to keep in pinned host memory when ``free_bytes`` of HBM are available.
+
+    The reference sizes its GPU share of the optimizer state from a memory margin measured during warm-up,
+    ``margin / (chunk_size * 12) * margin_use_ratio`` chunks (``patrickstar/core/memtracer/memtracer.py:190-214``),
+    and gives the FIRST chunks to the GPU (``patrickstar/ops/chunk_io_buff.py:234-239``).  Here a resident position
+    costs 14 B/element (fp16 + fp32 + m + v) and the streaming path needs ``staging_slots`` more positions' worth of
+    HBM; positions that do not fit go to the host, last positions first.  Returns a ``set`` of position indices,
+    usable as ``host_chunk_policy = planned.__contains__``.
+    """
+    per_position = 14 * chunk_size
+    budget = free_bytes * margin_use_ratio
+    if budget >= n_positions * per_position:
+        return set()
+    resident = int((budget - staging_slots * per_position) // per_position)
+    resident = max(0, min(n_positions, resident))
+    return set(range(resident, n_positions))
+
+
 class PatrickStarClient:
     def __init__(self, rank: int, default_chunk_size: int, config=None, device=None):
         self.local_rank = rank

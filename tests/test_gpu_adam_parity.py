@@ -385,3 +385,55 @@ def test_adam_update_mismatched_phases_fall_back_to_elementwise():
     assert_bits_equal(dp.cpu().numpy()[1:1 + n], po, "param")
     assert_bits_equal(dm.cpu().numpy()[2:2 + n], mo, "exp_avg")
     assert_bits_equal(dv.cpu().numpy()[:n], vo, "exp_avg_sq")
+
+
+def test_randomised_call_sequences_match_the_oracle_state_machine():
+    """Random hyper-parameters, step patterns (consecutive, repeated, jumping), beta changes, bias correction on/off,
+    weight-decay forms, scales (none, powers of two, arbitrary) and sizes: the operator's host state machine and the
+    kernels must track the oracle call for call, through both the flat-tensor and the chunk-list entry points."""
+    lib = _lib.load()
+    stream = _lib.current_stream_handle()
+    rng = np.random.default_rng(2024)
+    for trial in range(40):
+        adamw = bool(rng.integers(0, 2))
+        wd = float(rng.choice([0.0, 0.01, 0.3]))
+        lr = float(10 ** rng.uniform(-5, -1))
+        eps = float(10 ** rng.uniform(-10, -5))
+        betas = [float(rng.choice([0.9, 0.8, 0.0, 0.95])), float(rng.choice([0.999, 0.99, 0.5]))]
+        n = int(rng.choice([1, 63, 256, 257, 1000, 4096, 5000]))
+        use_chunks = bool(rng.integers(0, 2))
+        oid = 1000 + trial
+        lib.ps_adam_create(oid, lr, betas[0], betas[1], eps, wd, int(adamw), 0)
+        o = oracle.AdamOracle(lr, betas[0], betas[1], eps, wd, adamw)
+        p = rng.normal(0, 0.05, n).astype(np.float32)
+        m = rng.normal(0, 1e-3, n).astype(np.float32)
+        v = np.abs(rng.normal(0, 1e-5, n)).astype(np.float32)
+        dp, dm, dv = _dev(p.copy()), _dev(m.copy()), _dev(v.copy())
+        step = int(rng.choice([0, 0, 10, 1000]))
+        for call in range(5):
+            step = {0: step + 1, 1: step + 1, 2: step, 3: step + int(rng.integers(2, 50))}[int(rng.integers(0, 4))]
+            step = max(step, 1)
+            if rng.random() < 0.2:
+                betas[int(rng.integers(0, 2))] = float(rng.choice([0.85, 0.97, 0.9]))
+            if rng.random() < 0.3:
+                lr = float(10 ** rng.uniform(-5, -1))
+            scale = float(rng.choice([-1.0, 0.0, 1.0, 8.0, 2.0**16, 1000.0, 3.3]))
+            bias_correction = int(rng.random() < 0.8)
+            g = (rng.normal(0, 1e-2, n) * (scale if scale > 0 else 1.0)).astype(np.float16)
+            dg = _dev(g.copy())
+            if use_chunks:
+                table = _lib.chunk_array([[dp.data_ptr(), dm.data_ptr(), dv.data_ptr(), dg.data_ptr()]])
+                rc = lib.ps_adam_step_chunks(oid, step, lr, betas[0], betas[1], eps, wd, bias_correction, table, 1, n, scale, stream)
+            else:
+                rc = lib.ps_adam_update(oid, step, lr, betas[0], betas[1], eps, wd, bias_correction, dp.data_ptr(), dg.data_ptr(), 1,
+                                        dm.data_ptr(), dv.data_ptr(), n, scale, None, stream)
+            assert rc == 0
+            o.update(step, lr, betas[0], betas[1], eps, wd, bool(bias_correction), p, g, m, v, scale)
+            torch.cuda.synchronize()
+            what = f"trial {trial} call {call} (n={n}, step={step}, scale={scale}, chunks={use_chunks}, adamw={adamw}, wd={wd}, bc={bias_correction})"
+            assert_bits_equal(dp.cpu().numpy(), p, what + " param")
+            assert_bits_equal(dm.cpu().numpy(), m, what + " exp_avg")
+            assert_bits_equal(dv.cpu().numpy(), v, what + " exp_avg_sq")
+            if use_chunks:
+                assert_bits_equal(dg.cpu().numpy(), oracle.cast_fp32_to_fp16(p), what + " fp16 param")
+        lib.ps_adam_destroy(oid)

@@ -224,3 +224,19 @@ def test_host_chunk_policy_is_for_directly_driven_chunk_lists():
     client = ps.PatrickStarClient(0, 64, device="cpu", config={"host_chunk_policy": lambda pos: True})
     with pytest.raises(NotImplementedError, match="register_model"):
         client.register_model(torch.nn.Linear(4, 4))
+
+
+def test_plan_host_positions():
+    n = 64 * 1024 * 1024
+    per = 14 * n
+    # everything fits: nothing goes to the host
+    assert ps.plan_host_positions(24, n, free_bytes=288e9) == set()
+    # the 12 B-parameter shape on a 160 GB budget: the last positions are the ones that leave
+    planned = ps.plan_host_positions(180, n, free_bytes=160e9, staging_slots=2, margin_use_ratio=0.8)
+    resident = 180 - len(planned)
+    assert planned == set(range(resident, 180)) and 0 < resident < 180
+    assert (resident + 2) * per <= 160e9 * 0.8 < (resident + 3) * per
+    # nothing fits: all on the host
+    assert ps.plan_host_positions(5, n, free_bytes=1e9) == set(range(5))
+    policy = planned.__contains__
+    assert policy(179) and not policy(0)
