@@ -97,6 +97,7 @@ class FP16Adam(torch.optim.Optimizer):
         self._dynamic = isinstance(loss_scaler, DynamicLossScaler)
         self._host_overflow = False
         self._steps_dirty = False
+        self._host_step = None  # shared step counter of the host-decided path; taken from state[p]["step"] at first use
         self.staging_slots = 2  # HBM staging slots for host-resident chunks (double buffering)
 
         assert len(self.param_groups) == 1, "Only support one param group at the moment."
@@ -232,11 +233,19 @@ class FP16Adam(torch.optim.Optimizer):
                     return g(st, "lr"), g(st, "betas"), g(st, "eps"), g(st, "weight_decay")
         return None
 
+    def _first_step_entry(self):
+        for group in self.param_groups:
+            for p in group["params"]:
+                if p.requires_grad:
+                    return dict.__getitem__(self.state[p], "step")
+        return 0
+
     def _sync_steps(self):
+        """Write the shared step counter (device-resident or host-side) into every state[p]["step"]."""
         if not self._steps_dirty:
             return
         self._steps_dirty = False
-        step = self.loss_scaler.adam_step
+        step = self.loss_scaler.adam_step if self._dynamic else self._host_step
         for group in self.param_groups:
             for p in group["params"]:
                 if p.requires_grad:
@@ -276,13 +285,13 @@ class FP16Adam(torch.optim.Optimizer):
                 return loss
 
             # Static or absent scaler: the host knows every scalar (the static scaler never reports overflow).
-            step_no = None
-            for group in self.param_groups:
-                for p in group["params"]:
-                    if p.requires_grad:
-                        st = self.state[p]
-                        step_no = dict.__getitem__(st, "step") + 1
-                        dict.__setitem__(st, "step", step_no)
+            # every parameter's "step" advances together: one host counter, written back to the per-parameter
+            # entries only when somebody reads them
+            if self._host_step is None:
+                self._host_step = self._first_step_entry()
+            self._host_step += 1
+            self._steps_dirty = True
+            step_no = self._host_step
             loss_scale = self.loss_scaler.loss_scale if self.loss_scaler is not None else -1
             if host_positions:
                 self._streamer.step(self.opt_id, step_no, lr, beta1, beta2, eps, weight_decay, loss_scale, table, n_dev)
@@ -338,6 +347,7 @@ class FP16Adam(torch.optim.Optimizer):
                     dict.__setitem__(mine, k, saved[k])
                     if k == "step":
                         step_seen = saved[k]
+        self._host_step = step_seen
         if self._dynamic:
             self.loss_scaler.materialize(self.client.device)
             if step_seen is not None:
