@@ -240,3 +240,13 @@ def test_plan_host_positions():
     assert ps.plan_host_positions(5, n, free_bytes=1e9) == set(range(5))
     policy = planned.__contains__
     assert policy(179) and not policy(0)
+
+
+def test_product_never_touches_the_oracle():
+    """The oracle is test infrastructure: nothing under patrickstar_amd/ may import, load or name it."""
+    pkg = os.path.join(ROOT, "patrickstar_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.lower(), os.path.join(dirpath, f)
