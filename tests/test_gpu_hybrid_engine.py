@@ -155,3 +155,34 @@ def test_engine_end_to_end_against_oracle(loss_scale):
     w = engine.module.fc1.weight
     info = client.chunk_tensor_index.get_tensor_info(w.ps_attr.data_id())
     assert w.data_ptr() == cl[info.chunk_id].payload.data_ptr() + 2 * info.start_offset
+
+
+def test_hybrid_full_size_placement_invariance():
+    """At the real chunk size (64 Mi elements): where a chunk lives must not change a single bit.  The same seeded
+    state and gradients are stepped twice, once with every chunk in HBM and once with half of them in pinned host
+    memory; the oracle checks one resident and one host-resident chunk."""
+    from _harness import N_FULL
+
+    kw = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
+    host = [1, 2, 5]
+    a = HybridHarness(6, N_FULL, host, ps.LossScaler(2**12), seed=42, **kw)
+    b = HybridHarness(6, N_FULL, [], ps.LossScaler(2**12), seed=42, **kw)
+    for h in (a, b):
+        h.fill_state()
+        h.fill_grads(1e-3, 2**12)
+        for prm in h.params:
+            dict.__setitem__(h.opt.state[prm], "step", 99)
+    idx = [0, 5]
+    oc = a.oracle_chunks(idx)
+    oopt = oracle.OptimizerStepOracle(oc, oracle.StaticScalerOracle(2**12), **kw)
+    oopt.step_count = 99
+    for h in (a, b):
+        h.opt.step()
+    torch.cuda.synchronize()
+    oopt.step()
+    a.compare(oc, idx, what="hybrid full size vs oracle")
+    for i in range(6):
+        for x, y in zip(a.payloads(i), b.payloads(i)):
+            y = y.cpu() if x.device.type == "cpu" else y
+            assert torch.equal(x.view(torch.int16 if x.dtype == torch.half else torch.int32),
+                               y.view(torch.int16 if y.dtype == torch.half else torch.int32)), f"chunk {i}"
