@@ -90,6 +90,14 @@ def cpu_baseline(reps):
         cores = len(os.sched_getaffinity(0))
     except AttributeError:
         cores = os.cpu_count()
+    cpu_model = "unknown CPU"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                cpu_model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
     omp = os.environ.get("OMP_NUM_THREADS")
     if omp and omp.isdigit():
         cores = min(cores, int(omp))
@@ -100,7 +108,7 @@ def cpu_baseline(reps):
         "kind": "port",
         "sample": f"1 chunk of {n} elements (one-chunk CPU-path inputs, static scale 8), best of {reps} steps after 2 warm-up; "
         f"oracle code path {['', 'scalar', 'AVX2', 'AVX-512'][isa]}; 26 B/element -> {26 * n / best / 1e9:.0f} GB/s; "
-        f"scalar code path of the same oracle, 1 step: {n / scalar_s / 1e9:.2f} G params/s",
+        f"scalar code path of the same oracle, 1 step: {n / scalar_s / 1e9:.2f} G params/s; host CPU: {cpu_model}",
     }
 
 
