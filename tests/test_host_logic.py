@@ -250,3 +250,31 @@ def test_product_never_touches_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.lower(), os.path.join(dirpath, f)
+
+
+@pytest.mark.skipif(not os.path.exists(_lib.LIB_PATH), reason="HIP library not built")
+def test_argument_checks_happen_before_any_gpu_work():
+    """Bad arguments are rejected on the host with a code and a message (no GPU is needed to see that)."""
+    lib = _lib.load()
+    lib.ps_adam_create(88, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, 0)
+    fake = _lib.chunk_array([[16, 32, 48, 64]])  # never dereferenced: every call below fails validation first
+    bad_slot = _lib.chunk_array([[16, 0, 48, 64]])
+    E = _lib.PS_ERR_BAD_ARG
+    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, None, 2, 1.0, None, None) == E
+    assert b"staging" in lib.ps_last_error()
+    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, fake, 0, 1.0, None, None) == E
+    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, fake, 9, 1.0, None, None) == E
+    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, bad_slot, 1, 1.0, None, None) == E
+    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, bad_slot, 1, 1024, fake, 1, 1.0, None, None) == E
+    assert b"host chunk 0" in lib.ps_last_error()
+    assert lib.ps_adam_step_hybrid(4711, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, fake, 1, 1.0, None, None) == _lib.PS_ERR_UNKNOWN_ID
+    assert lib.ps_adam_step_chunks_gated(88, 1e-3, 1e-8, 0.0, 1, fake, 1, 1024, None, None) == E
+    assert lib.ps_overflow_scan_host_chunks(fake, 1, 1024, fake, 1, None, None) == E
+    assert lib.ps_overflow_scan(None, 10, None, None) == E
+    assert lib.ps_adam_set_grad_clamp(4711, 1.0) == _lib.PS_ERR_UNKNOWN_ID
+    assert lib.ps_adam_set_grad_clamp(88, 1.0) == 0
+    assert lib.ps_state_init(ctypes.c_void_p(16), 1.0, 1, 2.0, 1, 0, 1.0, 1, 1, 0, 0.9, 0.999, None) == E  # window 0
+    assert b"scale_window" in lib.ps_last_error()
+    assert lib.ps_scaler_update(ctypes.c_void_p(16), 3, None, 0, None) == E
+    assert lib.ps_state_seed_step(ctypes.c_void_p(16), -1, 0.9, 0.999, None) == E
+    lib.ps_adam_destroy(88)
