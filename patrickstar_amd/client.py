@@ -226,13 +226,15 @@ class PatrickStarClient:
                 for chunk in chunks:
                     chunk.allocate_payload(self.device)
                 continue
-            total = sum(c.capacity for c in chunks)
-            slab = torch.zeros(total, dtype=chunks[0].data_type, device=self.device)
+            # every payload starts on a 512-element boundary of its slab (>= 1 KiB for every dtype), so that odd
+            # chunk sizes do not push later chunks off the alignment the vector kernels want
+            stride = lambda c: -(-c.capacity // 512) * 512
+            slab = torch.zeros(sum(stride(c) for c in chunks), dtype=chunks[0].data_type, device=self.device)
             self._slabs.append(slab)
             cursor = 0
             for chunk in chunks:
                 chunk.payload = slab.narrow(0, cursor, chunk.capacity)
-                cursor += chunk.capacity
+                cursor += stride(chunk)
 
     def chunk_ids_generator(self, chunk_type):
         for cid in self.chunk_tensor_index.chunk_type_to_chunk_id_list_map.get(chunk_type, []):

@@ -437,3 +437,45 @@ def test_randomised_call_sequences_match_the_oracle_state_machine():
             if use_chunks:
                 assert_bits_equal(dg.cpu().numpy(), oracle.cast_fp32_to_fp16(p), what + " fp16 param")
         lib.ps_adam_destroy(oid)
+
+
+@pytest.mark.parametrize("offsets", [(1, 1, 1, 1), (0, 2, 0, 4), (3, 0, 1, 7), (0, 0, 0, 4)])
+def test_chunk_step_with_unaligned_payload_bases(offsets):
+    """Chunk payloads handed over at bases that are not 16-byte aligned (or aligned differently per list) take the
+    element-wise tile path and must produce the same bits."""
+    lib = _lib.load()
+    rng = np.random.default_rng(sum(offsets))
+    n, C = 256 * 5 + 19, 3
+    op, om, ov, oh = offsets
+    host = []
+    dev = []
+    rows = []
+    for c in range(C):
+        p = rng.normal(0, 0.02, n + 8).astype(np.float32)
+        m = rng.normal(0, 1e-4, n + 8).astype(np.float32)
+        v = np.abs(rng.normal(0, 1e-6, n + 8)).astype(np.float32)
+        g = (rng.normal(0, 1e-3, n + 8) * 16).astype(np.float16)
+        host.append((p, m, v, g))
+        d = tuple(_dev(x.copy()) for x in (p, m, v, g))
+        dev.append(d)
+        rows.append([d[0][op:].data_ptr(), d[1][om:].data_ptr(), d[2][ov:].data_ptr(), d[3][oh:].data_ptr()])
+    oid = 905
+    lib.ps_adam_create(oid, 1e-3, 0.9, 0.999, 1e-8, 0.01, 1, 0)
+    assert lib.ps_adam_step_chunks(oid, 3, 1e-3, 0.9, 0.999, 1e-8, 0.01, 1, _lib.chunk_array(rows), C, n, 16.0,
+                                   _lib.current_stream_handle()) == 0
+    torch.cuda.synchronize()
+    lib.ps_adam_destroy(oid)
+    o = oracle.AdamOracle(1e-3, 0.9, 0.999, 1e-8, 0.01, True)
+    o.advance(3, 0.9, 0.999)
+    o.set(1e-3, 1e-8, 0.01, True)
+    for (p, m, v, g), d in zip(host, dev):
+        po, mo, vo, go = p[op:op + n].copy(), m[om:om + n].copy(), v[ov:ov + n].copy(), g[oh:oh + n].copy()
+        assert oracle.lib().oracle_adam_span(o._buf, po.ctypes.data, go.ctypes.data, 1, mo.ctypes.data, vo.ctypes.data, n, 16.0, 0) > 0
+        assert_bits_equal(d[0].cpu().numpy()[op:op + n], po, "param")
+        assert_bits_equal(d[1].cpu().numpy()[om:om + n], mo, "exp_avg")
+        assert_bits_equal(d[2].cpu().numpy()[ov:ov + n], vo, "exp_avg_sq")
+        assert_bits_equal(d[3].cpu().numpy()[oh:oh + n], oracle.cast_fp32_to_fp16(po), "fp16 param")
+        # nothing outside the views was touched
+        assert_bits_equal(d[0].cpu().numpy()[:op], p[:op], "before")
+        assert_bits_equal(d[0].cpu().numpy()[op + n:], p[op + n:], "after")
+        assert_bits_equal(d[3].cpu().numpy()[oh + n:], g[oh + n:], "after fp16")
