@@ -45,6 +45,9 @@ def parse_args():
                     help="static: the 1.5 B-parameter configuration as specified (static loss scale, one fused kernel per step). "
                     "dynamic: same data with a DynamicLossScaler: inf/nan scan (2 B/element) + device-gated kernel + "
                     "scaler update per step, no host sync")
+    ap.add_argument("--arithmetic", choices=["operator", "torch"], default="operator",
+                    help="operator: the native operator's order of operations (default, the headline line); "
+                    "torch: the formula of the reference's GPU branch")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also launch one plain device-to-device copy of 1 Gi floats (4 GiB read, 4 GiB written) "
                     "so that a rocprofv3 --pmc run holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -293,7 +296,7 @@ def main():
     else:
         scaler = ps.DynamicLossScaler(init_scale=2**12, scale_factor=2, scale_window=1000, min_scale=1)
     opt = ps.FP16Adam(client, params, loss_scaler=scaler, lr=1e-4, betas=(0.9, 0.999), eps=1e-8,
-                      weight_decay=0.01, use_adamw=True)
+                      weight_decay=0.01, use_adamw=True, arithmetic=args.arithmetic)
     gen = torch.Generator(device=dev)
     gen.manual_seed(0)
     cl = client.chunk_list
@@ -357,9 +360,10 @@ def main():
             "AdamW lr 1e-4 betas (0.9,0.999) eps 1e-8 wd 0.01, static loss scale 2^12, fp16 grads -> fp32 p/m/v + fp16 params",
             "chunks": C,
             "chunk_numel": N,
-            "kernel": "adam_chunks_kernel<decoupled, exact-reciprocal unscale>" if args.mode == "static"
+            "kernel": f"adam_chunks_kernel<{args.arithmetic}, decoupled, reciprocal unscale>" if args.mode == "static"
             else "scan_chunks_kernel + adam_chunks_gated_kernel<decoupled> + scaler_update_kernel",
             "mode": args.mode,
+            "arithmetic": args.arithmetic,
         },
         "roofline": {
             "bound": "hbm",

@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define PS_ABI_VERSION 1
+#define PS_ABI_VERSION 2
 
 #define PS_ERR_BAD_ARG (-10001)     /* null pointer, negative count, unknown mode */
 #define PS_ERR_UNKNOWN_ID (-10002)  /* optimizer id was never created (the reference dereferences null here) */
@@ -65,7 +65,7 @@ typedef struct ps_chunk {
  * (fp16_cpu_adam.py:279-285) and the Adam step counter with its float
  * beta^t running products (cpu_adam.h:143-162).  It lives in device memory
  * so that "was there an overflow -> skip, restore, halve" needs no host
- * round trip.  128 bytes, 16-byte aligned.
+ * round trip.  160 bytes, 16-byte aligned.
  */
 typedef struct ps_step_state {
     double cur_scale;           /* loss_scale; Python float semantics (binary64) */
@@ -89,6 +89,12 @@ typedef struct ps_step_state {
     float beta1_t_next;         /* beta1^t for t = adam_step + 1 */
     float beta2_t_next;
     uint32_t reserved[4];
+    /* torch-formula arithmetic (PS_ARITH_TORCH): the Python floats behind the betas and the
+     * binary64 bias corrections 1 - beta ** t for t = adam_step + 1 (fp16_cpu_adam.py:412-413) */
+    double beta1_f64;
+    double beta2_f64;
+    double bias_correction1_next;
+    double bias_correction2_next;
 } ps_step_state;
 
 /* One entry of the optional per-iteration log written by ps_scaler_update. */
@@ -120,6 +126,26 @@ int ps_adam_create(int optimizer_id, float alpha, float beta1, float beta2, floa
  * reference clamps in Python before it calls the operator).  <= 0 switches it off (default). */
 int ps_adam_set_grad_clamp(int optimizer_id, double gradient_clipping);
 
+#define PS_ARITH_OPERATOR 0
+#define PS_ARITH_TORCH 1
+/* Which of the reference's two arithmetics the chunk-list entry points (ps_adam_step_chunks,
+ * _gated, _hybrid) apply to chunks that are updated in place in HBM.  FP16Adam picks by where a
+ * chunk's optimizer state lives (patrickstar/ops/fp16_cpu_adam.py:415-443):
+ *   PS_ARITH_OPERATOR (default)  the native operator's order of operations (cpu_adam.cpp:91-141)
+ *                                with its float step scalars (cpu_adam.h:143-175): what the
+ *                                reference runs for state held in host memory;
+ *   PS_ARITH_TORCH               FP16Adam.torch_adam_update (fp16_cpu_adam.py:245-277): what the
+ *                                reference runs for state held in GPU memory.  Each torch
+ *                                element-wise kernel it calls is restated with the rounding that
+ *                                torch's GPU kernels have: Python-double scalars narrowed to float
+ *                                at the kernel, `x / python_scalar` = x * (float)(1.0 / s),
+ *                                add(alpha) / addcmul / addcdiv as one fused multiply-add around
+ *                                the separately rounded product or quotient, bias corrections
+ *                                1 - beta ** t in binary64.
+ * Host-resident chunks streamed by ps_adam_step_hybrid always take the operator's arithmetic, as
+ * the reference updates those with the operator.  ps_adam_update is the operator itself. */
+int ps_adam_set_arithmetic(int optimizer_id, int arithmetic);
+
 /* destroy_adam (cpu_adam.cpp:744-749).  Unknown ids are ignored, as there. */
 int ps_adam_destroy(int optimizer_id);
 
@@ -143,18 +169,23 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
  * read fp16 grad, fp32 param, m, v once; write fp32 param, m, v and the fp16
  * param (over the grad) once: 28 bytes per element.  Host scalar state is
  * advanced ONCE for the call (the chunk list is one flat tensor for the
- * operator).  chunks is a host array of n_chunks descriptors. */
-int ps_adam_step_chunks(int optimizer_id, size_t step, float lr, float beta1, float beta2,
-                        float epsilon, float weight_decay, int bias_correction,
+ * operator).  chunks is a host array of n_chunks descriptors.
+ * Hyper-parameters and loss_scale are the Python numbers (binary64).  The operator's
+ * arithmetic narrows them to float first, as the pybind signature of adam_update does
+ * (cpu_adam.cpp:700-712); the torch arithmetic uses them as torch does.
+ * loss_scale <= 0: no unscale (no loss scaler). */
+int ps_adam_step_chunks(int optimizer_id, size_t step, double lr, double beta1, double beta2,
+                        double epsilon, double weight_decay, int bias_correction,
                         const ps_chunk* chunks, int n_chunks, size_t chunk_numel,
-                        float loss_scale, ps_stream_t stream);
+                        double loss_scale, ps_stream_t stream);
 
 /* Same pass, decided on the device: if d_state->overflow is set, every chunk's
  * fp16 payload is restored from the fp32 master copy (fp16_cpu_adam.py:298-309)
  * and nothing else changes; otherwise the Adam update runs with
- * loss_scale = (float)d_state->cur_scale and t = d_state->adam_step + 1
- * (beta^t from d_state).  Follow with ps_scaler_update(..., PS_FLAG_FROM_DEVICE). */
-int ps_adam_step_chunks_gated(int optimizer_id, float lr, float epsilon, float weight_decay,
+ * loss_scale = d_state->cur_scale and t = d_state->adam_step + 1 (beta^t, or
+ * the binary64 bias corrections of the torch arithmetic, from d_state).  Follow
+ * with ps_scaler_update(..., PS_FLAG_FROM_DEVICE). */
+int ps_adam_step_chunks_gated(int optimizer_id, double lr, double epsilon, double weight_decay,
                               int bias_correction, const ps_chunk* chunks, int n_chunks,
                               size_t chunk_numel, const ps_step_state* d_state,
                               ps_stream_t stream);
@@ -185,11 +216,11 @@ int ps_restore_fp16_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_nu
  * Work queued on `stream` before the call is waited for; work queued on it
  * afterwards waits for the last write-back.  The call itself never blocks.
  * Calls that overlap in time on one device share the side streams and race. */
-int ps_adam_step_hybrid(int optimizer_id, size_t step, float lr, float beta1, float beta2,
-                        float epsilon, float weight_decay, int bias_correction,
+int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, double beta2,
+                        double epsilon, double weight_decay, int bias_correction,
                         const ps_chunk* chunks, int n_chunks, const ps_chunk* host_chunks,
                         int n_host_chunks, size_t chunk_numel, const ps_chunk* staging, int n_slots,
-                        float loss_scale, const ps_step_state* d_state, ps_stream_t stream);
+                        double loss_scale, const ps_step_state* d_state, ps_stream_t stream);
 
 /* The inf/nan probe for host-resident chunks: only the fp16 payloads are
  * streamed (2 B/element) through staging[i].param_fp16. */
@@ -204,16 +235,18 @@ int ps_cast_fp32_to_fp16(const float* d_src, uint16_t* d_dst, size_t numel, ps_s
 
 /* Initialise *d_state (DynamicLossScaler.__init__, loss_scaler.py:107-125, plus
  * adam_step = 0, beta^t_next = beta).  *_is_int carry the Python types of the
- * three numbers so that loss_scale reads back as int or float like the reference. */
+ * three numbers so that loss_scale reads back as int or float like the reference.
+ * The betas are the Python floats; the operator's fields hold them narrowed. */
 int ps_state_init(ps_step_state* d_state, double init_scale, int init_is_int, double scale_factor,
                   int factor_is_int, int64_t scale_window, double min_scale, int min_is_int,
-                  int delayed_shift, int consecutive_hysteresis, float beta1, float beta2,
+                  int delayed_shift, int consecutive_hysteresis, double beta1, double beta2,
                   ps_stream_t stream);
 
 /* Set the Adam step counter (load_state_dict, fp16_cpu_adam.py:660-694) and
- * betas; beta^t for the next step is pow(beta, adam_step + 1) evaluated in
- * double on the host and narrowed, i.e. the reference's cold branch. */
-int ps_state_seed_step(ps_step_state* d_state, int64_t adam_step, float beta1, float beta2,
+ * betas; the operator's beta^t for the next step is pow((float)beta, adam_step + 1)
+ * evaluated in double on the host and narrowed, i.e. the reference's cold branch;
+ * the torch arithmetic's bias corrections are 1 - pow(beta, adam_step + 1). */
+int ps_state_seed_step(ps_step_state* d_state, int64_t adam_step, double beta1, double beta2,
                        ps_stream_t stream);
 
 /* Overwrite the loss-scaler fields only (restoring a checkpointed scaler). */
@@ -244,8 +277,9 @@ int ps_grad_to_chunk(const void* d_grad, int grad_is_half, uint16_t* d_slot_fp16
 #define PS_FLAG_FROM_DEVICE 2
 /* DynamicLossScaler.update_scale (loss_scaler.py:158-182) on the device.
  * flag_mode chooses the `overflow` argument: a host-given bool or the sticky
- * device flag.  A clean step also advances adam_step and beta^t (the float
- * running product of cpu_adam.h:158-159).  Clears the sticky flag.  If d_log
+ * device flag.  A clean step also advances adam_step, beta^t (the float
+ * running product of cpu_adam.h:158-159) and the binary64 bias corrections of
+ * the torch arithmetic.  Clears the sticky flag.  If d_log
  * is not NULL, entry [cur_iter % log_capacity] (cur_iter before the
  * increment) records the decision. */
 int ps_scaler_update(ps_step_state* d_state, int flag_mode, ps_scale_record* d_log,

@@ -9,6 +9,10 @@ Contents
 ``AdamOracle``            ctypes front-end of ``adam_oracle.c`` (the native operator,
                           ``patrickstar/ops/csrc/adam/cpu_adam.cpp:33-185,700-742`` and
                           ``csrc/includes/cpu_adam.h:143-175``).
+``torch_formula_update``  ``FP16Adam.torch_adam_update`` (``patrickstar/ops/fp16_cpu_adam.py:245-277``
+                          with the scalars of ``:412-413``), the branch the reference takes for
+                          optimizer state in GPU memory; scalars formed here in Python arithmetic as
+                          there, per-element rounding in ``adam_oracle.c: oracle_torch_adam_span``.
 ``cast_fp32_to_fp16``     whole-chunk RNE write-back (``patrickstar/ops/chunk_io_buff.py:116-126``).
 ``has_inf_or_nan``        ``patrickstar/fp16/loss_scaler.py:133-155``.
 ``ScalerOracle``          ``patrickstar/fp16/loss_scaler.py:107-182`` state machine.
@@ -24,6 +28,7 @@ and invariants).  The reference's own tests hold no golden vectors for this
 path; its loss-scale sequence is asserted nowhere in the reference.
 """
 import ctypes
+import math
 import os
 import subprocess
 
@@ -78,6 +83,8 @@ def lib():
         L.oracle_cast_f32_to_f16.restype = None
         L.oracle_any_nonfinite_f16.argtypes = [vp, sz]
         L.oracle_any_nonfinite_f16.restype = ci
+        L.oracle_torch_adam_span.argtypes = [vp, ci, ci, vp, vp, vp, vp, sz]
+        L.oracle_torch_adam_span.restype = None
         _lib = L
     return _lib
 
@@ -160,6 +167,51 @@ class AdamOracle:
         if took < 0:
             raise RuntimeError(f"oracle code path {isa} is not supported by this CPU")
         return took
+
+
+def torch_formula_update(params, grads_fp16, exp_avg, exp_avg_sq, step, lr, beta1, beta2, eps, weight_decay,
+                         use_adamw, loss_scale=None, gradient_clipping=-1):
+    """The reference's torch-formula branch on flat numpy arrays, in place.
+
+    Follows ``fp16_chunk_adam_ops`` / ``torch_adam_update`` statement by statement
+    (``patrickstar/ops/fp16_cpu_adam.py``): ``:364-379`` element-wise clamp of the fp16 gradient (GPU
+    branch), ``:412-413`` bias corrections in Python arithmetic, ``:430`` ``.float()``, ``:259-277`` the
+    update.  ``loss_scale`` is the Python number of the scaler (None: no scaler).  Every scalar is
+    computed here with Python floats exactly as the reference's Python does; narrowing to float32 is
+    what torch does where a kernel takes a Python scalar.
+    """
+    _check(params, np.float32)
+    _check(exp_avg, np.float32)
+    _check(exp_avg_sq, np.float32)
+    _check(grads_fp16, np.float16)
+    f32 = np.float32
+    bias_correction1 = 1 - beta1**step
+    bias_correction2 = 1 - beta2**step
+    step_size = lr / bias_correction1
+    k = np.zeros(10, dtype=np.float32)
+    if loss_scale is not None:
+        k[0] = f32(1.0 / loss_scale)
+    wd_mode = 0
+    if weight_decay != 0:
+        if use_adamw:
+            wd_mode, k[1] = 2, f32(1 - lr * weight_decay)
+        else:
+            wd_mode, k[1] = 1, f32(weight_decay)
+    k[2], k[3] = f32(beta1), f32(1 - beta1)
+    k[4], k[5] = f32(beta2), f32(1 - beta2)
+    k[6] = f32(1.0 / math.sqrt(bias_correction2))
+    k[7] = f32(eps)
+    k[8] = f32(-step_size)
+    if gradient_clipping > 0:
+        bound = gradient_clipping
+        if loss_scale is not None:
+            bound = bound * loss_scale
+        bound = min(65504.0, bound)
+        k[9] = f32(np.float16(f32(bound)))
+    lib().oracle_torch_adam_span(
+        _ptr(k), wd_mode, int(loss_scale is not None), _ptr(params), _ptr(grads_fp16), _ptr(exp_avg),
+        _ptr(exp_avg_sq), params.size,
+    )
 
 
 def cast_fp32_to_fp16(src):
@@ -288,7 +340,8 @@ class OptimizerStepOracle:
     """
 
     def __init__(self, chunks, loss_scaler=None, lr=1e-3, betas=(0.9, 0.999), eps=1e-8,
-                 weight_decay=0.0, use_adamw=False, isa=ISA_AUTO, gradient_clipping=-1):
+                 weight_decay=0.0, use_adamw=False, isa=ISA_AUTO, gradient_clipping=-1, arithmetic="operator",
+                 operator_chunks=()):
         self.chunks = chunks
         self.loss_scaler = loss_scaler
         self.lr, self.betas, self.eps, self.weight_decay = lr, betas, eps, weight_decay
@@ -297,6 +350,13 @@ class OptimizerStepOracle:
         self.has_overflow = False
         self.isa = isa
         self.gradient_clipping = gradient_clipping
+        # The reference picks per tensor by where its optimizer state lives (:415-443):
+        # "operator": every chunk through the native operator (state in host memory);
+        # "torch": chunks through torch_adam_update (state in GPU memory), except those listed
+        # in operator_chunks (indices of chunks whose state is in host memory).
+        assert arithmetic in ("operator", "torch")
+        self.arithmetic = arithmetic
+        self.operator_chunks = set(operator_chunks)
         self.native = AdamOracle(lr, betas[0], betas[1], eps, weight_decay, use_adamw)
 
     def check_overflow(self):
@@ -318,9 +378,14 @@ class OptimizerStepOracle:
             self.loss_scaler.update_scale(True)
             return True
         self.step_count += 1
-        scale = self.loss_scaler.loss_scale if self.loss_scaler is not None else -1
-        self.native.advance(self.step_count, self.betas[0], self.betas[1])
-        self.native.set(self.lr, self.eps, self.weight_decay, True)
+        scaler_scale = self.loss_scaler.loss_scale if self.loss_scaler is not None else None
+        via_torch = [
+            self.arithmetic == "torch" and i not in self.operator_chunks for i in range(len(self.chunks))
+        ]
+        if not all(via_torch):
+            # the native object is only touched when the operator runs at all
+            self.native.advance(self.step_count, self.betas[0], self.betas[1])
+            self.native.set(self.lr, self.eps, self.weight_decay, True)
         L = lib()
         if self.gradient_clipping > 0:
             # fp16_cpu_adam.py:364-379, GPU branch: clamp_ of the fp16 gradient tensor to
@@ -334,12 +399,18 @@ class OptimizerStepOracle:
                 g = c["p16"]
                 g[g < -b16] = -b16
                 g[g > b16] = b16
-        for c in self.chunks:
-            took = L.oracle_adam_span(
-                self.native._buf, _ptr(c["p32"]), _ptr(c["p16"]), 1, _ptr(c["m"]), _ptr(c["v"]),
-                c["p32"].size, float(scale), self.isa,
-            )
-            assert took > 0
+        for c, torch_branch in zip(self.chunks, via_torch):
+            if torch_branch:
+                torch_formula_update(
+                    c["p32"], c["p16"], c["m"], c["v"], self.step_count, self.lr, self.betas[0], self.betas[1],
+                    self.eps, self.weight_decay, self.use_adamw, scaler_scale,
+                )
+            else:
+                took = L.oracle_adam_span(
+                    self.native._buf, _ptr(c["p32"]), _ptr(c["p16"]), 1, _ptr(c["m"]), _ptr(c["v"]),
+                    c["p32"].size, float(scaler_scale if scaler_scale is not None else -1), self.isa,
+                )
+                assert took > 0
             c["p16"][...] = cast_fp32_to_fp16(c["p32"])
         if self.loss_scaler:
             self.loss_scaler.update_scale(False)

@@ -11,6 +11,7 @@
  *   patrickstar/ops/csrc/adam/cpu_adam.cpp:42-46       step_size / w_decay scalars
  *   patrickstar/ops/csrc/adam/cpu_adam.cpp:91-141      per-element op order (SIMD body)
  *   patrickstar/ops/chunk_io_buff.py:116-126,143-146   fp32 -> fp16 write-back (RNE cast)
+ *   patrickstar/ops/fp16_cpu_adam.py:245-277,430       the torch-formula (GPU) branch
  *
  * The per-element order is that of the reference's explicit-intrinsic body:
  * every product-sum the reference writes as SIMD_FMA is ONE fused rounding,
@@ -28,6 +29,14 @@
  *   oracle_adam_advance/set pinned: float32 running-product and pow() closed forms.
  *   oracle_f32_to_f16       pinned: numpy RNE cast over every binade incl. all
  *                           65536 fp16 values and their fp32 neighbours.
+ *   oracle_torch_adam_span  the reference's GPU branch delegates its arithmetic to PyTorch's
+ *                           element-wise kernels (third-party; torch is unpinned in the
+ *                           reference's requirements.txt:1); this restates each kernel of the call
+ *                           sequence at fp16_cpu_adam.py:259-277 as one rounding step.  Pinned:
+ *                           against that literal call sequence executed by torch itself, on CPU
+ *                           tensors in tests/test_oracle_torch_formula.py and bit for bit against
+ *                           torch's GPU kernels in tests/test_gpu_torch_arithmetic.py; against
+ *                           torch.optim.Adam/AdamW; against the textbook recurrences in float64.
  *   The reference ships no golden vectors for this path, and its C++ cannot be
  *   compiled in this image without CUDA headers, so no oracle/_ref build exists.
  *
@@ -361,3 +370,49 @@ int oracle_adam_update(oracle_adam* o, uint64_t step, float lr, float beta1, flo
 }
 
 int oracle_sizeof_state(void) { return (int)sizeof(oracle_adam); }
+
+/* ---- the torch-formula branch (FP16Adam.torch_adam_update) ------------------
+ *
+ * fp16_cpu_adam.py:430 and :259-277, one statement per torch kernel, each kernel one rounding
+ * step per element the way torch's GPU kernels compute it:
+ *   x.mul_(s), x.add_(s)                 separately rounded, the Python scalar narrowed to float
+ *   x.div_(s), x / s   (Python scalar)   x * (float)(1.0 / s): the reciprocal is formed in double
+ *   a.add_(b, alpha=s), a.add(b, alpha)  fmaf(b, s, a)
+ *   a.addcmul_(b, c, value=s)            fmaf(s, b * c, a)
+ *   a.addcdiv_(b, c, value=s)            fmaf(s, b / c, a)
+ *   sqrt                                 correctly rounded
+ * The caller (oracle/__init__.py: TorchFormulaOracle) forms the scalars in Python arithmetic
+ * exactly as the reference's Python does and narrows them:
+ *   k[0] (float)(1.0 / loss_scale)       grad.div_(loss_scale)             (if has_scale)
+ *   k[1] (float)(1 - lr * wd) | (float)wd  data.mul_(..) | grad.add(data, alpha=wd)
+ *   k[2] (float)beta1   k[3] (float)(1 - beta1)   k[4] (float)beta2   k[5] (float)(1 - beta2)
+ *   k[6] (float)(1.0 / math.sqrt(bias_correction2))   k[7] (float)eps
+ *   k[8] (float)(-(lr / bias_correction1))
+ *   k[9] clamp bound of the fp16 gradients (fp16_cpu_adam.py:375-379), 0 = off
+ * wd_mode: 0 none, 1 L2 (grad.add), 2 decoupled (data.mul_). */
+void oracle_torch_adam_span(const float k[10], int wd_mode, int has_scale, float* p,
+                            const uint16_t* g16, float* m, float* v, size_t n)
+{
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < n; ++i) {
+        float g = oracle_f16_to_f32(g16[i]); /* fp16_grad_tensor.float() */
+        if (k[9] > 0.0f) g = g < -k[9] ? -k[9] : (g > k[9] ? k[9] : g); /* clamp_ on the fp16 tensor */
+        float pp = p[i], mm = m[i], vv = v[i];
+        if (has_scale) g = g * k[0];
+        if (wd_mode == 2) pp = pp * k[1];
+        if (wd_mode == 1) g = fmaf(pp, k[1], g);
+        mm = mm * k[2];
+        mm = fmaf(g, k[3], mm);
+        vv = vv * k[4];
+        float gg = g * g;
+        vv = fmaf(k[5], gg, vv);
+        float d = sqrtf(vv);
+        d = d * k[6];
+        d = d + k[7];
+        float q = mm / d;
+        pp = fmaf(k[8], q, pp);
+        p[i] = pp;
+        m[i] = mm;
+        v[i] = vv;
+    }
+}

@@ -10,6 +10,8 @@ LIB_PATH = os.path.join(PKG_DIR, "libps_adam.so")
 
 PS_FLAG_FALSE, PS_FLAG_TRUE, PS_FLAG_FROM_DEVICE = 0, 1, 2
 PS_ERR_BAD_ARG, PS_ERR_UNKNOWN_ID, PS_ERR_NO_DEVICE = -10001, -10002, -10003
+PS_ARITH_OPERATOR, PS_ARITH_TORCH = 0, 1
+PS_ABI_VERSION = 2
 
 
 class ps_chunk(ctypes.Structure):
@@ -44,6 +46,10 @@ class ps_step_state(ctypes.Structure):
         ("beta1_t_next", ctypes.c_float),
         ("beta2_t_next", ctypes.c_float),
         ("reserved", ctypes.c_uint32 * 4),
+        ("beta1_f64", ctypes.c_double),
+        ("beta2_f64", ctypes.c_double),
+        ("bias_correction1_next", ctypes.c_double),
+        ("bias_correction2_next", ctypes.c_double),
     ]
 
 
@@ -56,7 +62,7 @@ class ps_scale_record(ctypes.Structure):
 
 
 assert ctypes.sizeof(ps_chunk) == 32
-assert ctypes.sizeof(ps_step_state) == 128
+assert ctypes.sizeof(ps_step_state) == 160
 assert ctypes.sizeof(ps_scale_record) == 16
 
 _f, _d, _i, _i64, _sz, _vp = (
@@ -74,16 +80,17 @@ SIGNATURES = {
     "ps_last_error": (ctypes.c_char_p, []),
     "ps_adam_create": (_i, [_i, _f, _f, _f, _f, _f, _i, _i]),
     "ps_adam_set_grad_clamp": (_i, [_i, _d]),
+    "ps_adam_set_arithmetic": (_i, [_i, _i]),
     "ps_adam_destroy": (_i, [_i]),
     "ps_adam_update": (_i, [_i, _sz, _f, _f, _f, _f, _f, _i, _vp, _vp, _i, _vp, _vp, _sz, _f, _vp, _vp]),
-    "ps_adam_step_chunks": (_i, [_i, _sz, _f, _f, _f, _f, _f, _i, _vp, _i, _sz, _f, _vp]),
-    "ps_adam_step_chunks_gated": (_i, [_i, _f, _f, _f, _i, _vp, _i, _sz, _vp, _vp]),
-    "ps_adam_step_hybrid": (_i, [_i, _sz, _f, _f, _f, _f, _f, _i, _vp, _i, _vp, _i, _sz, _vp, _i, _f, _vp, _vp]),
+    "ps_adam_step_chunks": (_i, [_i, _sz, _d, _d, _d, _d, _d, _i, _vp, _i, _sz, _d, _vp]),
+    "ps_adam_step_chunks_gated": (_i, [_i, _d, _d, _d, _i, _vp, _i, _sz, _vp, _vp]),
+    "ps_adam_step_hybrid": (_i, [_i, _sz, _d, _d, _d, _d, _d, _i, _vp, _i, _vp, _i, _sz, _vp, _i, _d, _vp, _vp]),
     "ps_overflow_scan_host_chunks": (_i, [_vp, _i, _sz, _vp, _i, _vp, _vp]),
     "ps_restore_fp16_chunks": (_i, [_vp, _i, _sz, _vp, _vp]),
     "ps_cast_fp32_to_fp16": (_i, [_vp, _vp, _sz, _vp]),
-    "ps_state_init": (_i, [_vp, _d, _i, _d, _i, _i64, _d, _i, _i, _i, _f, _f, _vp]),
-    "ps_state_seed_step": (_i, [_vp, _i64, _f, _f, _vp]),
+    "ps_state_init": (_i, [_vp, _d, _i, _d, _i, _i64, _d, _i, _i, _i, _d, _d, _vp]),
+    "ps_state_seed_step": (_i, [_vp, _i64, _d, _d, _vp]),
     "ps_state_set_scaler": (_i, [_vp, _d, _i, _i64, _i64, _i, _vp]),
     "ps_overflow_scan": (_i, [_vp, _sz, _vp, _vp]),
     "ps_overflow_scan_f32": (_i, [_vp, _sz, _vp, _vp]),
@@ -115,8 +122,10 @@ def load():
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
-    if lib.ps_abi_version() != 1:
-        raise HipLibraryMissing(f"{LIB_PATH} has ABI version {lib.ps_abi_version()}, expected 1; rebuild it")
+    if lib.ps_abi_version() != PS_ABI_VERSION:
+        raise HipLibraryMissing(
+            f"{LIB_PATH} has ABI version {lib.ps_abi_version()}, expected {PS_ABI_VERSION}; rebuild it"
+        )
     _lib = lib
     return lib
 

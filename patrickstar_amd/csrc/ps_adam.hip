@@ -99,6 +99,7 @@ struct HostAdam {
     size_t step = 0;
     bool adamw;
     double grad_clamp = -1.0;  // FP16Adam.gradient_clipping; <= 0: off
+    int arith = PS_ARITH_OPERATOR;  // arithmetic for chunks updated in place in HBM
 
     // cpu_adam.h:143-162
     void advance(size_t s, float b1, float b2)
@@ -241,7 +242,34 @@ __host__ __device__ inline void finish_consts(StepConsts& c, float lr, float bet
     }
 }
 
-template <int WD, int UNS>
+// The constants of FP16Adam.torch_adam_update (fp16_cpu_adam.py:245-277,412-413) as torch's GPU
+// kernels see them: every Python double is narrowed to float where a kernel takes it as a scalar;
+// `tensor / python_scalar` multiplies by the reciprocal formed in binary64 and then narrowed.
+// bc1, bc2 are the binary64 bias corrections 1 - beta ** step.
+__host__ __device__ inline void torch_consts(StepConsts& c, double lr, double beta1, double beta2,
+                                             double eps, double wd, bool adamw, double bc1,
+                                             double bc2, double loss_scale, float clip)
+{
+    c.clip = clip;
+    c.beta1 = (float)beta1;          // exp_avg.mul_(beta1)
+    c.beta2 = (float)beta2;          // exp_avg_sq.mul_(beta2)
+    c.b1m = (float)(1.0 - beta1);    // .add_(grad, alpha=1 - beta1)
+    c.b2m = (float)(1.0 - beta2);    // .addcmul_(grad, grad, value=1 - beta2)
+    c.bc2inv = (float)(1.0 / sqrt(bc2));  // exp_avg_sq.sqrt() / math.sqrt(bias_correction2)
+    c.eps = (float)eps;              // .add_(eps)
+    c.step_size = (float)(-(lr / bc1));   // addcdiv_(..., value=-step_size)
+    c.wd_mode = wd != 0.0 ? (adamw ? WD_DECOUPLED : WD_L2) : WD_NONE;
+    c.wd_term = adamw ? (float)(1.0 - lr * wd)  // data.mul_(1 - lr * weight_decay)
+                      : (float)wd;              // grad.add(data, alpha=weight_decay)
+    c.unscale = UNSCALE_NONE;
+    c.scale = 1.0f;
+    if (loss_scale > 0.0) {          // grad.div_(loss_scale)
+        c.unscale = UNSCALE_MUL;
+        c.scale = (float)(1.0 / loss_scale);
+    }
+}
+
+template <int ARITH, int WD, int UNS>
 __device__ __forceinline__ void adam_element(const StepConsts& c, float g, float& p, float& m,
                                              float& v)
 {
@@ -249,31 +277,48 @@ __device__ __forceinline__ void adam_element(const StepConsts& c, float g, float
     if (c.clip > 0.0f) g = g < -c.clip ? -c.clip : (g > c.clip ? c.clip : g);
     if (UNS == UNSCALE_DIV) g = g / c.scale;
     if (UNS == UNSCALE_MUL) g = g * c.scale;
-    if (WD == WD_L2) g = __builtin_fmaf(p, c.wd_term, g);
-    m = m * c.beta1;
-    m = __builtin_fmaf(g, c.b1m, m);
-    v = v * c.beta2;
-    float gg = g * g;
-    v = __builtin_fmaf(gg, c.b2m, v);
-    float d = __builtin_sqrtf(v);
-    d = __builtin_fmaf(d, c.bc2inv, c.eps);
-    float u = m / d;
-    if (WD == WD_DECOUPLED) p = __builtin_fmaf(p, c.wd_term, p);
-    p = __builtin_fmaf(u, c.step_size, p);
+    if (ARITH == PS_ARITH_OPERATOR) {
+        // Adam_Optimizer::Step, cpu_adam.cpp:91-141
+        if (WD == WD_L2) g = __builtin_fmaf(p, c.wd_term, g);
+        m = m * c.beta1;
+        m = __builtin_fmaf(g, c.b1m, m);
+        v = v * c.beta2;
+        float gg = g * g;
+        v = __builtin_fmaf(gg, c.b2m, v);
+        float d = __builtin_sqrtf(v);
+        d = __builtin_fmaf(d, c.bc2inv, c.eps);
+        float u = m / d;
+        if (WD == WD_DECOUPLED) p = __builtin_fmaf(p, c.wd_term, p);
+        p = __builtin_fmaf(u, c.step_size, p);
+    } else {
+        // FP16Adam.torch_adam_update, fp16_cpu_adam.py:259-277, one torch kernel per line
+        if (WD == WD_DECOUPLED) p = p * c.wd_term;             // data.mul_(1 - lr * wd)
+        if (WD == WD_L2) g = __builtin_fmaf(p, c.wd_term, g);  // grad.add(data, alpha=wd)
+        m = m * c.beta1;                                       // exp_avg.mul_(beta1)
+        m = __builtin_fmaf(g, c.b1m, m);                       //   .add_(grad, alpha=1 - beta1)
+        v = v * c.beta2;                                       // exp_avg_sq.mul_(beta2)
+        float gg = g * g;
+        v = __builtin_fmaf(c.b2m, gg, v);                      //   .addcmul_(grad, grad, value=1 - beta2)
+        float d = __builtin_sqrtf(v);                          // exp_avg_sq.sqrt()
+        d = d * c.bc2inv;                                      //   / math.sqrt(bias_correction2)
+        d = d + c.eps;                                         //   .add_(eps)
+        float q = m / d;
+        p = __builtin_fmaf(c.step_size, q, p);                 // data.addcdiv_(exp_avg, denom, value=-step_size)
+    }
 }
 
-template <int WD, int UNS>
+template <int ARITH, int WD, int UNS>
 __device__ __forceinline__ void element_any(const StepConsts& c, float g, float& p, float& m,
                                             float& v)
 {
     if (UNS != UNSCALE_RUNTIME)
-        adam_element<WD, UNS>(c, g, p, m, v);
+        adam_element<ARITH, WD, UNS>(c, g, p, m, v);
     else if (c.unscale == UNSCALE_MUL)
-        adam_element<WD, UNSCALE_MUL>(c, g, p, m, v);
+        adam_element<ARITH, WD, UNSCALE_MUL>(c, g, p, m, v);
     else if (c.unscale == UNSCALE_DIV)
-        adam_element<WD, UNSCALE_DIV>(c, g, p, m, v);
+        adam_element<ARITH, WD, UNSCALE_DIV>(c, g, p, m, v);
     else
-        adam_element<WD, UNSCALE_NONE>(c, g, p, m, v);
+        adam_element<ARITH, WD, UNSCALE_NONE>(c, g, p, m, v);
 }
 
 __device__ __forceinline__ float half_bits_to_float(uint32_t h)
@@ -394,7 +439,7 @@ struct LaneTile {
     HalfWords h[kUnroll];
 };
 
-template <int WD, int UNS>
+template <int ARITH, int WD, int UNS>
 __device__ __forceinline__ void lane_math(const StepConsts& c, LaneTile& r)
 {
 #pragma unroll
@@ -409,8 +454,8 @@ __device__ __forceinline__ void lane_math(const StepConsts& c, LaneTile& r)
                   v0 = r.v[u][e0 >> 2][e0 & 3];
             float p1 = r.p[u][e1 >> 2][e1 & 3], m1 = r.m[u][e1 >> 2][e1 & 3],
                   v1 = r.v[u][e1 >> 2][e1 & 3];
-            adam_element<WD, UNS>(c, g0, p0, m0, v0);
-            adam_element<WD, UNS>(c, g1, p1, m1, v1);
+            adam_element<ARITH, WD, UNS>(c, g0, p0, m0, v0);
+            adam_element<ARITH, WD, UNS>(c, g1, p1, m1, v1);
             r.p[u][e0 >> 2][e0 & 3] = p0;
             r.m[u][e0 >> 2][e0 & 3] = m0;
             r.v[u][e0 >> 2][e0 & 3] = v0;
@@ -426,7 +471,7 @@ __device__ __forceinline__ void lane_math(const StepConsts& c, LaneTile& r)
 // bases are 16-byte aligned.  All loads of the tile are issued before the
 // first use.  Loads and stores are written once, outside any branch on the
 // arithmetic variant.
-template <int WD, int UNS>
+template <int ARITH, int WD, int UNS>
 __device__ __forceinline__ void adam_tile_vec(const StepConsts& c, float* __restrict__ p32,
                                               float* __restrict__ m32, float* __restrict__ v32,
                                               uint16_t* __restrict__ h16, size_t base)
@@ -444,13 +489,13 @@ __device__ __forceinline__ void adam_tile_vec(const StepConsts& c, float* __rest
         for (int q = 0; q < kQuads; ++q) r.v[u][q] = ld_f4(v32 + i + 4 * q);
     }
     if (UNS != UNSCALE_RUNTIME) {
-        lane_math<WD, UNS>(c, r);
+        lane_math<ARITH, WD, UNS>(c, r);
     } else if (c.unscale == UNSCALE_MUL) {
-        lane_math<WD, UNSCALE_MUL>(c, r);
-    } else if (c.unscale == UNSCALE_DIV) {
-        lane_math<WD, UNSCALE_DIV>(c, r);
+        lane_math<ARITH, WD, UNSCALE_MUL>(c, r);
+    } else if (ARITH == PS_ARITH_OPERATOR && c.unscale == UNSCALE_DIV) {
+        lane_math<ARITH, WD, UNSCALE_DIV>(c, r);
     } else {
-        lane_math<WD, UNSCALE_NONE>(c, r);
+        lane_math<ARITH, WD, UNSCALE_NONE>(c, r);
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
@@ -466,14 +511,14 @@ __device__ __forceinline__ void adam_tile_vec(const StepConsts& c, float* __rest
 }
 
 // Same elements, one at a time: ragged tile ends and unaligned bases.
-template <int WD, int UNS>
+template <int ARITH, int WD, int UNS>
 __device__ __forceinline__ void adam_tile_scalar(const StepConsts& c, float* p32, float* m32,
                                                  float* v32, uint16_t* h16, size_t base, size_t end)
 {
     for (size_t i = base + threadIdx.x; i < end; i += kBlock) {
         float g = half_bits_to_float(h16[i]);
         float p = p32[i], m = m32[i], v = v32[i];
-        element_any<WD, UNS>(c, g, p, m, v);
+        element_any<ARITH, WD, UNS>(c, g, p, m, v);
         p32[i] = p;
         m32[i] = m;
         v32[i] = v;
@@ -487,17 +532,18 @@ __device__ __forceinline__ bool aligned16(const void* a, const void* b, const vo
     return (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)d) & 15u) == 0;
 }
 
-template <int WD, int UNS>
+template <int ARITH, int WD, int UNS>
 __device__ __forceinline__ void adam_tile(const StepConsts& c, const ps_chunk& ch, size_t base,
                                           size_t chunk_numel)
 {
     size_t end = base + kTile;
     if (end <= chunk_numel && aligned16(ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16)) {
-        adam_tile_vec<WD, UNS>(c, ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16, base);
+        adam_tile_vec<ARITH, WD, UNS>(c, ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16,
+                                      base);
     } else {
         if (end > chunk_numel) end = chunk_numel;
-        adam_tile_scalar<WD, UNS>(c, ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16, base,
-                                  end);
+        adam_tile_scalar<ARITH, WD, UNS>(c, ch.param_fp32, ch.exp_avg, ch.exp_avg_sq,
+                                         ch.param_fp16, base, end);
     }
 }
 
@@ -538,28 +584,30 @@ constexpr int kBatch = 64;
 struct ChunkBatch {
     ps_chunk c[kBatch];
 };
+static_assert(sizeof(ps_chunk) == 32 && sizeof(ps_step_state) == 160 && sizeof(ps_scale_record) == 16,
+              "layout of the boundary structs");
 
 // Host-decided step: all scalars arrive as kernel arguments and the
 // arithmetic variant is a compile-time property of the kernel.
-template <int WD, int UNS>
+template <int ARITH, int WD, int UNS>
 __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
     adam_chunks_kernel(ChunkBatch b, size_t chunk_numel, StepConsts c)
 {
-    adam_tile<WD, UNS>(c, b.c[blockIdx.y], (size_t)blockIdx.x * kTile, chunk_numel);
+    adam_tile<ARITH, WD, UNS>(c, b.c[blockIdx.y], (size_t)blockIdx.x * kTile, chunk_numel);
 }
 
 struct GatedArgs {
-    float lr, eps, wd;
+    double lr, eps, wd;  // the Python numbers; the operator's arithmetic narrows them to float
+    double grad_clamp;
     int adamw;
     int bias_correction;
-    double grad_clamp;
 };
 
 // Device-decided step: overflow flag, loss scale and beta^t come from the
 // device-resident state; a flagged step restores fp16 from fp32 instead.
 // The weight-decay form is known to the host; the unscale form depends on
 // the device-resident scale and is a uniform branch around the arithmetic.
-template <int WD>
+template <int ARITH, int WD>
 __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
     adam_chunks_gated_kernel(ChunkBatch b, size_t chunk_numel, GatedArgs ga,
                              const ps_step_state* __restrict__ st)
@@ -571,11 +619,19 @@ __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
         return;
     }
     StepConsts c;
-    // The operator takes loss_scale as a C float: the Python number narrows (RNE).
-    finish_consts(c, ga.lr, st->beta1, st->beta2, ga.eps, ga.wd, ga.adamw != 0, st->beta1_t_next,
-                  st->beta2_t_next, ga.bias_correction != 0, (float)st->cur_scale,
-                  clamp_bound(ga.grad_clamp, st->cur_scale));
-    adam_tile<WD, UNSCALE_RUNTIME>(c, ch, base, chunk_numel);
+    const float clip = clamp_bound(ga.grad_clamp, st->cur_scale);
+    if (ARITH == PS_ARITH_OPERATOR) {
+        // The operator takes its scalars and loss_scale as C floats: the Python numbers narrow (RNE).
+        finish_consts(c, (float)ga.lr, st->beta1, st->beta2, (float)ga.eps, (float)ga.wd,
+                      ga.adamw != 0, st->beta1_t_next, st->beta2_t_next, ga.bias_correction != 0,
+                      (float)st->cur_scale, clip);
+    } else {
+        const bool bc = ga.bias_correction != 0;
+        torch_consts(c, ga.lr, st->beta1_f64, st->beta2_f64, ga.eps, ga.wd, ga.adamw != 0,
+                     bc ? st->bias_correction1_next : 1.0, bc ? st->bias_correction2_next : 1.0,
+                     st->cur_scale, clip);
+    }
+    adam_tile<ARITH, WD, UNSCALE_RUNTIME>(c, ch, base, chunk_numel);
 }
 
 __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
@@ -612,7 +668,7 @@ __global__ void __launch_bounds__(kAuxBlock)
     for (size_t i = (size_t)blockIdx.x * kAuxBlock + threadIdx.x; i < numel; i += stride) {
         float g = GRAD_HALF ? half_bits_to_float(gh[i]) : gf[i];
         float p = p32[i], m = m32[i], v = v32[i];
-        element_any<WD, UNSCALE_RUNTIME>(c, g, p, m, v);
+        element_any<PS_ARITH_OPERATOR, WD, UNSCALE_RUNTIME>(c, g, p, m, v);
         p32[i] = p;
         m32[i] = m;
         v32[i] = v;
@@ -648,7 +704,7 @@ __global__ void __launch_bounds__(64)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             float pe = p[e], me = m[e], ve = v[e];
-            element_any<WD, UNSCALE_RUNTIME>(c, g[e], pe, me, ve);
+            element_any<PS_ARITH_OPERATOR, WD, UNSCALE_RUNTIME>(c, g[e], pe, me, ve);
             p[e] = pe;
             m[e] = me;
             v[e] = ve;
@@ -855,16 +911,51 @@ __global__ void state_init_kernel(ps_step_state* st, ps_step_state init)
     if (threadIdx.x == 0 && blockIdx.x == 0) *st = init;
 }
 
-__global__ void state_seed_kernel(ps_step_state* st, int64_t adam_step, float beta1, float beta2,
-                                  float b1t_next, float b2t_next)
+struct SeedArgs {
+    int64_t adam_step;
+    float beta1, beta2, b1t_next, b2t_next;
+    double beta1_f64, beta2_f64, bc1_next, bc2_next;
+};
+
+__global__ void state_seed_kernel(ps_step_state* st, SeedArgs a)
 {
     if (threadIdx.x == 0 && blockIdx.x == 0) {
-        st->adam_step = adam_step;
-        st->beta1 = beta1;
-        st->beta2 = beta2;
-        st->beta1_t_next = b1t_next;
-        st->beta2_t_next = b2t_next;
+        st->adam_step = a.adam_step;
+        st->beta1 = a.beta1;
+        st->beta2 = a.beta2;
+        st->beta1_t_next = a.b1t_next;
+        st->beta2_t_next = a.b2t_next;
+        st->beta1_f64 = a.beta1_f64;
+        st->beta2_f64 = a.beta2_f64;
+        st->bias_correction1_next = a.bc1_next;
+        st->bias_correction2_next = a.bc2_next;
     }
+}
+
+// beta ** n for a non-negative integer n in binary64, by squaring in double-double arithmetic: the
+// result is the correctly rounded power except within ~2^-90 of a rounding boundary, which is what
+// Python's float ** int (the C library's pow) returns for all but about one step in 10^4; the
+// float constants derived from 1 - beta ** n did not differ on any of 1.8 million (beta, n) pairs.
+struct TwoDouble {
+    double hi, lo;
+};
+__device__ inline TwoDouble two_double_mul(TwoDouble a, TwoDouble b)
+{
+    double p = a.hi * b.hi;
+    double e = __builtin_fma(a.hi, b.hi, -p);
+    e += a.hi * b.lo + a.lo * b.hi;
+    double s = p + e;
+    return TwoDouble{s, e - (s - p)};
+}
+__device__ inline double pow_int(double base, int64_t n)
+{
+    TwoDouble r{1.0, 0.0}, x{base, 0.0};
+    while (n > 0) {
+        if (n & 1) r = two_double_mul(r, x);
+        n >>= 1;
+        if (n) x = two_double_mul(x, x);
+    }
+    return r.hi;
 }
 
 __global__ void state_set_scaler_kernel(ps_step_state* st, double cur_scale, int scale_is_int,
@@ -915,6 +1006,9 @@ __global__ void scaler_update_kernel(ps_step_state* st, int flag_mode, ps_scale_
         s.adam_step += 1;
         s.beta1_t_next = s.beta1_t_next * s.beta1;
         s.beta2_t_next = s.beta2_t_next * s.beta2;
+        // fp16_cpu_adam.py:412-413 for the next step
+        s.bias_correction1_next = 1.0 - pow_int(s.beta1_f64, s.adam_step + 1);
+        s.bias_correction2_next = 1.0 - pow_int(s.beta2_f64, s.adam_step + 1);
     }
     if (log != nullptr && log_capacity > 0) {
         ps_scale_record r;
@@ -947,11 +1041,17 @@ struct ChunkList {
     size_t tiles_per_chunk;  // of kTile elements
 };
 
+// All descriptors are checked here, before anything is enqueued or any host state advances.
 int make_chunk_list(ChunkList& a, const ps_chunk* chunks, int n_chunks, size_t chunk_numel,
-                    size_t tile)
+                    size_t tile, bool fp16_only = false, const char* what = "chunk")
 {
     if (n_chunks < 0) return fail(PS_ERR_BAD_ARG, "n_chunks = %d is negative", n_chunks);
     if (chunks == nullptr && n_chunks > 0) return fail(PS_ERR_BAD_ARG, "chunks is NULL");
+    for (int i = 0; i < n_chunks; ++i) {
+        const ps_chunk& c = chunks[i];
+        if (!c.param_fp16 || (!fp16_only && (!c.param_fp32 || !c.exp_avg || !c.exp_avg_sq)))
+            return fail(PS_ERR_BAD_ARG, "%s %d has a NULL payload address", what, i);
+    }
     a.chunks = chunks;
     a.n_chunks = n_chunks;
     a.chunk_numel = chunk_numel;
@@ -970,53 +1070,117 @@ int for_each_batch(const ChunkList& a, F launch)
         int n = a.n_chunks - first < kBatch ? a.n_chunks - first : kBatch;
         ChunkBatch b;
         memset(&b, 0, sizeof(b));
-        for (int i = 0; i < n; ++i) {
-            const ps_chunk& c = a.chunks[first + i];
-            if (!c.param_fp32 || !c.exp_avg || !c.exp_avg_sq || !c.param_fp16)
-                return fail(PS_ERR_BAD_ARG, "chunk %d has a NULL payload address", first + i);
-            b.c[i] = c;
-        }
+        for (int i = 0; i < n; ++i) b.c[i] = a.chunks[first + i];
         launch(b, dim3((unsigned)a.tiles_per_chunk, (unsigned)n));
         PS_HIP(hipGetLastError());
     }
     return 0;
 }
 
-template <int WD>
+template <int ARITH, int WD>
 void launch_adam_batch_wd(const ChunkBatch& b, dim3 grid, size_t chunk_numel, const StepConsts& c,
                           hipStream_t s)
 {
     dim3 block(kBlock);
     if (c.unscale == UNSCALE_MUL)
-        hipLaunchKernelGGL((adam_chunks_kernel<WD, UNSCALE_MUL>), grid, block, kLdsBytes, s, b, chunk_numel, c);
-    else if (c.unscale == UNSCALE_DIV)
-        hipLaunchKernelGGL((adam_chunks_kernel<WD, UNSCALE_DIV>), grid, block, kLdsBytes, s, b, chunk_numel, c);
+        hipLaunchKernelGGL((adam_chunks_kernel<ARITH, WD, UNSCALE_MUL>), grid, block, kLdsBytes, s, b, chunk_numel, c);
+    else if (ARITH == PS_ARITH_OPERATOR && c.unscale == UNSCALE_DIV)  // the torch formula never divides
+        hipLaunchKernelGGL((adam_chunks_kernel<ARITH, WD, UNSCALE_DIV>), grid, block, kLdsBytes, s, b, chunk_numel, c);
     else
-        hipLaunchKernelGGL((adam_chunks_kernel<WD, UNSCALE_NONE>), grid, block, kLdsBytes, s, b, chunk_numel, c);
+        hipLaunchKernelGGL((adam_chunks_kernel<ARITH, WD, UNSCALE_NONE>), grid, block, kLdsBytes, s, b, chunk_numel, c);
 }
 
-void launch_adam_batch(const ChunkBatch& b, dim3 grid, size_t chunk_numel, const StepConsts& c,
-                       hipStream_t s)
+template <int ARITH>
+void launch_adam_batch_arith(const ChunkBatch& b, dim3 grid, size_t chunk_numel,
+                             const StepConsts& c, hipStream_t s)
 {
     if (c.wd_mode == WD_DECOUPLED)
-        launch_adam_batch_wd<WD_DECOUPLED>(b, grid, chunk_numel, c, s);
+        launch_adam_batch_wd<ARITH, WD_DECOUPLED>(b, grid, chunk_numel, c, s);
     else if (c.wd_mode == WD_L2)
-        launch_adam_batch_wd<WD_L2>(b, grid, chunk_numel, c, s);
+        launch_adam_batch_wd<ARITH, WD_L2>(b, grid, chunk_numel, c, s);
     else
-        launch_adam_batch_wd<WD_NONE>(b, grid, chunk_numel, c, s);
+        launch_adam_batch_wd<ARITH, WD_NONE>(b, grid, chunk_numel, c, s);
 }
 
-void launch_gated_batch(const ChunkBatch& b, dim3 grid, size_t chunk_numel, const GatedArgs& ga,
-                        const ps_step_state* d_state, hipStream_t s)
+// `c` must have been built for `arith` (finish_consts / torch_consts).
+void launch_adam_batch(int arith, const ChunkBatch& b, dim3 grid, size_t chunk_numel,
+                       const StepConsts& c, hipStream_t s)
+{
+    if (arith == PS_ARITH_TORCH)
+        launch_adam_batch_arith<PS_ARITH_TORCH>(b, grid, chunk_numel, c, s);
+    else
+        launch_adam_batch_arith<PS_ARITH_OPERATOR>(b, grid, chunk_numel, c, s);
+}
+
+template <int ARITH>
+void launch_gated_batch_arith(const ChunkBatch& b, dim3 grid, size_t chunk_numel,
+                              const GatedArgs& ga, const ps_step_state* d_state, hipStream_t s)
 {
     dim3 block(kBlock);
-    const bool decay = ga.wd > 0.0f;
+    // the operator tests its float weight decay "> 0" (cpu_adam.cpp:42), the torch formula "!= 0"
+    const bool decay = ARITH == PS_ARITH_OPERATOR ? (float)ga.wd > 0.0f : ga.wd != 0.0;
     if (decay && ga.adamw)
-        hipLaunchKernelGGL(adam_chunks_gated_kernel<WD_DECOUPLED>, grid, block, kLdsBytes, s, b, chunk_numel, ga, d_state);
+        hipLaunchKernelGGL((adam_chunks_gated_kernel<ARITH, WD_DECOUPLED>), grid, block, kLdsBytes, s, b, chunk_numel, ga, d_state);
     else if (decay)
-        hipLaunchKernelGGL(adam_chunks_gated_kernel<WD_L2>, grid, block, kLdsBytes, s, b, chunk_numel, ga, d_state);
+        hipLaunchKernelGGL((adam_chunks_gated_kernel<ARITH, WD_L2>), grid, block, kLdsBytes, s, b, chunk_numel, ga, d_state);
     else
-        hipLaunchKernelGGL(adam_chunks_gated_kernel<WD_NONE>, grid, block, kLdsBytes, s, b, chunk_numel, ga, d_state);
+        hipLaunchKernelGGL((adam_chunks_gated_kernel<ARITH, WD_NONE>), grid, block, kLdsBytes, s, b, chunk_numel, ga, d_state);
+}
+
+void launch_gated_batch(int arith, const ChunkBatch& b, dim3 grid, size_t chunk_numel,
+                        const GatedArgs& ga, const ps_step_state* d_state, hipStream_t s)
+{
+    if (arith == PS_ARITH_TORCH)
+        launch_gated_batch_arith<PS_ARITH_TORCH>(b, grid, chunk_numel, ga, d_state, s);
+    else
+        launch_gated_batch_arith<PS_ARITH_OPERATOR>(b, grid, chunk_numel, ga, d_state, s);
+}
+
+// The Python numbers of one step as they cross the boundary.
+struct HyperParams {
+    double lr, beta1, beta2, eps, wd;
+    double loss_scale;  // <= 0: no loss scaler
+    bool bias_correction;
+};
+
+// Host-decided step, operator arithmetic: narrow like the pybind signature of adam_update
+// (float arguments, cpu_adam.cpp:700-712), advance the operator's step scalars, derive the rest.
+StepConsts operator_step_consts(HostAdam& o, size_t step, const HyperParams& hp)
+{
+    o.advance(step, (float)hp.beta1, (float)hp.beta2);
+    o.set((float)hp.lr, (float)hp.eps, (float)hp.wd);
+    StepConsts c;
+    finish_consts(c, o.alpha, o.beta1, o.beta2, o.eps, o.weight_decay, o.adamw, o.beta1_t,
+                  o.beta2_t, hp.bias_correction, (float)hp.loss_scale,
+                  clamp_bound(o.grad_clamp, hp.loss_scale));
+    return c;
+}
+
+// Host-decided step, torch arithmetic (fp16_cpu_adam.py:412-413: Python's float ** int is the C
+// library's pow).  The operator object is not touched: the reference does not call it here.
+StepConsts torch_step_consts(const HostAdam& o, size_t step, const HyperParams& hp)
+{
+    double bc1 = 1.0, bc2 = 1.0;
+    if (hp.bias_correction) {
+        bc1 = 1.0 - std::pow(hp.beta1, (double)step);
+        bc2 = 1.0 - std::pow(hp.beta2, (double)step);
+    }
+    StepConsts c;
+    torch_consts(c, hp.lr, hp.beta1, hp.beta2, hp.eps, hp.wd, o.adamw, bc1, bc2, hp.loss_scale,
+                 clamp_bound(o.grad_clamp, hp.loss_scale));
+    return c;
+}
+
+GatedArgs gated_args(const HostAdam& o, double lr, double eps, double wd, int bias_correction)
+{
+    GatedArgs ga;
+    ga.lr = lr;
+    ga.eps = eps;
+    ga.wd = wd;
+    ga.grad_clamp = o.grad_clamp;
+    ga.adamw = o.adamw ? 1 : 0;
+    ga.bias_correction = bias_correction;
+    return ga;
 }
 
 // ------------------------------------------- host-resident chunks: streaming
@@ -1118,6 +1282,16 @@ int ps_adam_set_grad_clamp(int optimizer_id, double gradient_clipping)
     return 0;
 }
 
+int ps_adam_set_arithmetic(int optimizer_id, int arithmetic)
+{
+    auto o = find_opt(optimizer_id);
+    if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
+    if (arithmetic != PS_ARITH_OPERATOR && arithmetic != PS_ARITH_TORCH)
+        return fail(PS_ERR_BAD_ARG, "arithmetic = %d is neither PS_ARITH_OPERATOR nor PS_ARITH_TORCH", arithmetic);
+    o->arith = arithmetic;
+    return 0;
+}
+
 int ps_adam_destroy(int optimizer_id)
 {
     std::lock_guard<std::mutex> lock(g_registry_mutex);
@@ -1209,28 +1383,29 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
     return 0;
 }
 
-int ps_adam_step_chunks(int optimizer_id, size_t step, float lr, float beta1, float beta2,
-                        float epsilon, float weight_decay, int bias_correction,
+int ps_adam_step_chunks(int optimizer_id, size_t step, double lr, double beta1, double beta2,
+                        double epsilon, double weight_decay, int bias_correction,
                         const ps_chunk* chunks, int n_chunks, size_t chunk_numel,
-                        float loss_scale, ps_stream_t stream)
+                        double loss_scale, ps_stream_t stream)
 {
     auto o = find_opt(optimizer_id);
     if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
     ChunkList a;
     if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, kTile)) return rc;
-    o->advance(step, beta1, beta2);
-    o->set(lr, epsilon, weight_decay);
+    const HyperParams hp{lr, beta1, beta2, epsilon, weight_decay, loss_scale, bias_correction != 0};
     StepConsts c;
-    finish_consts(c, o->alpha, o->beta1, o->beta2, o->eps, o->weight_decay, o->adamw, o->beta1_t,
-                  o->beta2_t, bias_correction != 0, loss_scale,
-                  clamp_bound(o->grad_clamp, (double)loss_scale));
+    if (o->arith == PS_ARITH_TORCH)
+        c = torch_step_consts(*o, step, hp);
+    else
+        c = operator_step_consts(*o, step, hp);
+    const int arith = o->arith;
     hipStream_t s = static_cast<hipStream_t>(stream);
     return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid) {
-        launch_adam_batch(b, grid, chunk_numel, c, s);
+        launch_adam_batch(arith, b, grid, chunk_numel, c, s);
     });
 }
 
-int ps_adam_step_chunks_gated(int optimizer_id, float lr, float epsilon, float weight_decay,
+int ps_adam_step_chunks_gated(int optimizer_id, double lr, double epsilon, double weight_decay,
                               int bias_correction, const ps_chunk* chunks, int n_chunks,
                               size_t chunk_numel, const ps_step_state* d_state,
                               ps_stream_t stream)
@@ -1240,16 +1415,11 @@ int ps_adam_step_chunks_gated(int optimizer_id, float lr, float epsilon, float w
     if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
     ChunkList a;
     if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, kTile)) return rc;
-    GatedArgs ga;
-    ga.lr = lr;
-    ga.eps = epsilon;
-    ga.wd = weight_decay;
-    ga.adamw = o->adamw ? 1 : 0;
-    ga.bias_correction = bias_correction;
-    ga.grad_clamp = o->grad_clamp;
+    const GatedArgs ga = gated_args(*o, lr, epsilon, weight_decay, bias_correction);
+    const int arith = o->arith;
     hipStream_t s = static_cast<hipStream_t>(stream);
     return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid) {
-        launch_gated_batch(b, grid, chunk_numel, ga, d_state, s);
+        launch_gated_batch(arith, b, grid, chunk_numel, ga, d_state, s);
     });
 }
 
@@ -1275,40 +1445,29 @@ int ps_cast_fp32_to_fp16(const float* d_src, uint16_t* d_dst, size_t numel, ps_s
     return 0;
 }
 
-int ps_adam_step_hybrid(int optimizer_id, size_t step, float lr, float beta1, float beta2,
-                        float epsilon, float weight_decay, int bias_correction,
+int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, double beta2,
+                        double epsilon, double weight_decay, int bias_correction,
                         const ps_chunk* chunks, int n_chunks, const ps_chunk* host_chunks,
                         int n_host_chunks, size_t chunk_numel, const ps_chunk* staging, int n_slots,
-                        float loss_scale, const ps_step_state* d_state, ps_stream_t stream)
+                        double loss_scale, const ps_step_state* d_state, ps_stream_t stream)
 {
     auto o = find_opt(optimizer_id);
     if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
     ChunkList resident, host;
     if (int rc = make_chunk_list(resident, chunks, n_chunks, chunk_numel, kTile)) return rc;
-    if (int rc = make_chunk_list(host, host_chunks, n_host_chunks, chunk_numel, kTile)) return rc;
+    if (int rc = make_chunk_list(host, host_chunks, n_host_chunks, chunk_numel, kTile, false, "host chunk")) return rc;
     if (n_host_chunks > 0)
         if (int rc = check_slots(staging, n_slots, false)) return rc;
-    for (int i = 0; i < n_host_chunks; ++i) {
-        const ps_chunk& c = host_chunks[i];
-        if (!c.param_fp32 || !c.exp_avg || !c.exp_avg_sq || !c.param_fp16)
-            return fail(PS_ERR_BAD_ARG, "host chunk %d has a NULL payload address", i);
-    }
-    // one advance of the operator's step scalars for the whole list, resident and host alike
-    StepConsts c;
-    GatedArgs ga;
+    // Resident chunks take the optimizer's arithmetic, streamed host chunks the operator's (the
+    // reference updates those with the operator).  The operator's step scalars advance once for
+    // the whole list, and only if the operator's arithmetic is used at all.
+    const int arith = o->arith;
+    StepConsts c_resident, c_host;
+    const GatedArgs ga = gated_args(*o, lr, epsilon, weight_decay, bias_correction);
     if (d_state == nullptr) {
-        o->advance(step, beta1, beta2);
-        o->set(lr, epsilon, weight_decay);
-        finish_consts(c, o->alpha, o->beta1, o->beta2, o->eps, o->weight_decay, o->adamw,
-                      o->beta1_t, o->beta2_t, bias_correction != 0, loss_scale,
-                      clamp_bound(o->grad_clamp, (double)loss_scale));
-    } else {
-        ga.lr = lr;
-        ga.eps = epsilon;
-        ga.wd = weight_decay;
-        ga.adamw = o->adamw ? 1 : 0;
-        ga.bias_correction = bias_correction;
-        ga.grad_clamp = o->grad_clamp;
+        const HyperParams hp{lr, beta1, beta2, epsilon, weight_decay, loss_scale, bias_correction != 0};
+        if (arith == PS_ARITH_OPERATOR || n_host_chunks > 0) c_host = operator_step_consts(*o, step, hp);
+        c_resident = arith == PS_ARITH_TORCH ? torch_step_consts(*o, step, hp) : c_host;
     }
     hipStream_t caller = static_cast<hipStream_t>(stream);
     const bool stream_host = n_host_chunks > 0 && chunk_numel > 0;
@@ -1323,9 +1482,9 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, float lr, float beta1, fl
     }
     int rc = for_each_batch(resident, [&](const ChunkBatch& b, dim3 grid) {
         if (d_state == nullptr)
-            launch_adam_batch(b, grid, chunk_numel, c, caller);
+            launch_adam_batch(arith, b, grid, chunk_numel, c_resident, caller);
         else
-            launch_gated_batch(b, grid, chunk_numel, ga, d_state, caller);
+            launch_gated_batch(arith, b, grid, chunk_numel, ga, d_state, caller);
     });
     if (rc) return rc;
     if (!stream_host) return 0;
@@ -1350,9 +1509,9 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, float lr, float beta1, fl
         b.c[0] = d;
         dim3 grid((unsigned)host.tiles_per_chunk, 1);
         if (d_state == nullptr)
-            launch_adam_batch(b, grid, chunk_numel, c, p->compute);
+            launch_adam_batch(PS_ARITH_OPERATOR, b, grid, chunk_numel, c_host, p->compute);
         else
-            launch_gated_batch(b, grid, chunk_numel, ga, d_state, p->compute);
+            launch_gated_batch(PS_ARITH_OPERATOR, b, grid, chunk_numel, ga, d_state, p->compute);
         PS_HIP(hipGetLastError());
         PS_HIP(hipEventRecord(p->compute_done[s], p->compute));
 
@@ -1378,7 +1537,7 @@ int ps_overflow_scan_host_chunks(const ps_chunk* host_chunks, int n_chunks, size
 {
     if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
     ChunkList a;
-    if (int rc = make_chunk_list(a, host_chunks, n_chunks, chunk_numel, kScanTile)) return rc;
+    if (int rc = make_chunk_list(a, host_chunks, n_chunks, chunk_numel, kScanTile, true, "host chunk")) return rc;
     if (int rc = check_slots(staging, n_slots, true)) return rc;
     if (n_chunks == 0 || chunk_numel == 0) return 0;
     Pipeline* p = nullptr;
@@ -1392,8 +1551,6 @@ int ps_overflow_scan_host_chunks(const ps_chunk* host_chunks, int n_chunks, size
     for (int i = 0; i < kMaxSlots; ++i) p->slot_used[i] = false;
     for (int k = 0; k < n_chunks; ++k) {
         const int s = k % n_slots;
-        if (!host_chunks[k].param_fp16)
-            return fail(PS_ERR_BAD_ARG, "host chunk %d has a NULL fp16 payload address", k);
         if (p->slot_used[s]) PS_HIP(hipStreamWaitEvent(p->h2d, p->compute_done[s], 0));
         PS_HIP(hipMemcpyAsync(staging[s].param_fp16, host_chunks[k].param_fp16, b16,
                               hipMemcpyHostToDevice, p->h2d));
@@ -1412,7 +1569,7 @@ int ps_overflow_scan_host_chunks(const ps_chunk* host_chunks, int n_chunks, size
 
 int ps_state_init(ps_step_state* d_state, double init_scale, int init_is_int, double scale_factor,
                   int factor_is_int, int64_t scale_window, double min_scale, int min_is_int,
-                  int delayed_shift, int consecutive_hysteresis, float beta1, float beta2,
+                  int delayed_shift, int consecutive_hysteresis, double beta1, double beta2,
                   ps_stream_t stream)
 {
     if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
@@ -1432,33 +1589,44 @@ int ps_state_init(ps_step_state* d_state, double init_scale, int init_is_int, do
     s.delayed_shift = delayed_shift;
     s.cur_hysteresis = delayed_shift;
     s.consecutive_hysteresis = consecutive_hysteresis != 0;
-    s.beta1 = beta1;
-    s.beta2 = beta2;
+    s.beta1 = (float)beta1;
+    s.beta2 = (float)beta2;
     // Adam_Optimizer starts with beta^t = 1 and step 0; the first update multiplies once.
-    s.beta1_t_next = 1.0f * beta1;
-    s.beta2_t_next = 1.0f * beta2;
+    s.beta1_t_next = 1.0f * s.beta1;
+    s.beta2_t_next = 1.0f * s.beta2;
+    s.beta1_f64 = beta1;
+    s.beta2_f64 = beta2;
+    s.bias_correction1_next = 1.0 - std::pow(beta1, 1.0);
+    s.bias_correction2_next = 1.0 - std::pow(beta2, 1.0);
     hipLaunchKernelGGL(state_init_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
                        d_state, s);
     PS_HIP(hipGetLastError());
     return 0;
 }
 
-int ps_state_seed_step(ps_step_state* d_state, int64_t adam_step, float beta1, float beta2,
+int ps_state_seed_step(ps_step_state* d_state, int64_t adam_step, double beta1, double beta2,
                        ps_stream_t stream)
 {
     if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
     if (adam_step < 0) return fail(PS_ERR_BAD_ARG, "adam_step is negative");
-    float b1t, b2t;
+    SeedArgs a;
+    a.adam_step = adam_step;
+    a.beta1 = (float)beta1;
+    a.beta2 = (float)beta2;
     if (adam_step == 0) {
-        b1t = 1.0f * beta1;
-        b2t = 1.0f * beta2;
+        a.b1t_next = 1.0f * a.beta1;
+        a.b2t_next = 1.0f * a.beta2;
     } else {
         // a fresh native object that is first asked for step adam_step + 1 takes the pow branch
-        b1t = (float)std::pow((double)beta1, (double)(adam_step + 1));
-        b2t = (float)std::pow((double)beta2, (double)(adam_step + 1));
+        a.b1t_next = (float)std::pow((double)a.beta1, (double)(adam_step + 1));
+        a.b2t_next = (float)std::pow((double)a.beta2, (double)(adam_step + 1));
     }
+    a.beta1_f64 = beta1;
+    a.beta2_f64 = beta2;
+    a.bc1_next = 1.0 - std::pow(beta1, (double)(adam_step + 1));
+    a.bc2_next = 1.0 - std::pow(beta2, (double)(adam_step + 1));
     hipLaunchKernelGGL(state_seed_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
-                       d_state, adam_step, beta1, beta2, b1t, b2t);
+                       d_state, a);
     PS_HIP(hipGetLastError());
     return 0;
 }

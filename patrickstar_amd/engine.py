@@ -87,6 +87,8 @@ class PatrickStarEngine(torch.nn.Module):
             use_adamw=(optim_type == "AdamW"),
             use_hybrid_adam=optim_params["use_hybrid_adam"],
             scan_in_step=False,  # backward() probes while it copies the gradients
+            # optional key, absent from the reference's schema: "operator" (default) or "torch"
+            arithmetic=optim_params.get("arithmetic", "operator"),
         )
         self.client.init(self.module, self.optimizer)
         self.iteration_cnt_ = 0

@@ -13,6 +13,17 @@ the loss scale and the step counter live in a device struct, a flagged step
 restores the fp16 parameters from the fp32 master copy and halves the scale,
 and ``step()`` returns without synchronising.  ``state[p]["step"]`` and
 ``has_overflow`` read that struct back on demand.
+
+The reference has two arithmetics and picks per tensor by where the optimizer
+state lives (``fp16_cpu_adam.py:415-443``): the native operator for state in host
+memory, ``torch_adam_update`` (a sequence of torch kernels) for state in GPU
+memory.  They agree to about 1e-6 on the parameters and the first moment and
+to 5e-5 on the second moment (the operator forms ``1 - beta2`` in float).
+``arithmetic="operator"``
+(default) runs the operator's order of operations on every chunk;
+``arithmetic="torch"`` runs the torch formula, with the rounding of torch's GPU
+kernels, on chunks resident in HBM and keeps the operator's for host-resident
+chunks -- bit for bit what the reference computes under the same placement.
 """
 import weakref
 from copy import deepcopy
@@ -71,6 +82,7 @@ class FP16Adam(torch.optim.Optimizer):
         amsgrad=False,
         use_hybrid_adam=True,
         scan_in_step=True,
+        arithmetic="operator",
     ):
         if not 0.0 <= lr:
             raise ValueError("Invalid learning rate: {}".format(lr))
@@ -82,6 +94,8 @@ class FP16Adam(torch.optim.Optimizer):
             raise ValueError("Invalid beta parameter at index 1: {}".format(betas[1]))
         if not 0.0 <= weight_decay:
             raise ValueError("Invalid weight_decay value: {}".format(weight_decay))
+        if arithmetic not in ("operator", "torch"):
+            raise ValueError("Invalid arithmetic: {} (expected 'operator' or 'torch')".format(arithmetic))
         # fail now, not at the first step, if the HIP library was never built
         self._lib = _lib.load()
         defaults = dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay, amsgrad=amsgrad)
@@ -94,6 +108,7 @@ class FP16Adam(torch.optim.Optimizer):
         # True: step() itself probes every fp16 gradient chunk for inf/nan (one extra 2 B/element
         # pass).  False: the caller has already fed the flag through check_overflow().
         self.scan_in_step = scan_in_step
+        self.arithmetic = arithmetic
         self._dynamic = isinstance(loss_scaler, DynamicLossScaler)
         self._host_overflow = False
         self._steps_dirty = False
@@ -136,6 +151,8 @@ class FP16Adam(torch.optim.Optimizer):
         if gradient_clipping is not None and gradient_clipping > 0:
             # element-wise clamp of the fp16 gradients to +-min(65504, clipping * loss_scale), fused into the kernels
             _lib.check(self._lib.ps_adam_set_grad_clamp(self.opt_id, float(gradient_clipping)), "ps_adam_set_grad_clamp")
+        if arithmetic == "torch":
+            _lib.check(self._lib.ps_adam_set_arithmetic(self.opt_id, _lib.PS_ARITH_TORCH), "ps_adam_set_arithmetic")
         self._tables = None
         if self._dynamic and torch.cuda.is_available():
             self.loss_scaler.materialize(self.client.device, betas=betas)

@@ -7,41 +7,9 @@ import torch
 
 import oracle
 import patrickstar_amd as ps
-from _harness import ChunkHarness, assert_bits_equal
+from _harness import ChunkHarness, HybridHarness, assert_bits_equal
 
 pytestmark = pytest.mark.gpu
-
-
-class HybridHarness(ChunkHarness):
-    """Like ChunkHarness, with some positions kept in pinned host memory."""
-
-    def __init__(self, n_chunks, chunk_size, host_positions, loss_scaler=None, seed=0, **adam_kwargs):
-        self.device = torch.device("cuda:0")
-        self.n_chunks, self.chunk_size = n_chunks, chunk_size
-        host = set(host_positions)
-        self.client = ps.PatrickStarClient(0, chunk_size, config={"host_chunk_policy": lambda pos: pos in host})
-        self.params = self.client.append_flat_chunks(n_chunks)
-        self.opt = ps.FP16Adam(self.client, self.params, loss_scaler=loss_scaler, **adam_kwargs)
-        self.gen = torch.Generator(device=self.device)
-        self.gen.manual_seed(seed)
-        self.used = [p.ps_attr.numel for p in self.params]
-
-    def fill_state(self):
-        for i in range(self.n_chunks):
-            p, m, v, h = self.payloads(i)
-            n = self.chunk_size
-            p.copy_(torch.empty(n, device=self.device).normal_(0, 0.02, generator=self.gen))
-            m.copy_(torch.empty(n, device=self.device).normal_(0, 1e-4, generator=self.gen))
-            v.copy_(torch.empty(n, device=self.device).normal_(0, 1e-6, generator=self.gen).abs_())
-            h.copy_(p)
-        torch.cuda.synchronize()
-
-    def fill_grads(self, std, scale):
-        for i in range(self.n_chunks):
-            h = self.payloads(i)[3]
-            tmp = torch.empty(self.chunk_size, device=self.device).normal_(0, std, generator=self.gen).mul_(scale).half()
-            h.copy_(tmp)
-        torch.cuda.synchronize()
 
 
 @pytest.mark.parametrize("host_positions", [[1, 3, 4], [0, 1, 2, 3, 4], [4]])

@@ -161,6 +161,7 @@ def test_fp16adam_argument_checks():
         (dict(betas=(1.0, 0.999)), "Invalid beta parameter at index 0"),
         (dict(betas=(0.9, -0.1)), "Invalid beta parameter at index 1"),
         (dict(weight_decay=-0.1), "Invalid weight_decay value"),
+        (dict(arithmetic="fast"), "Invalid arithmetic"),
     ]:
         with pytest.raises(ValueError, match=msg):
             ps.FP16Adam(client, params, **kw)
@@ -184,14 +185,14 @@ def test_library_loads_and_exports_every_declared_symbol():
     lib = _lib.load()
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.ps_abi_version() == 1
+    assert lib.ps_abi_version() == 2
     # host-only entry points: registry and argument checks work without a GPU
     assert lib.ps_adam_create(77, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, 0) == 0
     assert lib.ps_adam_destroy(77) == 0
     assert lib.ps_scaler_update(None, 0, None, 0, None) == _lib.PS_ERR_BAD_ARG
     assert b"d_state" in lib.ps_last_error()
     assert lib.ps_state_init(None, 1.0, 1, 2.0, 1, 10, 1.0, 1, 1, 0, 0.9, 0.999, None) == _lib.PS_ERR_BAD_ARG
-    assert ctypes.sizeof(_lib.ps_step_state) == 128 and ctypes.sizeof(_lib.ps_chunk) == 32
+    assert ctypes.sizeof(_lib.ps_step_state) == 160 and ctypes.sizeof(_lib.ps_chunk) == 32
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
@@ -273,6 +274,13 @@ def test_argument_checks_happen_before_any_gpu_work():
     assert lib.ps_overflow_scan(None, 10, None, None) == E
     assert lib.ps_adam_set_grad_clamp(4711, 1.0) == _lib.PS_ERR_UNKNOWN_ID
     assert lib.ps_adam_set_grad_clamp(88, 1.0) == 0
+    assert lib.ps_adam_set_arithmetic(88, 7) == E
+    assert lib.ps_adam_set_arithmetic(88, _lib.PS_ARITH_TORCH) == 0
+    assert lib.ps_adam_set_arithmetic(88, _lib.PS_ARITH_OPERATOR) == 0
+    assert lib.ps_adam_set_arithmetic(4711, _lib.PS_ARITH_TORCH) == _lib.PS_ERR_UNKNOWN_ID
+    # descriptors are validated before the operator's step scalars advance or anything is enqueued
+    assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, bad_slot, 1, 1024, 1.0, None) == E
+    assert b"chunk 0 has a NULL payload" in lib.ps_last_error()
     assert lib.ps_state_init(ctypes.c_void_p(16), 1.0, 1, 2.0, 1, 0, 1.0, 1, 1, 0, 0.9, 0.999, None) == E  # window 0
     assert b"scale_window" in lib.ps_last_error()
     assert lib.ps_scaler_update(ctypes.c_void_p(16), 3, None, 0, None) == E
