@@ -35,7 +35,8 @@
  *                           sequence at fp16_cpu_adam.py:259-277 as one rounding step.  Pinned:
  *                           against that literal call sequence executed by torch itself, on CPU
  *                           tensors in tests/test_oracle_torch_formula.py and bit for bit against
- *                           torch's GPU kernels in tests/test_gpu_torch_arithmetic.py; against
+ *                           torch's GPU kernels in tests/test_gpu_torch_arithmetic.py and, on the CPU,
+ *                           against vectors those kernels wrote (tests/golden/torch_branch_vectors.npz); against
  *                           torch.optim.Adam/AdamW; against the textbook recurrences in float64.
  *   The reference ships no golden vectors for this path, and its C++ cannot be
  *   compiled in this image without CUDA headers, so no oracle/_ref build exists.

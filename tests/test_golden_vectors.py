@@ -103,3 +103,48 @@ def test_device_scaler_reproduces_golden_scale_trajectories():
             s.update_scale(f)
         for (flag, got), f, (want, typ) in zip(s.read_log(), t["flags"], t["scales"]):
             assert flag == f and got == want and ("int" if isinstance(got, int) else "float") == typ
+
+
+# ---- the torch-formula branch: vectors written by PyTorch's own GPU kernels (tests/golden/make_torch_branch_vectors.py)
+
+TVEC = np.load(os.path.join(HERE, "golden", "torch_branch_vectors.npz"))
+TCASES = [tuple(c) for c in json.loads(bytes(TVEC["meta"]).decode())["cases"]]
+
+
+@pytest.mark.parametrize("case", TCASES, ids=[c[0] for c in TCASES])
+def test_oracle_reproduces_torch_gpu_kernels_bitwise(case):
+    name, n, t0, steps, lr, b1, b2, eps, wd, adamw, scale, clip = case
+    p, m, v = (TVEC[f"{name}/{k}0"].copy() for k in "pmv")
+    for k in range(steps):
+        oracle.torch_formula_update(p, TVEC[f"{name}/g{k}"].copy(), m, v, t0 + k, lr, b1, b2, eps, wd, adamw, scale, clip)
+        assert _same(p, TVEC[f"{name}/p{k + 1}"]) and _same(m, TVEC[f"{name}/m{k + 1}"]) and _same(v, TVEC[f"{name}/v{k + 1}"])
+        assert _same(oracle.cast_fp32_to_fp16(p), TVEC[f"{name}/h{k + 1}"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", TCASES, ids=[c[0] for c in TCASES])
+def test_hip_torch_arithmetic_reproduces_torch_gpu_kernels_bitwise(case):
+    import torch
+
+    from patrickstar_amd import _lib
+
+    name, n, t0, steps, lr, b1, b2, eps, wd, adamw, scale, clip = case
+    lib = _lib.load()
+    dp, dm, dv = (torch.from_numpy(TVEC[f"{name}/{k}0"].copy()).cuda() for k in "pmv")
+    oid = 951
+    _lib.check(lib.ps_adam_create(oid, lr, b1, b2, eps, wd, int(adamw), 0), "create")
+    _lib.check(lib.ps_adam_set_arithmetic(oid, _lib.PS_ARITH_TORCH), "set_arithmetic")
+    if clip > 0:
+        _lib.check(lib.ps_adam_set_grad_clamp(oid, clip), "set_grad_clamp")
+    for k in range(steps):
+        h = torch.from_numpy(TVEC[f"{name}/g{k}"].copy()).cuda()  # gradients in, fp16 parameters out
+        rows = _lib.chunk_array([[dp.data_ptr(), dm.data_ptr(), dv.data_ptr(), h.data_ptr()]])
+        _lib.check(
+            lib.ps_adam_step_chunks(oid, t0 + k, lr, b1, b2, eps, wd, 1, rows, 1, n,
+                                    float(scale) if scale is not None else -1.0, _lib.current_stream_handle()),
+            "ps_adam_step_chunks",
+        )
+        torch.cuda.synchronize()
+        for got, key in ((dp, "p"), (dm, "m"), (dv, "v"), (h, "h")):
+            assert _same(got.cpu().numpy(), TVEC[f"{name}/{key}{k + 1}"]), (name, key, k)
+    lib.ps_adam_destroy(oid)
