@@ -41,6 +41,9 @@ def parse_args():
     ap.add_argument("--host-chunks", type=int, default=0,
                     help="with --mode hybrid: how many of --chunks live in pinned host memory (the LAST ones)")
     ap.add_argument("--slots", type=int, default=2, help="with --mode hybrid: HBM staging slots")
+    ap.add_argument("--host-fp16", choices=["host", "hbm"], default="host",
+                    help="with --mode hybrid: where a host-resident position keeps its fp16 payload (host: the whole "
+                    "position is streamed, 14 B/element each way; hbm: only fp32 param / m / v are, 12 B/element)")
     ap.add_argument("--mode", choices=["static", "dynamic", "hybrid"], default="static",
                     help="static: the 1.5 B-parameter configuration as specified (static loss scale, one fused kernel per step). "
                     "dynamic: same data with a DynamicLossScaler: inf/nan scan (2 B/element) + device-gated kernel + "
@@ -127,7 +130,11 @@ def run_hybrid(args):
     dev = torch.device("cuda:0")
     C, H, N = args.chunks, args.host_chunks, args.chunk_size
     first_host = C - H
-    client = ps.PatrickStarClient(0, N, config={"host_chunk_policy": lambda pos: pos >= first_host})
+    fp16_on_host = args.host_fp16 == "host"
+    link_per_element = 14 if fp16_on_host else 12
+    client = ps.PatrickStarClient(
+        0, N, config={"host_chunk_policy": lambda pos: pos >= first_host, "host_keeps_fp16": fp16_on_host}
+    )
     params = client.append_flat_chunks(C)
     opt = ps.FP16Adam(client, params, loss_scaler=ps.LossScaler(2**12), lr=1e-4, betas=(0.9, 0.999), eps=1e-8,
                       weight_decay=0.01, use_adamw=True)
@@ -171,14 +178,16 @@ def run_hybrid(args):
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1e-3
 
+    n_streamed = 4 if fp16_on_host else 3  # payloads of a host position that cross the link
+
     def h2d():
         for q in host_pos:
-            for dst, cid in zip(slot, (q.fp32, q.exp_avg, q.exp_avg_sq, q.fp16)):
+            for dst, cid in list(zip(slot, (q.fp32, q.exp_avg, q.exp_avg_sq, q.fp16)))[:n_streamed]:
                 dst.copy_(cl[cid].payload, non_blocking=True)
 
     def d2h():
         for q in host_pos:
-            for src, cid in zip(slot, (q.fp32, q.exp_avg, q.exp_avg_sq, q.fp16)):
+            for src, cid in list(zip(slot, (q.fp32, q.exp_avg, q.exp_avg_sq, q.fp16)))[:n_streamed]:
                 cl[cid].payload.copy_(src, non_blocking=True)
 
     lib = _lib.load()
@@ -200,7 +209,7 @@ def run_hybrid(args):
     lib.ps_adam_destroy(991)
     bound = max(t_h2d, t_d2h, t_kernel)
     elements = C * N
-    link_bytes = 14 * H * N
+    link_bytes = link_per_element * H * N
     out = {
         "metric": "Adam params/sec, chunk-list optimizer step with host-resident chunks streamed through HBM, 1 GPU",
         "value": elements / wall,
@@ -216,8 +225,9 @@ def run_hybrid(args):
         "data": "synthetic",
         "config": {
             "workload": f"hybrid placement: {C} chunks x {N} elements, {C - H} resident in HBM, {H} in pinned host memory "
-            f"streamed through {args.slots} HBM staging slots (14 B/element each way over the host link)",
-            "chunks": C, "host_chunks": H, "chunk_numel": N, "slots": args.slots,
+            f"streamed through {args.slots} HBM staging slots ({link_per_element} B/element each way over the host link; "
+            f"fp16 payloads of host positions in {'pinned host memory' if fp16_on_host else 'HBM'})",
+            "chunks": C, "host_chunks": H, "chunk_numel": N, "slots": args.slots, "host_fp16": args.host_fp16,
         },
         "hybrid": {
             "overlap_efficiency": bound / wall,

@@ -207,9 +207,14 @@ int ps_restore_fp16_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_nu
  * with n_slots >= 2 the copies of neighbouring chunks overlap the kernel.
  *   chunks       host array of descriptors of HBM-resident chunks (may be empty): updated
  *                by the same kernels on `stream`, concurrently with the first copies
- *   host_chunks  host array of descriptors whose addresses are PINNED HOST memory
+ *   host_chunks  host array of descriptors whose fp32 param / m / v addresses are PINNED HOST
+ *                memory.  param_fp16 is either pinned host memory too (streamed with the rest) or
+ *                a DEVICE address (the fp16 payload stays in HBM, where forward and backward use
+ *                it, as in the reference; it is then read and written in place and 12 instead of
+ *                14 B/element cross the link each way); the library asks the HIP runtime which
  *   staging      host array of n_slots (1..8) descriptors of DEVICE buffers of
- *                chunk_numel elements each, owned by the caller
+ *                chunk_numel elements each, owned by the caller; param_fp16 may be NULL when
+ *                every host chunk keeps its fp16 payload in HBM
  *   d_state      NULL: host-decided step with loss_scale, the operator's step scalars
  *                advanced ONCE for both lists; else device-gated exactly like
  *                ps_adam_step_chunks_gated (step, betas and loss_scale ignored)
@@ -223,7 +228,8 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, 
                         double loss_scale, const ps_step_state* d_state, ps_stream_t stream);
 
 /* The inf/nan probe for host-resident chunks: only the fp16 payloads are
- * streamed (2 B/element) through staging[i].param_fp16. */
+ * streamed (2 B/element) through staging[i].param_fp16; fp16 payloads that
+ * live in HBM are probed in place. */
 int ps_overflow_scan_host_chunks(const ps_chunk* host_chunks, int n_chunks, size_t chunk_numel,
                                  const ps_chunk* staging, int n_slots, ps_step_state* d_state,
                                  ps_stream_t stream);

@@ -34,21 +34,26 @@ class ChunkPosition:
         self.fp16, self.fp32, self.exp_avg, self.exp_avg_sq, self.on_host = fp16, fp32, exp_avg, exp_avg_sq, on_host
 
 
-def plan_host_positions(n_positions, chunk_size, free_bytes, staging_slots=2, margin_use_ratio=0.8):
+def plan_host_positions(n_positions, chunk_size, free_bytes, staging_slots=2, margin_use_ratio=0.8,
+                        host_keeps_fp16=True):
     """Which chunk positions to keep in pinned host memory when ``free_bytes`` of HBM are available.
 
     The reference sizes its GPU share of the optimizer state from a memory margin measured during warm-up,
     ``margin / (chunk_size * 12) * margin_use_ratio`` chunks (``patrickstar/core/memtracer/memtracer.py:190-214``),
     and gives the FIRST chunks to the GPU (``patrickstar/ops/chunk_io_buff.py:234-239``).  Here a resident position
     costs 14 B/element (fp16 + fp32 + m + v) and the streaming path needs ``staging_slots`` more positions' worth of
-    HBM; positions that do not fit go to the host, last positions first.  Returns a ``set`` of position indices,
-    usable as ``host_chunk_policy = planned.__contains__``.
+    HBM; positions that do not fit go to the host, last positions first.  With ``host_keeps_fp16=False`` a host
+    position still keeps its fp16 payload (2 B/element) in HBM and a staging slot holds 12 B/element.  Returns a
+    ``set`` of position indices, usable as ``host_chunk_policy = planned.__contains__``.
     """
     per_position = 14 * chunk_size
+    per_host_position = 0 if host_keeps_fp16 else 2 * chunk_size
+    per_slot = per_position - per_host_position
     budget = free_bytes * margin_use_ratio
     if budget >= n_positions * per_position:
         return set()
-    resident = int((budget - staging_slots * per_position) // per_position)
+    # resident * per_position + (n - resident) * per_host_position + slots * per_slot <= budget
+    resident = int((budget - staging_slots * per_slot - n_positions * per_host_position) // (per_position - per_host_position))
     resident = max(0, min(n_positions, resident))
     return set(range(resident, n_positions))
 
@@ -65,8 +70,11 @@ class PatrickStarClient:
         self.module = None
         self.optimizer = None
         self._param_idx = 0
-        # fp16 chunk ids kept in pinned host memory together with their fp32 / m / v chunks
+        # fp16 chunk ids of the positions whose fp32 / m / v chunks are kept in pinned host memory
         self.host_fp16_chunk_ids = set()
+        # True: such a position's fp16 payload is in pinned host memory as well (the whole position is streamed);
+        # False: it stays in HBM, where forward and backward use it (the only form a registered module can have)
+        self.host_keeps_fp16 = True
         self._slabs = []  # the allocations HBM-resident payloads are views of
         # called with (position index among fp16 chunks) -> True to keep that position in host memory
         self.host_chunk_policy: Optional[Callable[[int], bool]] = None
@@ -76,6 +84,7 @@ class PatrickStarClient:
             self.opt_config.update(config.get("opts", {}))
             if "host_chunk_policy" in config:
                 self.host_chunk_policy = config["host_chunk_policy"]
+            self.host_keeps_fp16 = bool(config.get("host_keeps_fp16", True))
 
     # -- building the lists -----------------------------------------------
     def append_chunk(self, data_type, chunk_type):
@@ -140,10 +149,9 @@ class PatrickStarClient:
         constructing before their parent does), copy the initial values into the fp16 and fp32
         payloads and re-point each parameter at its fp16 chunk slot."""
         self.module = model
-        if self.host_chunk_policy is not None:
-            # a module's parameters must be views of fp16 payloads in HBM; host-resident positions are for
-            # chunk lists that are driven directly (append_flat_chunks / explicit payload access)
-            raise NotImplementedError("host_chunk_policy cannot be combined with register_model")
+        # a module's parameters are views of the fp16 payloads, which forward and backward need in HBM:
+        # positions selected by the host-chunk policy keep only their optimizer state in host memory
+        self.host_keeps_fp16 = False
 
         def visit(m):
             for child in m.children():
@@ -217,7 +225,8 @@ class PatrickStarClient:
         for chunk_id, chunk in self.chunk_list.generate_chunk():
             if chunk.payload is not None:
                 continue
-            if self._fp16_chunk_of_position(chunk_id) in self.host_fp16_chunk_ids:
+            on_host = self._fp16_chunk_of_position(chunk_id) in self.host_fp16_chunk_ids
+            if on_host and (self.host_keeps_fp16 or chunk.chunk_type != ChunkType.PARAM_FP16):
                 chunk.allocate_payload("cpu", pin_memory=True)
             else:
                 pending.setdefault(chunk.chunk_type, []).append(chunk)

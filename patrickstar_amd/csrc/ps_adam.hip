@@ -1228,15 +1228,34 @@ int get_pipeline(Pipeline** out)
     return 0;
 }
 
-int check_slots(const ps_chunk* staging, int n_slots, bool fp16_only)
+int check_slots(const ps_chunk* staging, int n_slots, bool need_state, bool need_fp16)
 {
     if (n_slots < 1 || n_slots > kMaxSlots)
         return fail(PS_ERR_BAD_ARG, "n_slots = %d must be in 1..%d", n_slots, kMaxSlots);
     if (!staging) return fail(PS_ERR_BAD_ARG, "staging is NULL");
     for (int i = 0; i < n_slots; ++i) {
-        if (!staging[i].param_fp16 ||
-            (!fp16_only && (!staging[i].param_fp32 || !staging[i].exp_avg || !staging[i].exp_avg_sq)))
+        if ((need_fp16 && !staging[i].param_fp16) ||
+            (need_state && (!staging[i].param_fp32 || !staging[i].exp_avg || !staging[i].exp_avg_sq)))
             return fail(PS_ERR_BAD_ARG, "staging slot %d has a NULL buffer", i);
+    }
+    return 0;
+}
+
+// A host-resident chunk position may keep its fp16 payload in HBM (only the optimizer state lives in
+// host memory): say for every position whether its fp16 address is device memory.
+int fp16_payloads_in_hbm(const ps_chunk* host_chunks, int n, bool* in_hbm, bool* any_on_host)
+{
+    *any_on_host = false;
+    for (int i = 0; i < n; ++i) {
+        hipPointerAttribute_t attr;
+        hipError_t e = hipPointerGetAttributes(&attr, host_chunks[i].param_fp16);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(PS_ERR_BAD_ARG, "host chunk %d: the fp16 address is neither device nor pinned host memory (%s)",
+                        i, hipGetErrorString(e));
+        }
+        in_hbm[i] = attr.type == hipMemoryTypeDevice;
+        if (!in_hbm[i]) *any_on_host = true;
     }
     return 0;
 }
@@ -1456,8 +1475,14 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, 
     ChunkList resident, host;
     if (int rc = make_chunk_list(resident, chunks, n_chunks, chunk_numel, kTile)) return rc;
     if (int rc = make_chunk_list(host, host_chunks, n_host_chunks, chunk_numel, kTile, false, "host chunk")) return rc;
-    if (n_host_chunks > 0)
-        if (int rc = check_slots(staging, n_slots, false)) return rc;
+    std::unique_ptr<bool[]> fp16_in_hbm(new bool[n_host_chunks > 0 ? n_host_chunks : 1]);
+    if (n_host_chunks > 0) {
+        if (int rc = check_slots(staging, n_slots, true, false)) return rc;
+        bool any_on_host = false;
+        if (int rc = fp16_payloads_in_hbm(host_chunks, n_host_chunks, fp16_in_hbm.get(), &any_on_host)) return rc;
+        if (any_on_host)
+            if (int rc = check_slots(staging, n_slots, true, true)) return rc;
+    }
     // Resident chunks take the optimizer's arithmetic, streamed host chunks the operator's (the
     // reference updates those with the operator).  The operator's step scalars advance once for
     // the whole list, and only if the operator's arithmetic is used at all.
@@ -1494,10 +1519,15 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, 
     for (int k = 0; k < n_host_chunks; ++k) {
         const int s = k % n_slots;
         const ps_chunk& h = host_chunks[k];
-        const ps_chunk& d = staging[s];
+        ps_chunk d = staging[s];
+        // a fp16 payload that already lives in HBM is read and written in place: 12 instead of
+        // 14 bytes per element cross the link in each direction
+        const bool stage_fp16 = !fp16_in_hbm[k];
+        if (!stage_fp16) d.param_fp16 = h.param_fp16;
         // the slot is free once its previous occupant has been written back
         if (p->slot_used[s]) PS_HIP(hipStreamWaitEvent(p->h2d, p->d2h_done[s], 0));
-        PS_HIP(hipMemcpyAsync(d.param_fp16, h.param_fp16, b16, hipMemcpyHostToDevice, p->h2d));
+        if (stage_fp16)
+            PS_HIP(hipMemcpyAsync(d.param_fp16, h.param_fp16, b16, hipMemcpyHostToDevice, p->h2d));
         PS_HIP(hipMemcpyAsync(d.param_fp32, h.param_fp32, b32, hipMemcpyHostToDevice, p->h2d));
         PS_HIP(hipMemcpyAsync(d.exp_avg, h.exp_avg, b32, hipMemcpyHostToDevice, p->h2d));
         PS_HIP(hipMemcpyAsync(d.exp_avg_sq, h.exp_avg_sq, b32, hipMemcpyHostToDevice, p->h2d));
@@ -1518,7 +1548,8 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, 
         PS_HIP(hipStreamWaitEvent(p->d2h, p->compute_done[s], 0));
         // (on a device-skipped step fp32 param / m / v come back unchanged; copying them anyway
         // keeps the host free of any knowledge of the flag)
-        PS_HIP(hipMemcpyAsync(h.param_fp16, d.param_fp16, b16, hipMemcpyDeviceToHost, p->d2h));
+        if (stage_fp16)
+            PS_HIP(hipMemcpyAsync(h.param_fp16, d.param_fp16, b16, hipMemcpyDeviceToHost, p->d2h));
         PS_HIP(hipMemcpyAsync(h.param_fp32, d.param_fp32, b32, hipMemcpyDeviceToHost, p->d2h));
         PS_HIP(hipMemcpyAsync(h.exp_avg, d.exp_avg, b32, hipMemcpyDeviceToHost, p->d2h));
         PS_HIP(hipMemcpyAsync(h.exp_avg_sq, d.exp_avg_sq, b32, hipMemcpyDeviceToHost, p->d2h));
@@ -1538,19 +1569,32 @@ int ps_overflow_scan_host_chunks(const ps_chunk* host_chunks, int n_chunks, size
     if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
     ChunkList a;
     if (int rc = make_chunk_list(a, host_chunks, n_chunks, chunk_numel, kScanTile, true, "host chunk")) return rc;
-    if (int rc = check_slots(staging, n_slots, true)) return rc;
     if (n_chunks == 0 || chunk_numel == 0) return 0;
-    Pipeline* p = nullptr;
-    if (int rc = get_pipeline(&p)) return rc;
+    std::unique_ptr<bool[]> fp16_in_hbm(new bool[n_chunks]);
+    bool any_on_host = false;
+    if (int rc = fp16_payloads_in_hbm(host_chunks, n_chunks, fp16_in_hbm.get(), &any_on_host)) return rc;
     hipStream_t caller = static_cast<hipStream_t>(stream);
     const size_t b16 = chunk_numel * sizeof(uint16_t);
     const size_t n_tiles = a.tiles_per_chunk;
+    // fp16 payloads that live in HBM are probed in place on the caller's stream
+    for (int k = 0; k < n_chunks; ++k) {
+        if (!fp16_in_hbm[k]) continue;
+        hipLaunchKernelGGL(scan_f16_kernel, dim3(grid_1d(n_tiles)), dim3(kAuxBlock), 0, caller,
+                           host_chunks[k].param_fp16, chunk_numel, n_tiles, d_state);
+        PS_HIP(hipGetLastError());
+    }
+    if (!any_on_host) return 0;
+    if (int rc = check_slots(staging, n_slots, false, true)) return rc;
+    Pipeline* p = nullptr;
+    if (int rc = get_pipeline(&p)) return rc;
     PS_HIP(hipEventRecord(p->entry, caller));
     PS_HIP(hipStreamWaitEvent(p->h2d, p->entry, 0));
     PS_HIP(hipStreamWaitEvent(p->compute, p->entry, 0));
     for (int i = 0; i < kMaxSlots; ++i) p->slot_used[i] = false;
+    int streamed = 0;
     for (int k = 0; k < n_chunks; ++k) {
-        const int s = k % n_slots;
+        if (fp16_in_hbm[k]) continue;
+        const int s = streamed++ % n_slots;
         if (p->slot_used[s]) PS_HIP(hipStreamWaitEvent(p->h2d, p->compute_done[s], 0));
         PS_HIP(hipMemcpyAsync(staging[s].param_fp16, host_chunks[k].param_fp16, b16,
                               hipMemcpyHostToDevice, p->h2d));

@@ -6,7 +6,9 @@ updates them with the CPU operator (``patrickstar/ops/fp16_cpu_adam.py:415-428``
 copied into double-buffered HBM staging by ``hipMemcpyAsync`` on side streams,
 updated by the same fused kernel as resident chunks, and copied back, all ordered
 by events inside ``ps_adam_step_hybrid``; the Python side only owns the
-staging buffers.
+staging buffers.  A position's fp16 payload may stay in HBM (where forward and
+backward use it, as in the reference); it is then updated in place and only the
+optimizer state (12 B/element each way) crosses the link.
 """
 import torch
 
@@ -20,11 +22,17 @@ class HostChunkStreamer:
         self.chunk_numel = client.default_chunk_size
         cl = client.chunk_list
         rows = []
+        stage_fp16 = False  # does any position keep its fp16 payload in host memory?
         for pos in host_positions:
             payloads = [cl[c].payload for c in (pos.fp32, pos.exp_avg, pos.exp_avg_sq, pos.fp16)]
-            for t in payloads:
+            for t in payloads[:3]:
                 if t.device.type != "cpu" or not t.is_pinned():
-                    raise RuntimeError("host-resident chunk payloads must be pinned host memory")
+                    raise RuntimeError("host-resident optimizer state must be pinned host memory")
+            p16 = payloads[3]
+            if p16.device.type == "cpu":
+                if not p16.is_pinned():
+                    raise RuntimeError("a host-resident fp16 payload must be pinned host memory")
+                stage_fp16 = True
             rows.append([t.data_ptr() for t in payloads])
         self.host_table = _lib.chunk_array(rows)
         self.n_host = len(rows)
@@ -37,11 +45,13 @@ class HostChunkStreamer:
                 torch.empty(n, dtype=torch.float, device=dev),
                 torch.empty(n, dtype=torch.float, device=dev),
                 torch.empty(n, dtype=torch.float, device=dev),
-                torch.empty(n, dtype=torch.half, device=dev),
+                torch.empty(n if stage_fp16 else 0, dtype=torch.half, device=dev),
             )
             for _ in range(n_slots)
         ]
-        self.staging = _lib.chunk_array([[t.data_ptr() for t in slot] for slot in self._slots])
+        self.staging = _lib.chunk_array(
+            [[t.data_ptr() if t.numel() else None for t in slot] for slot in self._slots]
+        )
         self._lib = _lib.load()
 
     def step(self, opt_id, step_no, lr, beta1, beta2, eps, weight_decay, loss_scale, resident, n_resident, scaler=None):

@@ -84,11 +84,14 @@ class ChunkHarness:
 class HybridHarness(ChunkHarness):
     """Like ChunkHarness, with some positions kept in pinned host memory."""
 
-    def __init__(self, n_chunks, chunk_size, host_positions, loss_scaler=None, seed=0, **adam_kwargs):
+    def __init__(self, n_chunks, chunk_size, host_positions, loss_scaler=None, seed=0, host_keeps_fp16=True,
+                 **adam_kwargs):
         self.device = torch.device("cuda:0")
         self.n_chunks, self.chunk_size = n_chunks, chunk_size
         host = set(host_positions)
-        self.client = ps.PatrickStarClient(0, chunk_size, config={"host_chunk_policy": lambda pos: pos in host})
+        self.client = ps.PatrickStarClient(
+            0, chunk_size, config={"host_chunk_policy": lambda pos: pos in host, "host_keeps_fp16": host_keeps_fp16}
+        )
         self.params = self.client.append_flat_chunks(n_chunks)
         self.opt = ps.FP16Adam(self.client, self.params, loss_scaler=loss_scaler, **adam_kwargs)
         self.gen = torch.Generator(device=self.device)

@@ -12,15 +12,19 @@ from _harness import ChunkHarness, HybridHarness, assert_bits_equal
 pytestmark = pytest.mark.gpu
 
 
+@pytest.mark.parametrize("host_keeps_fp16", [True, False])
 @pytest.mark.parametrize("host_positions", [[1, 3, 4], [0, 1, 2, 3, 4], [4]])
 @pytest.mark.parametrize("chunk_size", [2048 * 3, 2048 + 77])
-def test_hybrid_static_bit_exact(host_positions, chunk_size):
+def test_hybrid_static_bit_exact(host_positions, chunk_size, host_keeps_fp16):
     h = HybridHarness(5, chunk_size, host_positions, ps.LossScaler(2**12), seed=chunk_size + len(host_positions),
+                      host_keeps_fp16=host_keeps_fp16,
                       lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
     for i in range(5):
         on_host = h.payloads(i)[0].device.type == "cpu"
         assert on_host == (i in host_positions)
-        assert (not on_host) or all(t.is_pinned() for t in h.payloads(i))
+        assert (not on_host) or all(t.is_pinned() for t in h.payloads(i)[:3])
+        # the fp16 payload follows the state to the host only when asked to
+        assert (h.payloads(i)[3].device.type == "cpu") == (on_host and host_keeps_fp16)
     h.fill_state()
     oc = h.oracle_chunks()
     oopt = oracle.OptimizerStepOracle(oc, oracle.StaticScalerOracle(2**12), lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
@@ -34,10 +38,11 @@ def test_hybrid_static_bit_exact(host_positions, chunk_size):
         h.compare(oc, what=f"hybrid step {step}")
 
 
-def test_hybrid_dynamic_skips_and_restores_host_chunks_too():
+@pytest.mark.parametrize("host_keeps_fp16", [True, False])
+def test_hybrid_dynamic_skips_and_restores_host_chunks_too(host_keeps_fp16):
     kw = dict(init_scale=2**10, scale_factor=2, scale_window=3, min_scale=1)
     scaler = ps.DynamicLossScaler(**kw)
-    h = HybridHarness(4, 2048 * 2 + 9, [1, 2], scaler, seed=12, lr=1e-3, weight_decay=0.01)
+    h = HybridHarness(4, 2048 * 2 + 9, [1, 2], scaler, seed=12, host_keeps_fp16=host_keeps_fp16, lr=1e-3, weight_decay=0.01)
     h.fill_state()
     oc = h.oracle_chunks()
     oscaler = oracle.ScalerOracle(**kw)
@@ -72,16 +77,26 @@ class _MLP(torch.nn.Module):
         return (self.fc2(torch.tanh(self.fc1(x))) * self.gain).float().pow(2).mean()
 
 
+def _snap(t):
+    """A private host copy (a host-resident payload would otherwise be aliased by ".cpu()")."""
+    return t.detach().to("cpu", copy=True).numpy()
+
+
+@pytest.mark.parametrize("host_positions", [(), (1,), (0, 1)])
 @pytest.mark.parametrize("loss_scale", [0, 128])
-def test_engine_end_to_end_against_oracle(loss_scale):
+def test_engine_end_to_end_against_oracle(loss_scale, host_positions):
     """initialize_engine -> forward -> backward -> step on a small fp16 model.  After backward the fp16 chunk payloads
-    hold the gradients; the oracle is fed exactly those and must agree bit for bit with what step() leaves behind."""
+    hold the gradients; the oracle is fed exactly those and must agree bit for bit with what step() leaves behind.
+    With a host-chunk policy the selected positions keep fp32 param / m / v in pinned host memory and the fp16
+    payload (the module's parameters) in HBM; where the state lives must not change a bit."""
     torch.manual_seed(0)
     config = {
         "optimizer": {"type": "AdamW", "params": {"lr": 1e-3, "betas": (0.9, 0.999), "eps": 1e-8, "weight_decay": 0.01}},
         "fp16": {"enabled": True, "loss_scale": loss_scale, "initial_scale_power": 7, "loss_scale_window": 4, "hysteresis": 2, "min_loss_scale": 1},
         "default_chunk_size": 1100,
     }
+    if host_positions:
+        config["client"] = {"host_chunk_policy": lambda pos: pos in host_positions}
     engine, optimizer = ps.initialize_engine(model_func=_MLP, local_rank=0, config=config)
     client = engine.client
     assert engine.optimizer is optimizer and isinstance(optimizer, ps.FP16Adam)
@@ -89,8 +104,13 @@ def test_engine_end_to_end_against_oracle(loss_scale):
     pos = client.positions()
     assert len(pos) == 2  # fc1 fills 1000 of 1100; fc2 (328) does not fit behind it -> second chunk, which also takes gain
     cl = client.chunk_list
-    mirror = [{"p32": cl[q.fp32].payload.cpu().numpy(), "m": cl[q.exp_avg].payload.cpu().numpy(),
-               "v": cl[q.exp_avg_sq].payload.cpu().numpy(), "p16": cl[q.fp16].payload.cpu().numpy()} for q in pos]
+    for i, q in enumerate(pos):
+        assert q.on_host == (i in host_positions)
+        assert cl[q.fp16].payload.is_cuda
+        for cid in (q.fp32, q.exp_avg, q.exp_avg_sq):
+            assert cl[cid].payload.is_cuda != q.on_host and (cl[cid].payload.is_pinned() or not q.on_host)
+    mirror = [{"p32": _snap(cl[q.fp32].payload), "m": _snap(cl[q.exp_avg].payload),
+               "v": _snap(cl[q.exp_avg_sq].payload), "p16": _snap(cl[q.fp16].payload)} for q in pos]
     oscaler = oracle.scaler_from_config(config["fp16"])
     oopt = oracle.OptimizerStepOracle(mirror, oscaler, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
     x = torch.randn(16, 24, device="cuda").half()
@@ -100,20 +120,21 @@ def test_engine_end_to_end_against_oracle(loss_scale):
         engine.backward(loss)
         assert all(p.grad is None for p in engine.module.parameters())
         for q, c in zip(pos, mirror):
-            c["p16"][...] = cl[q.fp16].payload.cpu().numpy()  # the gradients, as backward left them in the chunks
+            c["p16"][...] = _snap(cl[q.fp16].payload)  # the gradients, as backward left them in the chunks
         optimizer.step()
+        torch.cuda.synchronize()  # host-resident state is written by copies the host does not otherwise wait for
         oopt.check_overflow()
         skipped = oopt.step()
         if loss_scale == 0:
             assert skipped == (it == 3)
         for q, c in zip(pos, mirror):
             for key, cid in (("p32", q.fp32), ("m", q.exp_avg), ("v", q.exp_avg_sq), ("p16", q.fp16)):
-                got = cl[cid].payload.cpu().numpy()
+                got = _snap(cl[cid].payload)
                 if loss_scale != 0 and it >= 3:
                     assert np.array_equal(np.isnan(got), np.isnan(c[key]))  # static scale: the poison spreads, same places
                 else:
                     assert_bits_equal(got, c[key], f"iteration {it} {key}")
-        losses.append(float(loss))
+        losses.append(float(loss.detach()))
         if loss_scale == 0:
             assert optimizer.loss_scaler.loss_scale == oscaler.loss_scale
     if loss_scale == 0:

@@ -221,10 +221,12 @@ def test_bench_refuses_more_than_one_gpu():
     assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
 
 
-def test_host_chunk_policy_is_for_directly_driven_chunk_lists():
-    client = ps.PatrickStarClient(0, 64, device="cpu", config={"host_chunk_policy": lambda pos: True})
-    with pytest.raises(NotImplementedError, match="register_model"):
-        client.register_model(torch.nn.Linear(4, 4))
+def test_registered_module_keeps_fp16_payloads_in_hbm_under_a_host_policy():
+    client = ps.PatrickStarClient(0, 64, device="cpu", config={"host_chunk_policy": lambda pos: False})
+    assert client.host_keeps_fp16 is True  # directly driven chunk lists: whole positions go to the host
+    client.register_model(torch.nn.Linear(4, 4))
+    assert client.host_keeps_fp16 is False  # a module computes with its fp16 payloads: only p32 / m / v may leave
+    assert ps.PatrickStarClient(0, 64, device="cpu", config={"host_keeps_fp16": False}).host_keeps_fp16 is False
 
 
 def test_plan_host_positions():
@@ -241,6 +243,11 @@ def test_plan_host_positions():
     assert ps.plan_host_positions(5, n, free_bytes=1e9) == set(range(5))
     policy = planned.__contains__
     assert policy(179) and not policy(0)
+    # fp16 payloads of host positions stay in HBM: they cost 2 B/element there, and a staging slot 12
+    planned12 = ps.plan_host_positions(180, n, free_bytes=160e9, staging_slots=2, margin_use_ratio=0.8, host_keeps_fp16=False)
+    r12 = 180 - len(planned12)
+    used = lambda r: r * per + (180 - r) * 2 * n + 2 * 12 * n
+    assert planned12 == set(range(r12, 180)) and used(r12) <= 160e9 * 0.8 < used(r12 + 1) and r12 < resident
 
 
 def test_product_never_touches_the_oracle():
