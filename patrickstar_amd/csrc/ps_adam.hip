@@ -16,7 +16,9 @@
 //     1-read-1-write copy peaks at 6.2-6.3 TB/s on the same GPU);
 //   * chunk descriptors travel in the kernel-argument segment (64 per launch),
 //     so a wave's first data load depends on one scalar load, not two;
-//   * plain (temporal) loads/stores: non-temporal hints cost 20-25 %.
+//   * plain (temporal) loads/stores: non-temporal loads cost 6 % at this
+//     operating point (20-25 % with fully occupied CUs), non-temporal stores
+//     change nothing.
 //
 // Arithmetic contract (bit-exact with the explicit-intrinsic body of the
 // reference operator, patrickstar/ops/csrc/adam/cpu_adam.cpp:91-141): every
@@ -54,7 +56,7 @@
 #define PS_LDS_KB 17  // KiB of (unused) dynamic LDS requested per workgroup: caps resident workgroups per CU at floor(160 / PS_LDS_KB) = 9
 #endif
 #ifndef PS_STREAMING
-#define PS_STREAMING 0  // 1 marks chunk payload accesses non-temporal (slower on MI355X)
+#define PS_STREAMING 0  // bit 0: non-temporal loads, bit 1: non-temporal stores of chunk payloads (both slower on MI355X)
 #endif
 #if PS_MAX_WAVES_PER_EU > 0
 #define PS_OCCUPANCY __attribute__((amdgpu_waves_per_eu(1, PS_MAX_WAVES_PER_EU)))
@@ -353,7 +355,7 @@ typedef PS_GLOBAL uint2v guint2v;
 
 __device__ __forceinline__ float4v ld_f4(const float* p)
 {
-#if PS_STREAMING
+#if PS_STREAMING & 1
     return __builtin_nontemporal_load((const gfloat4v*)(p));
 #else
     return *(const gfloat4v*)(p);
@@ -361,7 +363,7 @@ __device__ __forceinline__ float4v ld_f4(const float* p)
 }
 __device__ __forceinline__ void st_f4(float* p, float4v v)
 {
-#if PS_STREAMING
+#if PS_STREAMING & 2
     __builtin_nontemporal_store(v, (gfloat4v*)(p));
 #else
     *(gfloat4v*)(p) = v;
@@ -369,7 +371,7 @@ __device__ __forceinline__ void st_f4(float* p, float4v v)
 }
 __device__ __forceinline__ uint4v ld_u4(const uint16_t* p)
 {
-#if PS_STREAMING
+#if PS_STREAMING & 1
     return __builtin_nontemporal_load((const guint4v*)(p));
 #else
     return *(const guint4v*)(p);
@@ -377,7 +379,7 @@ __device__ __forceinline__ uint4v ld_u4(const uint16_t* p)
 }
 __device__ __forceinline__ void st_u4(uint16_t* p, uint4v v)
 {
-#if PS_STREAMING
+#if PS_STREAMING & 2
     __builtin_nontemporal_store(v, (guint4v*)(p));
 #else
     *(guint4v*)(p) = v;
@@ -410,7 +412,11 @@ __device__ __forceinline__ HalfWords ld_halves(const uint16_t* p)
 #pragma unroll
         for (int k = 0; k < kWords; ++k) r.w[k] = t[k];
     } else {
+#if PS_STREAMING & 1
+        uint2v t = __builtin_nontemporal_load((const guint2v*)(p));
+#else
         uint2v t = *(const guint2v*)(p);
+#endif
 #pragma unroll
         for (int k = 0; k < kWords; ++k) r.w[k] = t[k];
     }
@@ -428,7 +434,11 @@ __device__ __forceinline__ void st_halves(uint16_t* p, const HalfWords& r)
         uint2v t;
 #pragma unroll
         for (int k = 0; k < kWords; ++k) t[k] = r.w[k];
+#if PS_STREAMING & 2
+        __builtin_nontemporal_store(t, (guint2v*)(p));
+#else
         *(guint2v*)(p) = t;
+#endif
     }
 }
 
