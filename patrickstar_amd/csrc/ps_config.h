@@ -1,0 +1,29 @@
+// Build-time tuning knobs of the fused Adam kernels (defaults = measured best on MI355X).
+#ifndef PS_CONFIG_H
+#define PS_CONFIG_H
+
+#ifndef PS_BLOCK
+#define PS_BLOCK 64  // threads per workgroup
+#endif
+#ifndef PS_LANE_ELEMS
+#define PS_LANE_ELEMS 4  // elements per lane per vector step (4 or 8)
+#endif
+#ifndef PS_UNROLL
+#define PS_UNROLL 1  // vector steps per lane per tile
+#endif
+#ifndef PS_MAX_WAVES_PER_EU
+#define PS_MAX_WAVES_PER_EU 0  // cap on resident waves per SIMD (0: no cap; the LDS request below does the capping)
+#endif
+#ifndef PS_LDS_KB
+#define PS_LDS_KB 17  // KiB of (unused) dynamic LDS requested per workgroup: caps resident workgroups per CU at floor(160 / PS_LDS_KB) = 9
+#endif
+#ifndef PS_STREAMING
+#define PS_STREAMING 0  // bit 0: non-temporal loads, bit 1: non-temporal stores of chunk payloads (both slower on MI355X)
+#endif
+#if PS_MAX_WAVES_PER_EU > 0
+#define PS_OCCUPANCY __attribute__((amdgpu_waves_per_eu(1, PS_MAX_WAVES_PER_EU)))
+#else
+#define PS_OCCUPANCY
+#endif
+
+#endif  // PS_CONFIG_H

@@ -1,0 +1,459 @@
+// The kernels: fused chunk-list step (host-decided and device-gated), restore / cast, flat-tensor operator, inf/nan probe, gradient-to-chunk copy, step-state maintenance.
+#ifndef PS_KERNELS_H
+#define PS_KERNELS_H
+
+#include "ps_tile.h"
+
+namespace {
+
+// ------------------------------------------------------- chunk-list kernels
+//
+// Grid: x = tile inside a chunk, y = chunk inside the batch.  Up to kBatch
+// descriptors are passed BY VALUE in the kernel-argument segment.
+
+constexpr int kBatch = 64;
+struct ChunkBatch {
+    ps_chunk c[kBatch];
+};
+static_assert(sizeof(ps_chunk) == 32 && sizeof(ps_step_state) == 160 && sizeof(ps_scale_record) == 16,
+              "layout of the boundary structs");
+
+// Host-decided step: all scalars arrive as kernel arguments and the
+// arithmetic variant is a compile-time property of the kernel.
+template <int ARITH, int WD, int UNS>
+__global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
+    adam_chunks_kernel(ChunkBatch b, size_t chunk_numel, StepConsts c)
+{
+    adam_tile<ARITH, WD, UNS>(c, b.c[blockIdx.y], (size_t)blockIdx.x * kTile, chunk_numel);
+}
+
+struct GatedArgs {
+    double lr, eps, wd;  // the Python numbers; the operator's arithmetic narrows them to float
+    double grad_clamp;
+    int adamw;
+    int bias_correction;
+};
+
+// Device-decided step: overflow flag, loss scale and beta^t come from the
+// device-resident state; a flagged step restores fp16 from fp32 instead.
+// The weight-decay form is known to the host; the unscale form depends on
+// the device-resident scale and is a uniform branch around the arithmetic.
+template <int ARITH, int WD>
+__global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
+    adam_chunks_gated_kernel(ChunkBatch b, size_t chunk_numel, GatedArgs ga,
+                             const ps_step_state* __restrict__ st)
+{
+    const ps_chunk& ch = b.c[blockIdx.y];
+    const size_t base = (size_t)blockIdx.x * kTile;
+    if (st->overflow) {
+        restore_tile(ch.param_fp32, ch.param_fp16, base, chunk_numel);
+        return;
+    }
+    StepConsts c;
+    const float clip = clamp_bound(ga.grad_clamp, st->cur_scale);
+    if (ARITH == PS_ARITH_OPERATOR) {
+        // The operator takes its scalars and loss_scale as C floats: the Python numbers narrow (RNE).
+        finish_consts(c, (float)ga.lr, st->beta1, st->beta2, (float)ga.eps, (float)ga.wd,
+                      ga.adamw != 0, st->beta1_t_next, st->beta2_t_next, ga.bias_correction != 0,
+                      (float)st->cur_scale, clip);
+    } else {
+        const bool bc = ga.bias_correction != 0;
+        torch_consts(c, ga.lr, st->beta1_f64, st->beta2_f64, ga.eps, ga.wd, ga.adamw != 0,
+                     bc ? st->bias_correction1_next : 1.0, bc ? st->bias_correction2_next : 1.0,
+                     st->cur_scale, clip);
+    }
+    adam_tile<ARITH, WD, UNSCALE_RUNTIME>(c, ch, base, chunk_numel);
+}
+
+__global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
+    restore_chunks_kernel(ChunkBatch b, size_t chunk_numel, const ps_step_state* __restrict__ st)
+{
+    if (st != nullptr && !st->overflow) return;
+    const ps_chunk& ch = b.c[blockIdx.y];
+    restore_tile(ch.param_fp32, ch.param_fp16, (size_t)blockIdx.x * kTile, chunk_numel);
+}
+
+__global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
+    cast_kernel(const float* __restrict__ src, uint16_t* __restrict__ dst, size_t numel,
+                size_t n_tiles)
+{
+    for (size_t t = blockIdx.x; t < n_tiles; t += gridDim.x)
+        restore_tile(src, dst, t * (size_t)kTile, numel);
+}
+
+// ------------------------------------------------- auxiliary (non-hot) kernels
+
+constexpr int kAuxBlock = 256;
+
+// Flat tensor, any grad dtype, optional fp16 output (adam_update of the operator).
+// Element-wise accesses: tensors handed to the operator are views at arbitrary
+// element offsets inside a chunk, so no alignment can be assumed.
+template <int WD, bool GRAD_HALF>
+__global__ void __launch_bounds__(kAuxBlock)
+    adam_flat_kernel(StepConsts c, float* p32, const void* grads, float* m32, float* v32,
+                     uint16_t* out16, size_t numel)
+{
+    const uint16_t* gh = static_cast<const uint16_t*>(grads);
+    const float* gf = static_cast<const float*>(grads);
+    size_t stride = (size_t)gridDim.x * kAuxBlock;
+    for (size_t i = (size_t)blockIdx.x * kAuxBlock + threadIdx.x; i < numel; i += stride) {
+        float g = GRAD_HALF ? half_bits_to_float(gh[i]) : gf[i];
+        float p = p32[i], m = m32[i], v = v32[i];
+        element_any<PS_ARITH_OPERATOR, WD, UNSCALE_RUNTIME>(c, g, p, m, v);
+        p32[i] = p;
+        m32[i] = m;
+        v32[i] = v;
+        if (out16) out16[i] = (uint16_t)float_to_half_bits(p);
+    }
+}
+
+// The same operator on a span whose four (five) addresses share one 16-byte phase: single-wave
+// workgroups over 256-element tiles with 16-byte accesses, resident-workgroup cap as for the chunk
+// kernels.  Gradients are read only; the fp16 output is optional.
+template <int WD, bool GRAD_HALF>
+__global__ void __launch_bounds__(64)
+    adam_flat_vec_kernel(StepConsts c, float* p32, const void* grads, float* m32, float* v32,
+                         uint16_t* out16,  // may alias grads (fp16 gradients overwritten by fp16 parameters)
+                         size_t n_tiles)
+{
+    for (size_t t = blockIdx.x; t < n_tiles; t += gridDim.x) {
+        const size_t i = (t * 64 + threadIdx.x) * 4;
+        float g[4];
+        if (GRAD_HALF) {
+            uint2v w = *(const guint2v*)(static_cast<const uint16_t*>(grads) + i);
+            g[0] = half_bits_to_float(w[0] & 0xFFFFu);
+            g[1] = half_bits_to_float(w[0] >> 16);
+            g[2] = half_bits_to_float(w[1] & 0xFFFFu);
+            g[3] = half_bits_to_float(w[1] >> 16);
+        } else {
+            float4v gv = ld_f4(static_cast<const float*>(grads) + i);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) g[e] = gv[e];
+        }
+        float4v p = ld_f4(p32 + i), m = ld_f4(m32 + i), v = ld_f4(v32 + i);
+        uint32_t h[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float pe = p[e], me = m[e], ve = v[e];
+            element_any<PS_ARITH_OPERATOR, WD, UNSCALE_RUNTIME>(c, g[e], pe, me, ve);
+            p[e] = pe;
+            m[e] = me;
+            v[e] = ve;
+            h[e] = float_to_half_bits(pe);
+        }
+        st_f4(p32 + i, p);
+        st_f4(m32 + i, m);
+        st_f4(v32 + i, v);
+        if (out16 != nullptr) {
+            uint2v o;
+            o[0] = h[0] | (h[1] << 16);
+            o[1] = h[2] | (h[3] << 16);
+            *(guint2v*)(out16 + i) = o;
+        }
+    }
+}
+
+// ----------------------------------------------------------- overflow scan
+//
+// A binary16 value is inf or nan iff its five exponent bits are all set.
+// For a 32-bit word holding two halves: mask the exponents, add one unit of
+// the lowest exponent bit to each; an all-ones exponent carries into bit 15 /
+// bit 31 (the masked low half is at most 0x7C00, so its carry stops at bit 15).
+
+__device__ __forceinline__ uint32_t nonfinite_halves(uint32_t w)
+{
+    return ((w & 0x7C007C00u) + 0x04000400u) & 0x80008000u;
+}
+
+// OR across the block: shuffle butterfly inside each wave, LDS across the
+// four waves, then at most one atomic per block (none when nothing was seen).
+__device__ __forceinline__ void block_flag_commit(uint32_t hit, uint32_t* flag)
+{
+    __shared__ uint32_t wave_hit[kAuxBlock / 64];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) hit |= (uint32_t)__shfl_xor((int)hit, off, 64);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) wave_hit[wave] = hit;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t any = 0;
+#pragma unroll
+        for (int w = 0; w < kAuxBlock / 64; ++w) any |= wave_hit[w];
+        if (any) atomicOr(flag, 1u);
+    }
+}
+
+constexpr int kScanUnroll = 4;
+constexpr int kScanTile = kAuxBlock * 8 * kScanUnroll;  // 16-byte loads of 8 halves: 8192 halves = 16 KiB per tile
+
+// One scan tile of a fp16 buffer.
+__device__ __forceinline__ uint32_t scan_tile_f16(const uint16_t* __restrict__ h, size_t numel,
+                                                  size_t tile)
+{
+    uint32_t hit = 0;
+    const size_t base = tile * (size_t)kScanTile;
+    if (base >= numel) return 0;
+    if ((((uintptr_t)h) & 15u) == 0 && base + kScanTile <= numel) {
+        uint4v w[kScanUnroll];
+#pragma unroll
+        for (int u = 0; u < kScanUnroll; ++u)
+            w[u] = ld_u4(h + base + ((size_t)u * kAuxBlock + threadIdx.x) * 8);
+#pragma unroll
+        for (int u = 0; u < kScanUnroll; ++u)
+            hit |= nonfinite_halves(w[u][0]) | nonfinite_halves(w[u][1]) |
+                   nonfinite_halves(w[u][2]) | nonfinite_halves(w[u][3]);
+    } else {
+        size_t end = base + kScanTile < numel ? base + kScanTile : numel;
+        for (size_t i = base + threadIdx.x; i < end; i += kAuxBlock)
+            hit |= ((h[i] & 0x7C00u) == 0x7C00u) ? 1u : 0u;
+    }
+    return hit;
+}
+
+__global__ void __launch_bounds__(kAuxBlock)
+    scan_f16_kernel(const uint16_t* __restrict__ h, size_t numel, size_t n_tiles,
+                    ps_step_state* st)
+{
+    uint32_t hit = 0;
+    for (size_t t = blockIdx.x; t < n_tiles; t += gridDim.x) hit |= scan_tile_f16(h, numel, t);
+    block_flag_commit(hit, &st->overflow);
+}
+
+__global__ void __launch_bounds__(kAuxBlock)
+    scan_f32_kernel(const float* __restrict__ f, size_t numel, ps_step_state* st)
+{
+    uint32_t hit = 0;
+    const uint32_t* w = reinterpret_cast<const uint32_t*>(f);
+    size_t stride = (size_t)gridDim.x * kAuxBlock;
+    for (size_t i = (size_t)blockIdx.x * kAuxBlock + threadIdx.x; i < numel; i += stride)
+        hit |= ((w[i] & 0x7F800000u) == 0x7F800000u) ? 1u : 0u;
+    block_flag_commit(hit, &st->overflow);
+}
+
+__global__ void __launch_bounds__(kAuxBlock)
+    scan_chunks_kernel(ChunkBatch b, size_t chunk_numel, ps_step_state* st)
+{
+    uint32_t hit = scan_tile_f16(b.c[blockIdx.y].param_fp16, chunk_numel, blockIdx.x);
+    block_flag_commit(hit, &st->overflow);
+}
+
+// Backward-side producer: copy one gradient into its slot of the fp16 chunk
+// (patrickstar/core/hook.py:212-216) and probe it for inf/nan in the same pass
+// (loss_scaler.py:133-155), instead of a separate cast + sum + host sync per
+// parameter.  Slots start at arbitrary element offsets, so accesses are per
+// element.  fp32 gradients are rounded to fp16 (RNE); the probe looks at the
+// value that lands in the chunk.
+template <bool SRC_HALF>
+__global__ void __launch_bounds__(kAuxBlock)
+    grad_to_chunk_kernel(const void* __restrict__ src, uint16_t* __restrict__ dst, size_t numel,
+                         ps_step_state* st)
+{
+    const uint16_t* sh = static_cast<const uint16_t*>(src);
+    const float* sf = static_cast<const float*>(src);
+    uint32_t hit = 0;
+    size_t stride = (size_t)gridDim.x * kAuxBlock;
+    for (size_t i = (size_t)blockIdx.x * kAuxBlock + threadIdx.x; i < numel; i += stride) {
+        uint32_t h = SRC_HALF ? (uint32_t)sh[i] : float_to_half_bits(sf[i]);
+        dst[i] = (uint16_t)h;
+        hit |= ((h & 0x7C00u) == 0x7C00u) ? 1u : 0u;
+    }
+    if (st != nullptr) block_flag_commit(hit, &st->overflow);
+}
+
+// Vector form of the same copy for long gradients.  The chunk slot sets the grid: 16-byte stores to
+// 16-byte aligned addresses of the slot.  A fp16 source is generally at a different phase, so each lane
+// loads the two ALIGNED 16-byte source blocks that straddle its output vector and funnel-shifts them by
+// S halves in registers; no misaligned memory access is made.  Every 16-byte block that is loaded holds
+// at least one element of the gradient, so it lies inside the gradient's allocation.
+template <int S>
+__device__ __forceinline__ uint4v shift_halves(const uint4v& a, const uint4v& b)
+{
+    const uint32_t w[8] = {a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+    constexpr int d = (2 * S) / 4, r = (2 * S) % 4;
+    uint4v o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = r ? ((w[i + d] >> 16) | (w[i + d + 1] << 16)) : w[i + d];
+    return o;
+}
+
+template <int S>
+__device__ __forceinline__ uint32_t copy_shifted_f16(const uint16_t* src_al, uint16_t* dst_al,
+                                                      size_t n_vec)
+{
+    uint32_t hit = 0;
+    size_t stride = (size_t)gridDim.x * kAuxBlock;
+    for (size_t j = (size_t)blockIdx.x * kAuxBlock + threadIdx.x; j < n_vec; j += stride) {
+        uint4v a = ld_u4(src_al + 8 * j);
+        uint4v b = a;
+        if (S != 0) b = ld_u4(src_al + 8 * j + 8);
+        uint4v o = shift_halves<S>(a, b);
+        hit |= nonfinite_halves(o[0]) | nonfinite_halves(o[1]) | nonfinite_halves(o[2]) |
+               nonfinite_halves(o[3]);
+        st_u4(dst_al + 8 * j, o);
+    }
+    return hit;
+}
+
+__global__ void __launch_bounds__(kAuxBlock)
+    grad_to_chunk_f16_vec_kernel(const uint16_t* __restrict__ src_al, int shift,
+                                 uint16_t* __restrict__ dst_al, size_t n_vec, ps_step_state* st)
+{
+    uint32_t hit = 0;
+    switch (shift) {
+        case 0: hit = copy_shifted_f16<0>(src_al, dst_al, n_vec); break;
+        case 1: hit = copy_shifted_f16<1>(src_al, dst_al, n_vec); break;
+        case 2: hit = copy_shifted_f16<2>(src_al, dst_al, n_vec); break;
+        case 3: hit = copy_shifted_f16<3>(src_al, dst_al, n_vec); break;
+        case 4: hit = copy_shifted_f16<4>(src_al, dst_al, n_vec); break;
+        case 5: hit = copy_shifted_f16<5>(src_al, dst_al, n_vec); break;
+        case 6: hit = copy_shifted_f16<6>(src_al, dst_al, n_vec); break;
+        default: hit = copy_shifted_f16<7>(src_al, dst_al, n_vec); break;
+    }
+    if (st != nullptr) block_flag_commit(hit, &st->overflow);
+}
+
+// fp32 gradients: eight dword-aligned floats per output vector (multi-dword loads need dword alignment only).
+typedef float4v __attribute__((aligned(4))) float4v_dword_aligned;
+__global__ void __launch_bounds__(kAuxBlock)
+    grad_to_chunk_f32_vec_kernel(const float* __restrict__ src, uint16_t* __restrict__ dst_al,
+                                 size_t n_vec, ps_step_state* st)
+{
+    uint32_t hit = 0;
+    size_t stride = (size_t)gridDim.x * kAuxBlock;
+    for (size_t j = (size_t)blockIdx.x * kAuxBlock + threadIdx.x; j < n_vec; j += stride) {
+        float4v x = *(const PS_GLOBAL float4v_dword_aligned*)(src + 8 * j);
+        float4v y = *(const PS_GLOBAL float4v_dword_aligned*)(src + 8 * j + 4);
+        uint4v o;
+        o[0] = float_to_half_bits(x[0]) | (float_to_half_bits(x[1]) << 16);
+        o[1] = float_to_half_bits(x[2]) | (float_to_half_bits(x[3]) << 16);
+        o[2] = float_to_half_bits(y[0]) | (float_to_half_bits(y[1]) << 16);
+        o[3] = float_to_half_bits(y[2]) | (float_to_half_bits(y[3]) << 16);
+        hit |= nonfinite_halves(o[0]) | nonfinite_halves(o[1]) | nonfinite_halves(o[2]) |
+               nonfinite_halves(o[3]);
+        st_u4(dst_al + 8 * j, o);
+    }
+    if (st != nullptr) block_flag_commit(hit, &st->overflow);
+}
+
+// ------------------------------------------------ device-resident step state
+
+__global__ void state_init_kernel(ps_step_state* st, ps_step_state init)
+{
+    if (threadIdx.x == 0 && blockIdx.x == 0) *st = init;
+}
+
+struct SeedArgs {
+    int64_t adam_step;
+    float beta1, beta2, b1t_next, b2t_next;
+    double beta1_f64, beta2_f64, bc1_next, bc2_next;
+};
+
+__global__ void state_seed_kernel(ps_step_state* st, SeedArgs a)
+{
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        st->adam_step = a.adam_step;
+        st->beta1 = a.beta1;
+        st->beta2 = a.beta2;
+        st->beta1_t_next = a.b1t_next;
+        st->beta2_t_next = a.b2t_next;
+        st->beta1_f64 = a.beta1_f64;
+        st->beta2_f64 = a.beta2_f64;
+        st->bias_correction1_next = a.bc1_next;
+        st->bias_correction2_next = a.bc2_next;
+    }
+}
+
+// beta ** n for a non-negative integer n in binary64, by squaring in double-double arithmetic: the
+// result is the correctly rounded power except within ~2^-90 of a rounding boundary, which is what
+// Python's float ** int (the C library's pow) returns for all but about one step in 10^4; the
+// float constants derived from 1 - beta ** n did not differ on any of 1.8 million (beta, n) pairs.
+struct TwoDouble {
+    double hi, lo;
+};
+__device__ inline TwoDouble two_double_mul(TwoDouble a, TwoDouble b)
+{
+    double p = a.hi * b.hi;
+    double e = __builtin_fma(a.hi, b.hi, -p);
+    e += a.hi * b.lo + a.lo * b.hi;
+    double s = p + e;
+    return TwoDouble{s, e - (s - p)};
+}
+__device__ inline double pow_int(double base, int64_t n)
+{
+    TwoDouble r{1.0, 0.0}, x{base, 0.0};
+    while (n > 0) {
+        if (n & 1) r = two_double_mul(r, x);
+        n >>= 1;
+        if (n) x = two_double_mul(x, x);
+    }
+    return r.hi;
+}
+
+__global__ void state_set_scaler_kernel(ps_step_state* st, double cur_scale, int scale_is_int,
+                                        int64_t cur_iter, int64_t last_overflow_iter,
+                                        int cur_hysteresis)
+{
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        st->cur_scale = cur_scale;
+        st->scale_is_int = scale_is_int;
+        st->cur_iter = cur_iter;
+        st->last_overflow_iter = last_overflow_iter;
+        st->cur_hysteresis = cur_hysteresis;
+    }
+}
+
+// DynamicLossScaler.update_scale (loss_scaler.py:158-182), one lane.
+__global__ void scaler_update_kernel(ps_step_state* st, int flag_mode, ps_scale_record* log,
+                                     int64_t log_capacity)
+{
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    ps_step_state s = *st;
+    const bool overflow = flag_mode == PS_FLAG_FROM_DEVICE ? (s.overflow != 0) : (flag_mode != 0);
+    if (overflow) {
+        if (s.delayed_shift == 1 || s.cur_hysteresis == 1) {
+            // Python: max(cur_scale / scale_factor, min_scale) -- true division gives a
+            // float; max keeps its first argument unless the second is strictly greater.
+            double q = s.cur_scale / s.scale_factor;
+            if (s.min_scale > q) {
+                s.cur_scale = s.min_scale;
+                s.scale_is_int = s.min_is_int;
+            } else {
+                s.cur_scale = q;
+                s.scale_is_int = 0;
+            }
+        } else {
+            s.cur_hysteresis -= 1;
+        }
+        s.last_overflow_iter = s.cur_iter;
+        s.skipped_steps += 1;
+    } else {
+        if (s.consecutive_hysteresis) s.cur_hysteresis = s.delayed_shift;
+        if ((s.cur_iter - s.last_overflow_iter) % s.scale_window == 0) {
+            if (!s.consecutive_hysteresis) s.cur_hysteresis = s.delayed_shift;
+            s.cur_scale = s.cur_scale * s.scale_factor;
+            s.scale_is_int = s.scale_is_int && s.factor_is_int;
+        }
+        // the step ran: state["step"] += 1 and the float running products advance
+        s.adam_step += 1;
+        s.beta1_t_next = s.beta1_t_next * s.beta1;
+        s.beta2_t_next = s.beta2_t_next * s.beta2;
+        // fp16_cpu_adam.py:412-413 for the next step
+        s.bias_correction1_next = 1.0 - pow_int(s.beta1_f64, s.adam_step + 1);
+        s.bias_correction2_next = 1.0 - pow_int(s.beta2_f64, s.adam_step + 1);
+    }
+    if (log != nullptr && log_capacity > 0) {
+        ps_scale_record r;
+        r.scale_after = s.cur_scale;
+        r.overflow = overflow ? 1u : 0u;
+        r.scale_is_int = (uint32_t)s.scale_is_int;
+        log[s.cur_iter % log_capacity] = r;
+    }
+    s.cur_iter += 1;
+    s.last_skipped = overflow ? 1u : 0u;
+    s.overflow = 0;
+    *st = s;
+}
+
+}  // namespace
+
+#endif  // PS_KERNELS_H

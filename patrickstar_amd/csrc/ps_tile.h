@@ -1,0 +1,258 @@
+// Vector accesses and the per-workgroup tile: one 256-element tile of one chunk, loaded, updated and stored by one wave.
+#ifndef PS_TILE_H
+#define PS_TILE_H
+
+#include "ps_arith.h"
+#include "ps_config.h"
+
+namespace {
+
+// ------------------------------------------------------- vector accesses
+
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
+
+// Chunk payloads are always device-global memory; saying so keeps the
+// compiler from falling back to flat_* instructions for pointers it did not
+// see being allocated.
+#define PS_GLOBAL __attribute__((address_space(1)))
+typedef PS_GLOBAL float4v gfloat4v;
+typedef PS_GLOBAL uint4v guint4v;
+typedef PS_GLOBAL uint2v guint2v;
+
+__device__ __forceinline__ float4v ld_f4(const float* p)
+{
+#if PS_STREAMING & 1
+    return __builtin_nontemporal_load((const gfloat4v*)(p));
+#else
+    return *(const gfloat4v*)(p);
+#endif
+}
+__device__ __forceinline__ void st_f4(float* p, float4v v)
+{
+#if PS_STREAMING & 2
+    __builtin_nontemporal_store(v, (gfloat4v*)(p));
+#else
+    *(gfloat4v*)(p) = v;
+#endif
+}
+__device__ __forceinline__ uint4v ld_u4(const uint16_t* p)
+{
+#if PS_STREAMING & 1
+    return __builtin_nontemporal_load((const guint4v*)(p));
+#else
+    return *(const guint4v*)(p);
+#endif
+}
+__device__ __forceinline__ void st_u4(uint16_t* p, uint4v v)
+{
+#if PS_STREAMING & 2
+    __builtin_nontemporal_store(v, (guint4v*)(p));
+#else
+    *(guint4v*)(p) = v;
+#endif
+}
+
+constexpr int kBlock = PS_BLOCK;
+constexpr unsigned kLdsBytes = PS_LDS_KB * 1024u;
+// Elements per lane per vector step.  8: one 16-byte access of fp16 and two
+// 16-byte accesses per fp32 array.  4: an 8-byte access of fp16 and one
+// 16-byte access per fp32 array.
+constexpr int kLaneElems = PS_LANE_ELEMS;
+constexpr int kUnroll = PS_UNROLL;  // vector steps per lane per tile
+constexpr int kTile = kBlock * kLaneElems * kUnroll;
+constexpr int kQuads = kLaneElems / 4;  // float4 accesses per fp32 array per step
+constexpr int kWords = kLaneElems / 2;  // 32-bit words of fp16 pairs per step
+static_assert(kLaneElems == 4 || kLaneElems == 8, "PS_LANE_ELEMS must be 4 or 8");
+static_assert(kBlock % 64 == 0 && kBlock >= 64 && kBlock <= 1024, "PS_BLOCK must be whole waves");
+
+// fp16 pairs of one lane and step: 2 or 4 words, moved with one 8- or 16-byte access
+struct HalfWords {
+    uint32_t w[kWords];
+};
+
+__device__ __forceinline__ HalfWords ld_halves(const uint16_t* p)
+{
+    HalfWords r;
+    if (kWords == 4) {
+        uint4v t = ld_u4(p);
+#pragma unroll
+        for (int k = 0; k < kWords; ++k) r.w[k] = t[k];
+    } else {
+#if PS_STREAMING & 1
+        uint2v t = __builtin_nontemporal_load((const guint2v*)(p));
+#else
+        uint2v t = *(const guint2v*)(p);
+#endif
+#pragma unroll
+        for (int k = 0; k < kWords; ++k) r.w[k] = t[k];
+    }
+    return r;
+}
+
+__device__ __forceinline__ void st_halves(uint16_t* p, const HalfWords& r)
+{
+    if (kWords == 4) {
+        uint4v t;
+#pragma unroll
+        for (int k = 0; k < kWords; ++k) t[k] = r.w[k];
+        st_u4(p, t);
+    } else {
+        uint2v t;
+#pragma unroll
+        for (int k = 0; k < kWords; ++k) t[k] = r.w[k];
+#if PS_STREAMING & 2
+        __builtin_nontemporal_store(t, (guint2v*)(p));
+#else
+        *(guint2v*)(p) = t;
+#endif
+    }
+}
+
+// The registers of one lane for one tile.
+struct LaneTile {
+    HalfWords g[kUnroll];
+    float4v p[kUnroll][kQuads], m[kUnroll][kQuads], v[kUnroll][kQuads];
+    HalfWords h[kUnroll];
+};
+
+template <int ARITH, int WD, int UNS>
+__device__ __forceinline__ void lane_math(const StepConsts& c, LaneTile& r)
+{
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+        for (int w = 0; w < kWords; ++w) {
+            uint32_t word = r.g[u].w[w];
+            float g0 = half_bits_to_float(word & 0xFFFFu);
+            float g1 = half_bits_to_float(word >> 16);
+            const int e0 = 2 * w, e1 = 2 * w + 1;
+            float p0 = r.p[u][e0 >> 2][e0 & 3], m0 = r.m[u][e0 >> 2][e0 & 3],
+                  v0 = r.v[u][e0 >> 2][e0 & 3];
+            float p1 = r.p[u][e1 >> 2][e1 & 3], m1 = r.m[u][e1 >> 2][e1 & 3],
+                  v1 = r.v[u][e1 >> 2][e1 & 3];
+            adam_element<ARITH, WD, UNS>(c, g0, p0, m0, v0);
+            adam_element<ARITH, WD, UNS>(c, g1, p1, m1, v1);
+            r.p[u][e0 >> 2][e0 & 3] = p0;
+            r.m[u][e0 >> 2][e0 & 3] = m0;
+            r.v[u][e0 >> 2][e0 & 3] = v0;
+            r.p[u][e1 >> 2][e1 & 3] = p1;
+            r.m[u][e1 >> 2][e1 & 3] = m1;
+            r.v[u][e1 >> 2][e1 & 3] = v1;
+            r.h[u].w[w] = float_to_half_bits(p0) | (float_to_half_bits(p1) << 16);
+        }
+    }
+}
+
+// One tile of one chunk, fast path: the whole tile is in range and all four
+// bases are 16-byte aligned.  All loads of the tile are issued before the
+// first use.  Loads and stores are written once, outside any branch on the
+// arithmetic variant.
+template <int ARITH, int WD, int UNS>
+__device__ __forceinline__ void adam_tile_vec(const StepConsts& c, float* __restrict__ p32,
+                                              float* __restrict__ m32, float* __restrict__ v32,
+                                              uint16_t* __restrict__ h16, size_t base)
+{
+    LaneTile r;
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        size_t i = base + ((size_t)u * kBlock + threadIdx.x) * kLaneElems;
+        r.g[u] = ld_halves(h16 + i);
+#pragma unroll
+        for (int q = 0; q < kQuads; ++q) r.p[u][q] = ld_f4(p32 + i + 4 * q);
+#pragma unroll
+        for (int q = 0; q < kQuads; ++q) r.m[u][q] = ld_f4(m32 + i + 4 * q);
+#pragma unroll
+        for (int q = 0; q < kQuads; ++q) r.v[u][q] = ld_f4(v32 + i + 4 * q);
+    }
+    if (UNS != UNSCALE_RUNTIME) {
+        lane_math<ARITH, WD, UNS>(c, r);
+    } else if (c.unscale == UNSCALE_MUL) {
+        lane_math<ARITH, WD, UNSCALE_MUL>(c, r);
+    } else if (ARITH == PS_ARITH_OPERATOR && c.unscale == UNSCALE_DIV) {
+        lane_math<ARITH, WD, UNSCALE_DIV>(c, r);
+    } else {
+        lane_math<ARITH, WD, UNSCALE_NONE>(c, r);
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        size_t i = base + ((size_t)u * kBlock + threadIdx.x) * kLaneElems;
+#pragma unroll
+        for (int q = 0; q < kQuads; ++q) st_f4(p32 + i + 4 * q, r.p[u][q]);
+#pragma unroll
+        for (int q = 0; q < kQuads; ++q) st_f4(m32 + i + 4 * q, r.m[u][q]);
+#pragma unroll
+        for (int q = 0; q < kQuads; ++q) st_f4(v32 + i + 4 * q, r.v[u][q]);
+        st_halves(h16 + i, r.h[u]);
+    }
+}
+
+// Same elements, one at a time: ragged tile ends and unaligned bases.
+template <int ARITH, int WD, int UNS>
+__device__ __forceinline__ void adam_tile_scalar(const StepConsts& c, float* p32, float* m32,
+                                                 float* v32, uint16_t* h16, size_t base, size_t end)
+{
+    for (size_t i = base + threadIdx.x; i < end; i += kBlock) {
+        float g = half_bits_to_float(h16[i]);
+        float p = p32[i], m = m32[i], v = v32[i];
+        element_any<ARITH, WD, UNS>(c, g, p, m, v);
+        p32[i] = p;
+        m32[i] = m;
+        v32[i] = v;
+        h16[i] = (uint16_t)float_to_half_bits(p);
+    }
+}
+
+__device__ __forceinline__ bool aligned16(const void* a, const void* b, const void* c,
+                                          const void* d)
+{
+    return (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)d) & 15u) == 0;
+}
+
+template <int ARITH, int WD, int UNS>
+__device__ __forceinline__ void adam_tile(const StepConsts& c, const ps_chunk& ch, size_t base,
+                                          size_t chunk_numel)
+{
+    size_t end = base + kTile;
+    if (end <= chunk_numel && aligned16(ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16)) {
+        adam_tile_vec<ARITH, WD, UNS>(c, ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16,
+                                      base);
+    } else {
+        if (end > chunk_numel) end = chunk_numel;
+        adam_tile_scalar<ARITH, WD, UNS>(c, ch.param_fp32, ch.exp_avg, ch.exp_avg_sq,
+                                         ch.param_fp16, base, end);
+    }
+}
+
+// fp16 <- RNE(fp32) for one tile (the restore of a skipped step and the
+// stand-alone write-back).
+__device__ __forceinline__ void restore_tile(const float* __restrict__ p32,
+                                             uint16_t* __restrict__ h16, size_t base,
+                                             size_t numel)
+{
+    size_t end = base + kTile;
+    if (end <= numel && ((((uintptr_t)p32 | (uintptr_t)h16) & 15u) == 0)) {
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            size_t i = base + ((size_t)u * kBlock + threadIdx.x) * kLaneElems;
+            float4v a[kQuads];
+#pragma unroll
+            for (int q = 0; q < kQuads; ++q) a[q] = ld_f4(p32 + i + 4 * q);
+            HalfWords out;
+#pragma unroll
+            for (int w = 0; w < kWords; ++w)
+                out.w[w] = float_to_half_bits(a[w >> 1][(2 * w) & 3]) |
+                           (float_to_half_bits(a[w >> 1][(2 * w + 1) & 3]) << 16);
+            st_halves(h16 + i, out);
+        }
+    } else {
+        if (end > numel) end = numel;
+        for (size_t i = base + threadIdx.x; i < end; i += kBlock)
+            h16[i] = (uint16_t)float_to_half_bits(p32[i]);
+    }
+}
+
+}  // namespace
+
+#endif  // PS_TILE_H
