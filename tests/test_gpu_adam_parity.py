@@ -262,10 +262,13 @@ def test_config2_padded_two_chunks_cold_t100():
         assert not t[used:].any(), "the zero-padded tail must stay exactly zero"
 
 
-def test_config4_first_and_last_chunk_of_24():
+@pytest.mark.parametrize("arithmetic", ["operator", "torch"])
+def test_config4_first_and_last_chunk_of_24(arithmetic):
     """Configuration "GPT-2-1.5B-sized" (the timed one): 24 chunks resident in HBM, AdamW lr 1e-4 eps 1e-8 wd .01, static scale 2^12,
-    t=100.  The oracle checks the first and the last chunk; a checksum guards the ones in between against being skipped."""
-    h = ChunkHarness(24, N_FULL, ps.LossScaler(2**12), seed=4, lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
+    t=100.  The oracle checks the first and the last chunk; a checksum guards the ones in between against being skipped.
+    Under the torch arithmetic one chunk in the middle is also compared with the reference's torch calls run by torch."""
+    h = ChunkHarness(24, N_FULL, ps.LossScaler(2**12), seed=4, lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True,
+                     arithmetic=arithmetic)
     h.fill_state()
     h.fill_grads(1e-3, 2**12)
     for prm in h.params:
@@ -273,11 +276,22 @@ def test_config4_first_and_last_chunk_of_24():
     idx = [0, 23]
     oc = h.oracle_chunks(idx)
     before = [h.payloads(i)[0].view(torch.int32).sum(dtype=torch.int64).item() for i in range(24)]
-    oopt = oracle.OptimizerStepOracle(oc, oracle.StaticScalerOracle(2**12), lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
+    oopt = oracle.OptimizerStepOracle(oc, oracle.StaticScalerOracle(2**12), lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True,
+                                      arithmetic=arithmetic)
     oopt.step_count = 99
+    if arithmetic == "torch":
+        from test_oracle_torch_formula import reference_call_sequence
+
+        tp, tm, tv, tg = (t.clone() for t in h.payloads(11))
+        reference_call_sequence(tp, tg, tm, tv, 100, 1e-4, 0.9, 0.999, 1e-8, 0.01, True, 2**12)
+        del tg
     h.opt.step()
     oopt.step()
     h.compare(oc, idx, what="config 4")
+    if arithmetic == "torch":
+        for got, want in zip(h.payloads(11)[:3], (tp, tm, tv)):
+            assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+        del tp, tm, tv
     after = [h.payloads(i)[0].view(torch.int32).sum(dtype=torch.int64).item() for i in range(24)]
     assert all(a != b for a, b in zip(after, before)), "every chunk must have been updated"
     # fp16 copy == RNE(fp32) everywhere (size-independent property, checked on the device)
