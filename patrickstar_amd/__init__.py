@@ -4,6 +4,7 @@ A drop-in for ONE path of PatrickStar: ``initialize_engine(config)`` /
 ``optimizer.step()`` over the four-list chunk layout, executed by hand-written
 HIP kernels (gfx950) behind the C ABI of ``include/ps_adam.h``.
 """
+from . import adam_op  # noqa: F401
 from .chunk_layout import (  # noqa: F401
     AccessType,
     Chunk,

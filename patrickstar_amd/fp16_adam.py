@@ -30,7 +30,7 @@ from copy import deepcopy
 
 import torch
 
-from . import _lib
+from . import _lib, adam_op
 from .chunk_layout import AccessType, ChunkType, ParamType, register_param
 from .loss_scaler import DynamicLossScaler
 
@@ -143,10 +143,8 @@ class FP16Adam(torch.optim.Optimizer):
 
         self.opt_id = FP16Adam.optimizer_id
         FP16Adam.optimizer_id = FP16Adam.optimizer_id + 1
-        _lib.check(
-            self._lib.ps_adam_create(self.opt_id, lr, betas[0], betas[1], eps, weight_decay, int(bool(use_adamw)), 0),
-            "ps_adam_create",
-        )
+        self.ds_opt_adam = adam_op  # the operator module, under the attribute name the reference uses
+        self.ds_opt_adam.create_adam(self.opt_id, lr, betas[0], betas[1], eps, weight_decay, self.use_adamw, False)
         self._created = True
         if gradient_clipping is not None and gradient_clipping > 0:
             # element-wise clamp of the fp16 gradients to +-min(65504, clipping * loss_scale), fused into the kernels

@@ -24,58 +24,86 @@ def _dev(a):
 
 # ---------------------------------------------------------------- native operator
 
+def torch_adam_update(step, lr, beta1, beta2, eps, weight_decay, bias_correction, param, grad, exp_avg, exp_avg_sq,
+                      loss_scale, use_adamw):
+    """The comparison formula of the reference's operator test (unitest/test_ds_cpu_adam.py:37-71), on torch tensors."""
+    if loss_scale > 0:
+        grad.div_(loss_scale)
+    bias_correction1 = 1 - beta1**step
+    bias_correction2 = 1 - beta2**step
+    if weight_decay != 0:
+        if use_adamw:
+            param.mul_(1 - lr * weight_decay)
+        else:
+            grad = grad.add(param, alpha=weight_decay)
+    exp_avg.mul_(beta1).add_(grad, alpha=1 - beta1)
+    exp_avg_sq.mul_(beta2).addcmul_(grad, grad, value=1 - beta2)
+    denom = (exp_avg_sq.sqrt() / math.sqrt(bias_correction2)).add_(eps)
+    param.addcdiv_(exp_avg, denom, value=-(lr / bias_correction1))
+
+
 @pytest.mark.parametrize("use_adamw", [False, True])
 @pytest.mark.parametrize("shape", [(1023,), (1024, 32)])
-@pytest.mark.parametrize("grad_dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("grad_dtype", [torch.float, torch.half])
 @pytest.mark.parametrize("loss_scale", [-1, 2**5])
 def test_adam_update_reference_test_grid(use_adamw, shape, grad_dtype, loss_scale):
-    """The grid of the reference's own operator test (unitest/test_ds_cpu_adam.py:157-192): step 1,
-    lr .01, betas (.9,.999), eps 1e-8, wd .001, uniform [0,1) inputs; its bar is 1e-4 absolute against
-    a torch formula, ours is additionally bit-exactness against the oracle."""
-    lib = _lib.load()
-    rng = np.random.default_rng(abs(hash((use_adamw, shape, str(grad_dtype), loss_scale))) % 2**32)
-    n = int(np.prod(shape))
-    p = rng.random(n, dtype=np.float32)
-    g = rng.random(n, dtype=np.float32).astype(grad_dtype)
+    """The reference's own operator test (unitest/test_ds_cpu_adam.py:77-192), with the operator module under its
+    reference names (create_adam / adam_update / destroy_adam on flat tensors): step 1, lr .01, betas (.9,.999),
+    eps 1e-8, wd .001, uniform [0,1) inputs.  Its bar is 1e-4 absolute against the torch formula; ours is additionally
+    bit-exactness against the CPU restatement of the operator, and the gradients must come back untouched."""
+    cpu_adam_op = ps.adam_op
+    step, lr, eps, beta1, beta2, weight_decay = 1, 0.01, 1e-8, 0.9, 0.999, 0.001
+    torch.manual_seed(abs(hash((use_adamw, shape, str(grad_dtype), loss_scale))) % 2**31)
+    opt_id = 900
+    p_data = torch.rand(shape)
+    p_grad = torch.rand(shape, dtype=grad_dtype)
     if loss_scale > 0:
-        g = (g.astype(np.float32) * loss_scale).astype(grad_dtype)
-    m = rng.random(n, dtype=np.float32)
-    v = rng.random(n, dtype=np.float32)
-    lr, b1, b2, eps, wd = 0.01, 0.9, 0.999, 1e-8, 0.001
+        p_grad.mul_(loss_scale)
+    exp_avg = torch.rand(shape)
+    exp_avg_sq = torch.rand(shape)
+    p_data_copy, exp_avg_copy, exp_avg_sq_copy = p_data.clone(), exp_avg.clone(), exp_avg_sq.clone()
+    p_grad_copy = p_grad.clone().float()
+    host = [t.clone().view(-1).numpy() for t in (p_data, p_grad, exp_avg, exp_avg_sq)]
 
-    dp, dg, dm, dv = _dev(p.copy()), _dev(g.copy()), _dev(m.copy()), _dev(v.copy())
-    oid = 900
-    _lib.check(lib.ps_adam_create(oid, lr, b1, b2, eps, wd, int(use_adamw), 0), "create")
-    _lib.check(
-        lib.ps_adam_update(oid, 1, lr, b1, b2, eps, wd, 1, dp.data_ptr(), dg.data_ptr(), int(grad_dtype == np.float16),
-                           dm.data_ptr(), dv.data_ptr(), n, float(loss_scale), None, _lib.current_stream_handle()),
-        "update",
-    )
+    d_data, d_grad, d_avg, d_sq = (t.cuda() for t in (p_data, p_grad, exp_avg, exp_avg_sq))
+    cpu_adam_op.create_adam(opt_id, lr, beta1, beta2, eps, weight_decay, use_adamw, False)
+    cpu_adam_op.adam_update(opt_id, step, lr, beta1, beta2, eps, weight_decay, True, d_data.view(-1), d_grad.view(-1),
+                            d_avg.view(-1), d_sq.view(-1), loss_scale)
     torch.cuda.synchronize()
-    lib.ps_adam_destroy(oid)
-    assert_bits_equal(dg.cpu().numpy(), g, "grads must not be written")
+    cpu_adam_op.destroy_adam(opt_id)
 
-    po, mo, vo = p.copy(), m.copy(), v.copy()
-    oracle.AdamOracle(lr, b1, b2, eps, wd, use_adamw).update(1, lr, b1, b2, eps, wd, True, po, g, mo, vo, float(loss_scale))
-    assert_bits_equal(dp.cpu().numpy(), po, "param")
-    assert_bits_equal(dm.cpu().numpy(), mo, "exp_avg")
-    assert_bits_equal(dv.cpu().numpy(), vo, "exp_avg_sq")
+    # the reference's check: within 1e-4 of the torch formula
+    torch_adam_update(step, lr, beta1, beta2, eps, weight_decay, True, p_data_copy, p_grad_copy, exp_avg_copy,
+                      exp_avg_sq_copy, loss_scale, use_adamw)
+    assert torch.max(torch.abs(p_data_copy - d_data.cpu())) < 1e-4
+    assert torch.max(torch.abs(exp_avg_copy - d_avg.cpu())) < 1e-4
+    assert torch.max(torch.abs(exp_avg_sq_copy - d_sq.cpu())) < 1e-4
 
-    # the reference's own check: within 1e-4 of the torch formula
-    tp, tg, tm, tv = (torch.from_numpy(x.astype(np.float32)) for x in (p, g, m, v))
-    if loss_scale > 0:
-        tg = tg / loss_scale
-    if use_adamw:
-        tp = tp * (1 - lr * wd)
-    else:
-        tg = tg + wd * tp
-    tm = tm * b1 + (1 - b1) * tg
-    tv = tv * b2 + (1 - b2) * tg * tg
-    denom = tv.sqrt() / math.sqrt(1 - b2) + eps
-    tp = tp - (lr / (1 - b1)) * tm / denom
-    assert (tp - dp.cpu()).abs().max() < 1e-4
-    assert (tm - dm.cpu()).abs().max() < 1e-4
-    assert (tv - dv.cpu()).abs().max() < 1e-4
+    # ours: the gradients are read only, and every bit equals the CPU restatement of the operator
+    assert_bits_equal(d_grad.cpu().view(-1).numpy(), host[1], "grads must not be written")
+    po, g, mo, vo = host
+    oracle.AdamOracle(lr, beta1, beta2, eps, weight_decay, use_adamw).update(
+        step, lr, beta1, beta2, eps, weight_decay, True, po, g, mo, vo, float(loss_scale))
+    assert_bits_equal(d_data.cpu().view(-1).numpy(), po, "param")
+    assert_bits_equal(d_avg.cpu().view(-1).numpy(), mo, "exp_avg")
+    assert_bits_equal(d_sq.cpu().view(-1).numpy(), vo, "exp_avg_sq")
+
+
+def test_operator_module_argument_checks():
+    op = ps.adam_op
+    op.create_adam(901, 1e-3, 0.9, 0.999, 1e-8, 0.0, True, False)
+    x = torch.zeros(8, device="cuda")
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        op.adam_update(901, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, True, torch.zeros(8), x, x, x, -1)
+    with pytest.raises(RuntimeError, match="flat and contiguous"):
+        op.adam_update(901, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, True, x.view(2, 4), x, x, x, -1)
+    with pytest.raises(TypeError, match="float32"):
+        op.adam_update(901, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, True, x.half(), x, x, x, -1)
+    with pytest.raises(RuntimeError, match="differ in length"):
+        op.adam_update(901, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, True, x, x[:4], x, x, -1)
+    op.destroy_adam(901)
+    with pytest.raises(RuntimeError, match="never created"):
+        op.adam_update(901, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, True, x, x, x, x, -1)
 
 
 def test_adam_update_unaligned_views_fp16_out_and_errors():
