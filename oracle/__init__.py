@@ -23,8 +23,8 @@ Contents
                           chunk list held as numpy arrays.
 
 Pinning: see the header of ``adam_oracle.c`` for the Adam arithmetic and
-``tests/test_oracle_scaler.py`` for the state machine (hand-derived trajectories
-and invariants).  The reference's own tests hold no golden vectors for this
+``tests/test_oracle_scaler.py`` for the state machine (torch's AMP scale-update
+routine on random overflow histories, hand-derived trajectories, invariants).  The reference's own tests hold no golden vectors for this
 path; its loss-scale sequence is asserted nowhere in the reference.
 """
 import ctypes

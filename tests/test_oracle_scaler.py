@@ -8,6 +8,7 @@ only prints), so the trajectories below are derived by hand from the rules:
   always:     iteration += 1
 """
 import numpy as np
+import pytest
 
 from oracle import ScalerOracle, StaticScalerOracle, scaler_from_config
 
@@ -131,3 +132,29 @@ def test_engine_wiring_quirks():
             pass
         else:
             raise AssertionError("expected an assertion")
+
+
+@pytest.mark.parametrize("window", [1, 2, 3, 7, 1000])
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_matches_torch_amp_scale_update(window, seed):
+    """A library routine with the same contract: torch's AMP scale update (the kernel behind
+    torch.amp.GradScaler.update, which the reference's own loss-scale test runs beside PatrickStar,
+    unitest/test_loss_scale.py:114-120): back off on a step that saw inf/nan, grow after `growth_interval`
+    consecutive clean steps.  With delayed_shift = 1 and no min-scale clamp in reach the reference's state machine
+    ("grow when (cur_iter - last_overflow_iter) % window == 0") is the same function of the overflow history."""
+    import torch
+
+    rng = np.random.default_rng(seed)
+    flags = rng.random(2000 if window > 100 else 300) < 1.0 / (window + 1)  # growth and back-off roughly in balance
+    s = ScalerOracle(init_scale=2**20, scale_factor=2, scale_window=window, min_scale=2**-200)
+    scale = torch.tensor([float(2**20)])
+    tracker = torch.zeros(1, dtype=torch.int32)
+    compared = 0
+    for f in flags:
+        s.update_scale(bool(f))
+        torch._amp_update_scale_(scale, tracker, torch.tensor([float(f)]), 2.0, 0.5, window)
+        if not 2.0**-100 < s.loss_scale < 2.0**100:
+            break  # torch keeps the scale in a float32 tensor (and refuses to grow it to inf); stay inside its range
+        assert float(s.loss_scale) == scale.item()
+        compared += 1
+    assert compared >= 100
