@@ -11,7 +11,7 @@ INCLUDE = os.path.join(ROOT, "include")
 
 # -ffp-contract=off: fused multiply-adds are written out explicitly; the compiler must not add or remove any.
 # -fhip-fp32-correctly-rounded-divide-sqrt: IEEE-rounded '/' and sqrtf (hipcc's default, stated on purpose).
-# -fno-gpu-flush-denormals-to-zero? not a flag: denormals are kept with -fgpu-flush-denormals-to-zero absent.
+# Denormals are kept: -fgpu-flush-denormals-to-zero is not given.
 # packed-fp32 ops are switched off: the compiler otherwise pairs independent float ops into v_pk_* forms.
 HIPCC_FLAGS = [
     "-O3",
@@ -40,10 +40,17 @@ def hipcc_path():
 
 def build(verbose=False, extra_flags=()):
     """Compile every HIP source into patrickstar_amd/libps_adam.so; returns its path."""
-    cmd = [hipcc_path(), *HIPCC_FLAGS, *extra_flags, "-I", INCLUDE, *SOURCES, "-o", LIB_PATH]
+    # compile beside the target and rename: a process that has the old library mapped keeps its own copy
+    tmp = LIB_PATH + f".{os.getpid()}.tmp"
+    cmd = [hipcc_path(), *HIPCC_FLAGS, *extra_flags, "-I", INCLUDE, *SOURCES, "-o", tmp]
     if verbose:
         print(" ".join(cmd), flush=True)
-    subprocess.check_call(cmd)
+    try:
+        subprocess.check_call(cmd)
+        os.replace(tmp, LIB_PATH)
+    finally:
+        if os.path.exists(tmp):
+            os.remove(tmp)
     return LIB_PATH
 
 

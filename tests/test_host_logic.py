@@ -293,3 +293,15 @@ def test_argument_checks_happen_before_any_gpu_work():
     assert lib.ps_scaler_update(ctypes.c_void_p(16), 3, None, 0, None) == E
     assert lib.ps_state_seed_step(ctypes.c_void_p(16), -1, 0.9, 0.999, None) == E
     lib.ps_adam_destroy(88)
+
+
+def test_build_entry_point_compiles_and_loads():
+    """__graft_entry__.build() in a fresh process: hipcc cross-compiles the library for gfx950 without a GPU, the CPU
+    checker is rebuilt, the package imports and the ABI version matches the binding."""
+    import subprocess
+    import sys
+
+    r = subprocess.run([sys.executable, "-c", "import __graft_entry__ as g; g.build()"], cwd=ROOT, capture_output=True,
+                       text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    assert "built" in r.stdout and os.path.exists(_lib.LIB_PATH)
