@@ -37,7 +37,8 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-unfused-baseline", action="store_true",
                     help="skip timing the reference's un-fused GPU branch (a sequence of torch element-wise kernels)")
-    ap.add_argument("--cpu-reps", type=int, default=20)
+    ap.add_argument("--cpu-reps", type=int, default=20, help="CPU baseline: at least this many timed steps")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0, help="CPU baseline: keep stepping for about this long")
     ap.add_argument("--host-chunks", type=int, default=0,
                     help="with --mode hybrid: how many of --chunks live in pinned host memory (the LAST ones)")
     ap.add_argument("--slots", type=int, default=2, help="with --mode hybrid: HBM staging slots")
@@ -68,7 +69,7 @@ def traffic_from_profile():
         return None
 
 
-def cpu_baseline(reps):
+def cpu_baseline(reps, seconds):
     """The CPU oracle on one 64 Mi-element chunk with the one-chunk reference-CPU-path inputs (p~N(0,.02), m=v=0, g16=(N(0,1e-3)*8).half(), static scale 8), all host cores of this process."""
     import numpy as np
 
@@ -83,11 +84,15 @@ def cpu_baseline(reps):
     o = oracle.AdamOracle(1e-3, 0.9, 0.999, 1e-6, 0.0, False)
     isa = o.update(1, 1e-3, 0.9, 0.999, 1e-6, 0.0, True, p, g, m, v, 8.0)
     o.update(2, 1e-3, 0.9, 0.999, 1e-6, 0.0, True, p, g, m, v, 8.0)
-    best = float("inf")
-    for r in range(reps):
+    times = []
+    started = time.perf_counter()
+    while len(times) < reps or (time.perf_counter() - started < seconds and len(times) < 100000):
         t0 = time.perf_counter()
-        o.update(3 + r, 1e-3, 0.9, 0.999, 1e-6, 0.0, True, p, g, m, v, 8.0)
-        best = min(best, time.perf_counter() - t0)
+        o.update(3 + len(times), 1e-3, 0.9, 0.999, 1e-6, 0.0, True, p, g, m, v, 8.0)
+        times.append(time.perf_counter() - t0)
+    best = min(times)
+    median = sorted(times)[len(times) // 2]
+    reps = len(times)
     # the un-vectorised code path as well (what the reference's own builder selects on a non-Intel host)
     t0 = time.perf_counter()
     o.update(3 + reps, 1e-3, 0.9, 0.999, 1e-6, 0.0, True, p, g, m, v, 8.0, oracle.ISA_SCALAR)
@@ -112,7 +117,8 @@ def cpu_baseline(reps):
         "unit": "params/s",
         "cores": cores,
         "kind": "port",
-        "sample": f"1 chunk of {n} elements (one-chunk CPU-path inputs, static scale 8), best of {reps} steps after 2 warm-up; "
+        "sample": f"1 chunk of {n} elements (one-chunk CPU-path inputs, static scale 8), best of {reps} steps over "
+        f"{sum(times):.1f} s after 2 warm-up (median step {n / median / 1e9:.2f} G params/s); "
         f"oracle code path {['', 'scalar', 'AVX2', 'AVX-512'][isa]}; 26 B/element -> {26 * n / best / 1e9:.0f} GB/s; "
         f"scalar code path of the same oracle, 1 step: {n / scalar_s / 1e9:.2f} G params/s; host CPU: {cpu_model}",
     }
@@ -393,7 +399,7 @@ def main():
         out["unfused_gpu_baseline"] = unfused_gpu_branch(C, N)
         torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(args.cpu_reps)
+        out["cpu_baseline"] = cpu_baseline(args.cpu_reps, args.cpu_seconds)
     print(json.dumps(out))
 
 
