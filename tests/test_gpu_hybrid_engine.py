@@ -175,3 +175,32 @@ def test_hybrid_full_size_placement_invariance():
             y = y.cpu() if x.device.type == "cpu" else y
             assert torch.equal(x.view(torch.int16 if x.dtype == torch.half else torch.int32),
                                y.view(torch.int16 if y.dtype == torch.half else torch.int32)), f"chunk {i}"
+
+
+@pytest.mark.parametrize("host_keeps_fp16", [True, False])
+@pytest.mark.parametrize("slots", [1, 3, 8])
+def test_hybrid_slot_counts_and_slot_reuse(slots, host_keeps_fp16):
+    """More host-resident positions than staging slots, for 1, 3 and 8 slots: every slot is reused, and a chunk's
+    write-back must have left its slot before the next occupant is copied in.  Dynamic scaler, one poisoned step."""
+    kw = dict(init_scale=2**12, scale_factor=2, scale_window=1000, min_scale=1)
+    scaler = ps.DynamicLossScaler(**kw)
+    host = [0, 2, 3, 4, 5, 6, 8, 9, 10]
+    h = HybridHarness(11, 256 * 40 + 3, host, scaler, seed=slots, host_keeps_fp16=host_keeps_fp16,
+                      lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
+    h.opt.staging_slots = slots
+    h.fill_state()
+    oc = h.oracle_chunks()
+    oscaler = oracle.ScalerOracle(**kw)
+    oopt = oracle.OptimizerStepOracle(oc, oscaler, lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
+    for step in range(4):
+        h.fill_grads(1e-3, float(oscaler.loss_scale))
+        if step == 1:
+            h.payloads(9)[3][-1] = float("-inf")  # last element of a host-resident position
+        for i, c in enumerate(oc):
+            c["p16"][...] = h.download(i)[3]
+        h.opt.step()
+        torch.cuda.synchronize()
+        oopt.check_overflow()
+        assert oopt.step() is (step == 1)
+        h.compare(oc, what=f"{slots} slots, step {step}")
+    assert h.opt._streamer.n_slots == slots and scaler.loss_scale == oscaler.loss_scale
