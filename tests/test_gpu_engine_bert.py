@@ -54,3 +54,54 @@ def test_engine_trains_a_small_bert():
     assert steps + optimizer.loss_scaler.skipped_steps == 12
     sd = optimizer.state_dict()
     assert len(sd["state"]) == len(list(engine.module.parameters())) and "loss_scaler" in sd
+
+
+def test_bert_base_at_the_reference_chunk_size_matches_the_oracle():
+    """The model of the reference's construction test (unitest/test_optimizer_init.py:47-60: BertConfig() defaults with a
+    small vocabulary, chunk size 32 Mi elements), trained for three iterations through the engine.  After every backward
+    the fp16 chunk payloads hold the gradients; the oracle is stepped on exactly those and every payload must come out
+    bit for bit the same (about 86 M parameters in 3 chunk positions)."""
+    transformers = pytest.importorskip("transformers")
+    import numpy as np
+
+    import oracle
+    from _harness import assert_bits_equal
+
+    cfg = transformers.BertConfig(vocab_size=10, hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0, num_labels=2)
+    torch.manual_seed(0)
+    config = {
+        "optimizer": {"type": "AdamW", "params": {"lr": 1e-4, "betas": (0.9, 0.999), "eps": 1e-8, "weight_decay": 0.01}},
+        "fp16": {"enabled": True, "loss_scale": 0, "initial_scale_power": 12, "loss_scale_window": 1000, "hysteresis": 2, "min_loss_scale": 1},
+        "default_chunk_size": 32 * 1024 * 1024,
+    }
+    engine, optimizer = ps.initialize_engine(
+        model_func=lambda: transformers.BertForSequenceClassification(cfg), local_rank=0, config=config
+    )
+    client = engine.client
+    cl = client.chunk_list
+    pos = client.positions()
+    n_params = sum(p.numel() for p in engine.module.parameters())
+    assert n_params > 80e6 and len(pos) >= 3
+
+    def snap(t):
+        return t.detach().to("cpu", copy=True).numpy()
+
+    mirror = [{"p32": snap(cl[q.fp32].payload), "m": snap(cl[q.exp_avg].payload), "v": snap(cl[q.exp_avg_sq].payload),
+               "p16": snap(cl[q.fp16].payload)} for q in pos]
+    oscaler = oracle.scaler_from_config(config["fp16"])
+    oopt = oracle.OptimizerStepOracle(mirror, oscaler, lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
+    ids = torch.randint(0, 10, (4, 64), device="cuda")
+    labels = torch.randint(0, 2, (4,), device="cuda")
+    for it in range(3):
+        loss = engine(input_ids=ids, labels=labels).loss
+        engine.backward(loss)
+        for q, c in zip(pos, mirror):
+            c["p16"][...] = snap(cl[q.fp16].payload)
+        optimizer.step()
+        oopt.check_overflow()
+        oopt.step()
+        for i, (q, c) in enumerate(zip(pos, mirror)):
+            for key, cid in (("p32", q.fp32), ("m", q.exp_avg), ("v", q.exp_avg_sq), ("p16", q.fp16)):
+                assert_bits_equal(snap(cl[cid].payload), c[key], f"iteration {it} position {i} {key}")
+        assert optimizer.loss_scaler.loss_scale == oscaler.loss_scale
+    assert np.isfinite(float(loss.detach()))
