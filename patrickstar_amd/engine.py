@@ -5,10 +5,10 @@ Only the configuration surface and the optimizer / loss-scaler wiring of
 are kept; the reference's hook-driven chunk movement, memory tracer and
 collectives are not part of this path.  With 288 GB of HBM every chunk stays
 resident: module parameters are fp16 views into the fp16 chunk payloads, so
-forward and backward are ordinary PyTorch, and ``backward`` ends by writing each
-gradient over its parameter's chunk slot while probing it for inf/nan (one
-fused pass per parameter, no host sync), which is the state ``optimizer.step()``
-expects.
+forward and backward are ordinary PyTorch; during ``backward`` each gradient is
+written over its parameter's chunk slot as soon as it is complete, probed for
+inf/nan in the same pass (one fused kernel per parameter, no host sync), which
+is the state ``optimizer.step()`` expects.
 """
 import torch
 
@@ -92,38 +92,62 @@ class PatrickStarEngine(torch.nn.Module):
         )
         self.client.init(self.module, self.optimizer)
         self.iteration_cnt_ = 0
+        self._copied = set()  # parameters whose gradient already sits in its chunk slot (this backward)
+        for p in self.client.chunk_based_param_fp16:
+            if p.requires_grad:
+                p.register_post_accumulate_grad_hook(self._on_gradient_ready)
 
     def forward(self, *inputs, **kwargs):
         return self.module(*inputs, **kwargs)
 
-    def _gradients_to_chunks(self):
-        """Write every gradient over its parameter's fp16 chunk slot, probing for inf/nan on the way."""
-        lib = _lib.load()
+    # -- backward-side producer ---------------------------------------------------------
+    def _gradient_to_chunk(self, p):
+        """Write ``p.grad`` over ``p``'s fp16 chunk slot, probing it for inf/nan in the same pass, and drop it."""
+        g = p.grad if p.grad.is_contiguous() else p.grad.contiguous()
+        if g.dtype not in (torch.half, torch.float):
+            raise TypeError(f"gradient dtype {g.dtype} is not supported")
         scaler = self.loss_scaler
         state_ptr = scaler.state_ptr if isinstance(scaler, DynamicLossScaler) else None
-        stream = _lib.current_stream_handle()
-        for p in self.client.chunk_based_param_fp16:
-            slot = self.client.access_data(p)
-            if p.grad is None:
-                slot.zero_()
-                continue
-            g = p.grad if p.grad.is_contiguous() else p.grad.contiguous()
-            if g.dtype not in (torch.half, torch.float):
-                raise TypeError(f"gradient dtype {g.dtype} is not supported")
+        slot = self.client.access_data(p)
+        with torch.cuda.device(self.client.device):
             _lib.check(
-                lib.ps_grad_to_chunk(g.data_ptr(), int(g.dtype == torch.half), slot.data_ptr(), g.numel(), state_ptr, stream),
+                _lib.load().ps_grad_to_chunk(
+                    g.data_ptr(), int(g.dtype == torch.half), slot.data_ptr(), g.numel(), state_ptr,
+                    _lib.current_stream_handle(),
+                ),
                 "ps_grad_to_chunk",
             )
-            p.grad = None
+        p.grad = None
+
+    def _on_gradient_ready(self, p):
+        """Post-accumulate-grad hook: runs during backward, as soon as ``p``'s gradient is complete (every use of the
+        parameter has been differentiated, so nothing in the rest of backward reads its value any more).  The
+        reference does the same copy in its post-backward module hook (``patrickstar/core/hook.py:200-230``); the
+        copies overlap the rest of backward and no second full set of gradients stays alive."""
+        self._gradient_to_chunk(p)
+        self._copied.add(p)
+
+    def _finish_gradients(self):
+        """After backward: parameters whose hook did not fire (no gradient this iteration, or a gradient that was
+        assigned by hand)."""
+        for p in self.client.chunk_based_param_fp16:
+            if p in self._copied:
+                continue
+            if p.grad is not None:
+                self._gradient_to_chunk(p)
+            else:
+                # the slot still holds the fp16 parameter, which step() would read as a gradient
+                self.client.access_data(p).zero_()
+        self._copied.clear()
 
     def backward(self, loss):
         self.optimizer.zero_grad()
+        self._copied.clear()
         if self.loss_scaler:
             self.loss_scaler.backward(loss)
         else:
             loss.backward()
-        with torch.cuda.device(self.client.device):
-            self._gradients_to_chunks()
+        self._finish_gradients()
         self.iteration_cnt_ += 1
 
 

@@ -204,3 +204,56 @@ def test_hybrid_slot_counts_and_slot_reuse(slots, host_keeps_fp16):
         assert oopt.step() is (step == 1)
         h.compare(oc, what=f"{slots} slots, step {step}")
     assert h.opt._streamer.n_slots == slots and scaler.loss_scale == oscaler.loss_scale
+
+
+class _Tied(torch.nn.Module):
+    """One weight used twice (as embedding and as output projection), one parameter that gets no gradient."""
+
+    def __init__(self):
+        super().__init__()
+        self.emb = torch.nn.Embedding(50, 16)
+        self.mid = torch.nn.Linear(16, 16)
+        self.unused = torch.nn.Parameter(torch.ones(7))
+
+    def forward(self, ids):
+        h = torch.tanh(self.mid(self.emb(ids)))
+        logits = h @ self.emb.weight.t()
+        return logits.float().logsumexp(-1).mean()
+
+
+def test_gradients_reach_their_slots_during_backward():
+    """The copy into the chunk slot runs from a post-accumulate-grad hook.  It must see the COMPLETE gradient of a
+    parameter that is used twice, must not disturb the rest of backward (the slot is the parameter's own storage),
+    must leave no .grad behind, and a parameter without a gradient must present a zero gradient to step()."""
+    torch.manual_seed(0)
+    config = {
+        "optimizer": {"type": "Adam", "params": {"lr": 1e-3, "betas": (0.9, 0.999), "eps": 1e-8, "weight_decay": 0}},
+        "fp16": {"enabled": True, "loss_scale": 64},
+        "default_chunk_size": 4096,
+    }
+    engine, optimizer = ps.initialize_engine(model_func=_Tied, local_rank=0, config=config)
+    client = engine.client
+    ids = torch.randint(0, 50, (8, 5), device="cuda")
+    params = [p for p in engine.module.parameters()]
+    loss = engine(ids)
+    used = [p for p in params if p is not engine.module.unused]
+    expected = torch.autograd.grad(loss * 64, used, retain_graph=True)  # no hooks fire for autograd.grad
+    before = {p: client.access_data(p).clone() for p in params}
+    for p, b in before.items():
+        assert torch.equal(p.data, b)  # the slot IS the parameter
+    engine.backward(loss)
+    torch.cuda.synchronize()
+    assert all(p.grad is None for p in params)
+    for p, g in zip(used, expected):
+        assert g.dtype == torch.half
+        assert torch.equal(client.access_data(p), g), f"slot of {p.ps_attr.name} does not hold its gradient"
+    assert not client.access_data(engine.module.unused).any()
+    # step() turns the slots back into parameters; the model keeps training through the same storage
+    optimizer.step()
+    torch.cuda.synchronize()
+    for p in used:
+        assert not torch.equal(p.data, before[p]) and torch.isfinite(p.data.float()).all()
+    loss2 = engine(ids)
+    engine.backward(loss2)
+    optimizer.step()
+    assert float(loss2.detach()) < float(loss.detach())
