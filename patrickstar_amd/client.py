@@ -237,7 +237,9 @@ class PatrickStarClient:
                 continue
             # every payload starts on a 512-element boundary of its slab (>= 1 KiB for every dtype), so that odd
             # chunk sizes do not push later chunks off the alignment the vector kernels want
-            stride = lambda c: -(-c.capacity // 512) * 512
+            def stride(c):
+                return -(-c.capacity // 512) * 512
+
             slab = torch.zeros(sum(stride(c) for c in chunks), dtype=chunks[0].data_type, device=self.device)
             self._slabs.append(slab)
             cursor = 0

@@ -7,7 +7,7 @@ import torch
 
 import oracle
 import patrickstar_amd as ps
-from _harness import ChunkHarness, HybridHarness, assert_bits_equal
+from _harness import HybridHarness, assert_bits_equal
 
 pytestmark = pytest.mark.gpu
 
