@@ -298,8 +298,50 @@ struct Pipeline {
     bool ready = false;
     hipStream_t h2d = nullptr, compute = nullptr, d2h = nullptr;
     hipEvent_t entry = nullptr;
+    hipEvent_t joined[3] = {};  // one per side stream: "everything queued there so far"
     hipEvent_t h2d_done[kMaxSlots] = {}, compute_done[kMaxSlots] = {}, d2h_done[kMaxSlots] = {};
     bool slot_used[kMaxSlots] = {};
+
+    int create()
+    {
+        // default priority on purpose
+        PS_HIP(hipStreamCreateWithFlags(&h2d, hipStreamNonBlocking));
+        PS_HIP(hipStreamCreateWithFlags(&compute, hipStreamNonBlocking));
+        PS_HIP(hipStreamCreateWithFlags(&d2h, hipStreamNonBlocking));
+        PS_HIP(hipEventCreateWithFlags(&entry, hipEventDisableTiming));
+        for (hipEvent_t& e : joined) PS_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+        for (int i = 0; i < kMaxSlots; ++i) {
+            PS_HIP(hipEventCreateWithFlags(&h2d_done[i], hipEventDisableTiming));
+            PS_HIP(hipEventCreateWithFlags(&compute_done[i], hipEventDisableTiming));
+            PS_HIP(hipEventCreateWithFlags(&d2h_done[i], hipEventDisableTiming));
+        }
+        return 0;
+    }
+
+    // give back whatever a failed create() got as far as making
+    void destroy()
+    {
+        for (hipStream_t* st : {&h2d, &compute, &d2h})
+            if (*st) (void)hipStreamDestroy(*st), *st = nullptr;
+        auto drop = [](hipEvent_t& e) {
+            if (e) (void)hipEventDestroy(e), e = nullptr;
+        };
+        drop(entry);
+        for (hipEvent_t& e : joined) drop(e);
+        for (int i = 0; i < kMaxSlots; ++i) drop(h2d_done[i]), drop(compute_done[i]), drop(d2h_done[i]);
+    }
+
+    // Later work on `caller` comes after everything queued on the side streams so far.  Also used on
+    // an error path, so that a half-queued step cannot race with whatever the caller does next.
+    int join(hipStream_t caller)
+    {
+        hipStream_t side[3] = {h2d, compute, d2h};
+        for (int i = 0; i < 3; ++i) {
+            PS_HIP(hipEventRecord(joined[i], side[i]));
+            PS_HIP(hipStreamWaitEvent(caller, joined[i], 0));
+        }
+        return 0;
+    }
 };
 
 std::mutex g_pipeline_mutex;
@@ -312,15 +354,9 @@ int get_pipeline(Pipeline** out)
     std::lock_guard<std::mutex> lock(g_pipeline_mutex);
     Pipeline& p = g_pipelines[dev];
     if (!p.ready) {
-        // default priority on purpose
-        PS_HIP(hipStreamCreateWithFlags(&p.h2d, hipStreamNonBlocking));
-        PS_HIP(hipStreamCreateWithFlags(&p.compute, hipStreamNonBlocking));
-        PS_HIP(hipStreamCreateWithFlags(&p.d2h, hipStreamNonBlocking));
-        PS_HIP(hipEventCreateWithFlags(&p.entry, hipEventDisableTiming));
-        for (int i = 0; i < kMaxSlots; ++i) {
-            PS_HIP(hipEventCreateWithFlags(&p.h2d_done[i], hipEventDisableTiming));
-            PS_HIP(hipEventCreateWithFlags(&p.compute_done[i], hipEventDisableTiming));
-            PS_HIP(hipEventCreateWithFlags(&p.d2h_done[i], hipEventDisableTiming));
+        if (int rc = p.create()) {
+            p.destroy();
+            return rc;
         }
         p.ready = true;
     }
@@ -616,7 +652,7 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, 
 
     const size_t b32 = chunk_numel * sizeof(float), b16 = chunk_numel * sizeof(uint16_t);
     for (int i = 0; i < kMaxSlots; ++i) p->slot_used[i] = false;
-    for (int k = 0; k < n_host_chunks; ++k) {
+    auto stream_chunk = [&](int k) -> int {
         const int s = k % n_slots;
         const ps_chunk& h = host_chunks[k];
         ps_chunk d = staging[s];
@@ -655,11 +691,12 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, 
         PS_HIP(hipMemcpyAsync(h.exp_avg_sq, d.exp_avg_sq, b32, hipMemcpyDeviceToHost, p->d2h));
         PS_HIP(hipEventRecord(p->d2h_done[s], p->d2h));
         p->slot_used[s] = true;
-    }
-    // later work on the caller's stream sees every chunk written back
-    for (int s = 0; s < n_slots; ++s)
-        if (p->slot_used[s]) PS_HIP(hipStreamWaitEvent(caller, p->d2h_done[s], 0));
-    return 0;
+        return 0;
+    };
+    for (int k = 0; k < n_host_chunks && rc == 0; ++k) rc = stream_chunk(k);
+    // later work on the caller's stream sees every chunk written back (also if queuing stopped half way)
+    const int joined = p->join(caller);
+    return rc ? rc : joined;
 }
 
 int ps_overflow_scan_host_chunks(const ps_chunk* host_chunks, int n_chunks, size_t chunk_numel,
@@ -692,8 +729,7 @@ int ps_overflow_scan_host_chunks(const ps_chunk* host_chunks, int n_chunks, size
     PS_HIP(hipStreamWaitEvent(p->compute, p->entry, 0));
     for (int i = 0; i < kMaxSlots; ++i) p->slot_used[i] = false;
     int streamed = 0;
-    for (int k = 0; k < n_chunks; ++k) {
-        if (fp16_in_hbm[k]) continue;
+    auto stream_chunk = [&](int k) -> int {
         const int s = streamed++ % n_slots;
         if (p->slot_used[s]) PS_HIP(hipStreamWaitEvent(p->h2d, p->compute_done[s], 0));
         PS_HIP(hipMemcpyAsync(staging[s].param_fp16, host_chunks[k].param_fp16, b16,
@@ -705,10 +741,13 @@ int ps_overflow_scan_host_chunks(const ps_chunk* host_chunks, int n_chunks, size
         PS_HIP(hipGetLastError());
         PS_HIP(hipEventRecord(p->compute_done[s], p->compute));
         p->slot_used[s] = true;
-    }
-    for (int s = 0; s < n_slots; ++s)
-        if (p->slot_used[s]) PS_HIP(hipStreamWaitEvent(caller, p->compute_done[s], 0));
-    return 0;
+        return 0;
+    };
+    int rc = 0;
+    for (int k = 0; k < n_chunks && rc == 0; ++k)
+        if (!fp16_in_hbm[k]) rc = stream_chunk(k);
+    const int joined = p->join(caller);
+    return rc ? rc : joined;
 }
 
 int ps_state_init(ps_step_state* d_state, double init_scale, int init_is_int, double scale_factor,
