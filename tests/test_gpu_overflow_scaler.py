@@ -339,3 +339,48 @@ def test_grad_to_chunk_all_alignments_and_probe(src_dtype):
     slot = torch.zeros(6001, dtype=torch.half, device="cuda")
     assert lib.ps_grad_to_chunk(g.data_ptr(), 1, slot[1:].data_ptr(), 6000, None, stream) == 0
     assert torch.equal(slot[1:], g)
+
+
+def test_device_gated_step_replays_from_a_hip_graph():
+    """Scale, overflow flag, step counter and bias corrections live on the device, so the whole dynamic step (probe,
+    gated update, scale update) is a fixed sequence of kernel launches: captured once into a HIP graph, it is replayed
+    for later iterations, clean and poisoned alike.  Every replay is compared with the oracle, with eager work and
+    synchronisation in between."""
+    kw = dict(init_scale=2**10, scale_factor=2, scale_window=3, min_scale=1)
+    scaler = ps.DynamicLossScaler(**kw)
+    h = ChunkHarness(3, 256 * 9 + 7, scaler, seed=77, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
+    h.fill_state()
+    oc = h.oracle_chunks()
+    oscaler = oracle.ScalerOracle(**kw)
+    oopt = oracle.OptimizerStepOracle(oc, oscaler, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
+
+    def one_iteration(run_step, it):
+        h.fill_grads(1e-3, float(oscaler.loss_scale))
+        if it in (2, 5):
+            h.payloads(it % 3)[3][it] = float("inf") if it == 2 else float("nan")
+        for i, c in enumerate(oc):
+            c["p16"][...] = h.download(i)[3]
+        run_step()
+        torch.cuda.synchronize()
+        oopt.check_overflow()
+        assert oopt.step() is (it in (2, 5))
+        h.compare(oc, what=f"iteration {it}")
+        assert scaler.loss_scale == oscaler.loss_scale and type(scaler.loss_scale) is type(oscaler.loss_scale)
+
+    one_iteration(h.opt.step, 0)  # eager: builds the descriptor tables, nothing is allocated afterwards
+    graph = torch.cuda.CUDAGraph()
+    h.fill_grads(1e-3, float(oscaler.loss_scale))
+    for i, c in enumerate(oc):
+        c["p16"][...] = h.download(i)[3]
+    with torch.cuda.graph(graph):
+        h.opt.step()
+    # capture records, it does not run: the state is untouched until the first replay
+    assert scaler.cur_iter == 1
+    graph.replay()
+    torch.cuda.synchronize()
+    oopt.check_overflow()
+    assert oopt.step() is False
+    h.compare(oc, what="first replay")
+    for it in range(2, 9):
+        one_iteration(graph.replay, it)
+    assert scaler.cur_iter == 9 and h.opt.state[h.params[0]]["step"] == 7 == oopt.step_count
