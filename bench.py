@@ -58,10 +58,18 @@ def parse_args():
     return ap.parse_args()
 
 
-def traffic_from_profile():
+PROFILE_OF = {
+    ("static", "operator"): "adam_chunks_config4_pmc.txt",
+    ("dynamic", "operator"): "adam_chunks_gated_config4_dynamic.txt",
+}
+
+
+def traffic_from_profile(mode="static", arithmetic="operator"):
     """HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (calibrated against a copy
     kernel), as recorded in the committed profile summary; None when no such summary exists."""
-    path = os.path.join(ROOT, "profiles", "adam_chunks_config4_pmc.txt")
+    if (mode, arithmetic) not in PROFILE_OF:
+        return None
+    path = os.path.join(ROOT, "profiles", PROFILE_OF[(mode, arithmetic)])
     try:
         m = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", open(path).read(), flags=re.M)
         return float(m.group(1)) if m else None
@@ -387,7 +395,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": traffic_from_profile() if (C, N, args.mode) == (24, N_CHUNK, "static") else None,
+            "traffic": traffic_from_profile(args.mode, args.arithmetic) if (C, N) == (24, N_CHUNK) else None,
             "algorithmic_bytes_per_launch": algorithmic,
             "avg_kernel_ms": avg_kernel_ms,
             "min_kernel_ms": min(kernel_ms),
