@@ -204,3 +204,33 @@ def test_device_bias_corrections_follow_python_pow():
             worst = max(worst, abs(st.bias_correction1_next - bc1) / bc1, abs(st.bias_correction2_next - bc2) / bc2)
             s.update_scale(False)
         assert worst < 4e-16
+
+
+def test_nonfinite_gradients_propagate_like_torch():
+    """A static scaler never skips: inf / nan gradients poison exactly the elements torch's kernels poison (NaN payload
+    bits are not compared, positions and every finite element are), and the subnormal range behaves the same."""
+    lr, betas, eps, wd, scale = 1e-3, (0.9, 0.999), 1e-8, 0.01, 8
+    h = ChunkHarness(2, 256 * 4 + 9, ps.LossScaler(scale), seed=13, lr=lr, betas=betas, eps=eps, weight_decay=wd,
+                     use_adamw=True, arithmetic="torch")
+    h.fill_state()
+    h.fill_grads(1e-3, float(scale))
+    g = h.payloads(0)[3]
+    g[3], g[64], g[300], g[1000] = float("inf"), float("-inf"), float("nan"), 65504.0
+    p, m, v, _ = h.payloads(1)
+    m[:4] = torch.tensor([1e-41, -3e-42, 0.0, 1e-30])
+    v[:4] = torch.tensor([2e-42, 1e-41, 0.0, 1e-35])
+    h.payloads(1)[3][:4] = torch.tensor([6e-8, -6e-8, 0.0, 1e-7]).half()  # subnormal fp16 gradients
+    mirror = TorchMirror(h)
+    mirror.step(1, lr, betas, eps, wd, True, scale)
+    h.opt.step()
+    torch.cuda.synchronize()
+    for i, (tp, tm, tv) in enumerate(mirror.state):
+        for got, want in zip(h.payloads(i)[:3], (tp, tm, tv)):
+            assert torch.equal(torch.isnan(got), torch.isnan(want))
+            ok = ~torch.isnan(want)
+            assert torch.equal(got[ok].view(torch.int32), want[ok].view(torch.int32))
+        hh, th = h.payloads(i)[3], tp.half()
+        assert torch.equal(torch.isnan(hh), torch.isnan(th))
+        ok = ~torch.isnan(th)
+        assert torch.equal(hh[ok].view(torch.int16), th[ok].view(torch.int16))
+    assert torch.isnan(h.payloads(0)[0][300])
