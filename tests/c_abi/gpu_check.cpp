@@ -1,0 +1,221 @@
+// TEST INFRASTRUCTURE.  A program without Python or PyTorch that drives the C ABI of include/ps_adam.h the way a
+// host application written in C or C++ would: device memory from hipMalloc, a stream from hipStreamCreate, chunk
+// descriptors as a plain host array.  Every result is compared bit for bit with the CPU restatement of the
+// reference operator (oracle/adam_oracle.c, linked as liboracle_adam.so) and, for the loss-scale decisions, with
+// the rules of patrickstar/fp16/loss_scaler.py:158-182 written out below.
+//
+// Built by tests/c_abi/Makefile on the CPU (host code only); run by tests/test_c_abi_gpu.py on a GPU.
+#include <hip/hip_runtime_api.h>
+
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "ps_adam.h"
+
+extern "C" {
+// oracle/adam_oracle.c
+struct oracle_adam_opaque {
+    unsigned char bytes[128];
+};
+int oracle_sizeof_state(void);
+void oracle_adam_init(void* o, float lr, float beta1, float beta2, float eps, float weight_decay, int adamw);
+void oracle_adam_advance(void* o, uint64_t step, float beta1, float beta2);
+void oracle_adam_set(void* o, float lr, float eps, float weight_decay, int bias_correction);
+int oracle_adam_span(const void* o, float* p, const void* g, int g_half, float* m, float* v, size_t n,
+                     float loss_scale, int isa);
+void oracle_cast_f32_to_f16(const float* src, uint16_t* dst, size_t n);
+uint16_t oracle_f32_to_f16(float f);
+}
+
+#define HIP_OK(call)                                                                          \
+    do {                                                                                      \
+        hipError_t e_ = (call);                                                               \
+        if (e_ != hipSuccess) {                                                               \
+            fprintf(stderr, "%s failed: %s (line %d)\n", #call, hipGetErrorString(e_), __LINE__); \
+            return 2;                                                                         \
+        }                                                                                     \
+    } while (0)
+#define PS_OK(call)                                                                        \
+    do {                                                                                   \
+        int rc_ = (call);                                                                  \
+        if (rc_ != 0) {                                                                    \
+            fprintf(stderr, "%s returned %d: %s (line %d)\n", #call, rc_, ps_last_error(), __LINE__); \
+            return 3;                                                                      \
+        }                                                                                  \
+    } while (0)
+
+namespace {
+
+struct Lcg {  // deterministic inputs without any library
+    uint64_t s;
+    double uniform() { s = s * 6364136223846793005ull + 1442695040888963407ull; return ((s >> 11) + 0.5) / 9007199254740992.0; }
+    double normal() { return std::sqrt(-2.0 * std::log(uniform())) * std::cos(6.283185307179586 * uniform()); }
+};
+
+struct HostChunk {
+    std::vector<float> p, m, v;
+    std::vector<uint16_t> h;
+};
+
+struct DeviceChunk {
+    float *p = nullptr, *m = nullptr, *v = nullptr;
+    uint16_t* h = nullptr;
+};
+
+int upload(const HostChunk& c, DeviceChunk& d, size_t n)
+{
+    HIP_OK(hipMemcpy(d.p, c.p.data(), n * 4, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(d.m, c.m.data(), n * 4, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(d.v, c.v.data(), n * 4, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(d.h, c.h.data(), n * 2, hipMemcpyHostToDevice));
+    return 0;
+}
+
+int compare(const HostChunk& want, const DeviceChunk& d, size_t n, const char* what, int chunk)
+{
+    std::vector<float> f(n);
+    std::vector<uint16_t> h(n);
+    const float* src[3] = {d.p, d.m, d.v};
+    const std::vector<float>* ref[3] = {&want.p, &want.m, &want.v};
+    const char* name[3] = {"fp32 param", "exp_avg", "exp_avg_sq"};
+    for (int k = 0; k < 3; ++k) {
+        HIP_OK(hipMemcpy(f.data(), src[k], n * 4, hipMemcpyDeviceToHost));
+        if (memcmp(f.data(), ref[k]->data(), n * 4) != 0) {
+            fprintf(stderr, "%s: chunk %d %s differs from the CPU restatement\n", what, chunk, name[k]);
+            return 4;
+        }
+    }
+    HIP_OK(hipMemcpy(h.data(), d.h, n * 2, hipMemcpyDeviceToHost));
+    if (memcmp(h.data(), want.h.data(), n * 2) != 0) {
+        fprintf(stderr, "%s: chunk %d fp16 param differs from the CPU restatement\n", what, chunk);
+        return 4;
+    }
+    return 0;
+}
+
+void new_gradients(Lcg& rng, HostChunk& c, double scale)
+{
+    for (size_t i = 0; i < c.h.size(); ++i) c.h[i] = oracle_f32_to_f16((float)(rng.normal() * 1e-3 * scale));
+}
+
+}  // namespace
+
+int main()
+{
+    int n_dev = 0;
+    HIP_OK(hipGetDeviceCount(&n_dev));
+    if (n_dev < 1) {
+        fprintf(stderr, "no GPU\n");
+        return 77;
+    }
+    HIP_OK(hipSetDevice(0));
+    hipStream_t stream;
+    HIP_OK(hipStreamCreate(&stream));
+
+    const int C = 3;
+    const size_t n = 256 * 13 + 5;  // whole tiles and a ragged one
+    const float lr = 1e-4f, b1 = 0.9f, b2 = 0.999f, eps = 1e-8f, wd = 0.01f;
+    Lcg rng{12345};
+    std::vector<HostChunk> host(C);
+    std::vector<DeviceChunk> dev(C);
+    ps_chunk table[C];
+    for (int c = 0; c < C; ++c) {
+        HostChunk& hc = host[c];
+        hc.p.resize(n), hc.m.resize(n), hc.v.resize(n), hc.h.resize(n);
+        for (size_t i = 0; i < n; ++i) {
+            hc.p[i] = (float)(rng.normal() * 0.02);
+            hc.m[i] = (float)(rng.normal() * 1e-4);
+            hc.v[i] = (float)std::fabs(rng.normal() * 1e-6);
+        }
+        HIP_OK(hipMalloc((void**)&dev[c].p, n * 4));
+        HIP_OK(hipMalloc((void**)&dev[c].m, n * 4));
+        HIP_OK(hipMalloc((void**)&dev[c].v, n * 4));
+        HIP_OK(hipMalloc((void**)&dev[c].h, n * 2));
+        table[c].param_fp32 = dev[c].p;
+        table[c].exp_avg = dev[c].m;
+        table[c].exp_avg_sq = dev[c].v;
+        table[c].param_fp16 = dev[c].h;
+    }
+    if (oracle_sizeof_state() > (int)sizeof(oracle_adam_opaque)) return 5;
+    oracle_adam_opaque native;
+    oracle_adam_init(&native, lr, b1, b2, eps, wd, 1);
+    PS_OK(ps_adam_create(31, lr, b1, b2, eps, wd, 1, 0));
+
+    // ---- host-decided steps with a static scale: t = 100 (cold), then 101 and 102 (running products)
+    const double scale = 4096.0;
+    for (uint64_t step = 100; step < 103; ++step) {
+        for (int c = 0; c < C; ++c) {
+            new_gradients(rng, host[c], scale);
+            if (upload(host[c], dev[c], n)) return 2;
+        }
+        PS_OK(ps_adam_step_chunks(31, step, lr, b1, b2, eps, wd, 1, table, C, n, scale, stream));
+        HIP_OK(hipStreamSynchronize(stream));
+        oracle_adam_advance(&native, step, b1, b2);
+        oracle_adam_set(&native, lr, eps, wd, 1);
+        for (int c = 0; c < C; ++c) {
+            if (oracle_adam_span(&native, host[c].p.data(), host[c].h.data(), 1, host[c].m.data(), host[c].v.data(),
+                                 n, (float)scale, 0) <= 0)
+                return 5;
+            oracle_cast_f32_to_f16(host[c].p.data(), host[c].h.data(), n);
+            if (int rc = compare(host[c], dev[c], n, "static step", c)) return rc;
+        }
+    }
+
+    // ---- device-decided steps: probe, gated update, scale update; nothing is read back until the end
+    ps_step_state* d_state = nullptr;
+    HIP_OK(hipMalloc((void**)&d_state, sizeof(ps_step_state)));
+    PS_OK(ps_state_init(d_state, 1024.0, 1, 2.0, 1, 3, 1.0, 1, 1, 0, b1, b2, stream));
+    PS_OK(ps_adam_create(32, lr, b1, b2, eps, wd, 1, 0));
+    oracle_adam_init(&native, lr, b1, b2, eps, wd, 1);
+    double cur_scale = 1024.0;  // loss_scaler.py:158-182 with delayed_shift = 1
+    int64_t cur_iter = 0, last_overflow = -1, adam_step = 0;
+    for (int it = 0; it < 8; ++it) {
+        const bool poison = it == 2 || it == 5;
+        for (int c = 0; c < C; ++c) {
+            new_gradients(rng, host[c], cur_scale);
+            if (poison && c == it % C) host[c].h[n - 1] = 0x7C00;  // +inf in the last element
+            if (upload(host[c], dev[c], n)) return 2;
+        }
+        PS_OK(ps_overflow_scan_chunks(table, C, n, d_state, stream));
+        PS_OK(ps_adam_step_chunks_gated(32, lr, eps, wd, 1, table, C, n, d_state, stream));
+        PS_OK(ps_scaler_update(d_state, PS_FLAG_FROM_DEVICE, NULL, 0, stream));
+        HIP_OK(hipStreamSynchronize(stream));
+        if (poison) {
+            for (int c = 0; c < C; ++c) oracle_cast_f32_to_f16(host[c].p.data(), host[c].h.data(), n);
+            cur_scale = cur_scale / 2.0 > 1.0 ? cur_scale / 2.0 : 1.0;
+            last_overflow = cur_iter;
+        } else {
+            adam_step += 1;
+            oracle_adam_advance(&native, (uint64_t)adam_step, b1, b2);
+            oracle_adam_set(&native, lr, eps, wd, 1);
+            for (int c = 0; c < C; ++c) {
+                if (oracle_adam_span(&native, host[c].p.data(), host[c].h.data(), 1, host[c].m.data(),
+                                     host[c].v.data(), n, (float)cur_scale, 0) <= 0)
+                    return 5;
+                oracle_cast_f32_to_f16(host[c].p.data(), host[c].h.data(), n);
+            }
+            if ((cur_iter - last_overflow) % 3 == 0) cur_scale *= 2.0;
+        }
+        cur_iter += 1;
+        for (int c = 0; c < C; ++c)
+            if (int rc = compare(host[c], dev[c], n, poison ? "skipped step" : "gated step", c)) return rc;
+    }
+    ps_step_state st;
+    PS_OK(ps_state_read(d_state, &st, stream));
+    if (st.cur_scale != cur_scale || st.cur_iter != cur_iter || st.adam_step != adam_step || st.skipped_steps != 2 ||
+        st.overflow != 0) {
+        fprintf(stderr, "step state: scale %g (want %g) iter %lld (%lld) step %lld (%lld) skipped %lld\n", st.cur_scale,
+                cur_scale, (long long)st.cur_iter, (long long)cur_iter, (long long)st.adam_step, (long long)adam_step,
+                (long long)st.skipped_steps);
+        return 6;
+    }
+    PS_OK(ps_adam_destroy(31));
+    PS_OK(ps_adam_destroy(32));
+    printf("c abi gpu check ok: 3 host-decided and 8 device-decided steps (2 skipped) over %d x %zu elements, loss scale %g\n",
+           C, n, st.cur_scale);
+    return 0;
+}
