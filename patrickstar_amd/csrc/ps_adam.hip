@@ -498,8 +498,9 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
 
     // Tensors handed to the operator are views at one element offset into the four chunk
     // payloads, so their addresses normally share a phase relative to 16-byte (4-element)
-    // boundaries: peel up to 3 leading elements, run whole 256-element tiles with vector
-    // accesses, finish the remainder element-wise.
+    // boundaries: whole 256-element tiles with vector accesses from the first aligned element on;
+    // the up to 3 elements before it and the remainder behind the last tile go element-wise, in
+    // the same launch.
     auto elem_phase = [](const void* a, size_t elem_size) -> int {
         uintptr_t u = reinterpret_cast<uintptr_t>(a);
         if (u % elem_size) return -1;
@@ -514,14 +515,13 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
     } else {
         const size_t head = (size_t)((4 - ph) & 3);
         const size_t n_tiles = (numel - head) / 256;
-        const size_t body_end = head + n_tiles * 256;
-        scalar_span(0, head);
-        dim3 grid(grid_1d(n_tiles)), block(64);
+        const int tail = (int)(numel - head - n_tiles * 256);
+        dim3 grid(grid_1d(n_tiles + 1)), block(64);  // + 1: the workgroup that does head and tail
         uint16_t* out = d_param_fp16_out ? d_param_fp16_out + head : nullptr;
 #define PS_FLAT_VEC(WD, HALF)                                                                     \
     hipLaunchKernelGGL((adam_flat_vec_kernel<WD, HALF>), grid, block, kLdsBytes, s, c,            \
                        d_params + head, static_cast<const void*>(gbytes + head * gsz),            \
-                       d_exp_avg + head, d_exp_avg_sq + head, out, n_tiles)
+                       d_exp_avg + head, d_exp_avg_sq + head, out, n_tiles, (int)head, tail)
         if (grads_are_half) {
             if (c.wd_mode == WD_DECOUPLED) PS_FLAT_VEC(WD_DECOUPLED, true);
             else if (c.wd_mode == WD_L2) PS_FLAT_VEC(WD_L2, true);
@@ -532,7 +532,6 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
             else PS_FLAT_VEC(WD_NONE, false);
         }
 #undef PS_FLAT_VEC
-        scalar_span(body_end, numel);
     }
     PS_HIP(hipGetLastError());
     return 0;

@@ -109,14 +109,46 @@ __global__ void __launch_bounds__(kAuxBlock)
 
 // The same operator on a span whose four (five) addresses share one 16-byte phase: single-wave
 // workgroups over 256-element tiles with 16-byte accesses, resident-workgroup cap as for the chunk
-// kernels.  Gradients are read only; the fp16 output is optional.
+// kernels.  Gradients are read only; the fp16 output is optional.  The pointers are those of the
+// first 16-byte aligned element; the up to 3 elements in front of it (`head`) and the up to 255
+// behind the last whole tile (`tail`) are done element-wise by one extra workgroup of the same launch.
+template <int WD, int UNS, bool GRAD_HALF>
+__device__ __forceinline__ void flat_tile_math(const StepConsts& c, const float (&g)[4], float4v& p, float4v& m,
+                                               float4v& v, uint32_t (&h)[4])
+{
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        float pe = p[e], me = m[e], ve = v[e];
+        adam_element<PS_ARITH_OPERATOR, WD, UNS>(c, g[e], pe, me, ve);
+        p[e] = pe;
+        m[e] = me;
+        v[e] = ve;
+        h[e] = float_to_half_bits(pe);
+    }
+}
+
 template <int WD, bool GRAD_HALF>
 __global__ void __launch_bounds__(64)
     adam_flat_vec_kernel(StepConsts c, float* p32, const void* grads, float* m32, float* v32,
                          uint16_t* out16,  // may alias grads (fp16 gradients overwritten by fp16 parameters)
-                         size_t n_tiles)
+                         size_t n_tiles, int head, int tail)
 {
-    for (size_t t = blockIdx.x; t < n_tiles; t += gridDim.x) {
+    // one tile per workgroup, like the chunk-list kernels; the loop only matters beyond 2^31 tiles
+    for (size_t t = blockIdx.x; t <= n_tiles; t += gridDim.x) {
+        if (t == n_tiles) {
+            for (int j = threadIdx.x; j < head + tail; j += 64) {
+                const ptrdiff_t i = j < head ? (ptrdiff_t)j - head : (ptrdiff_t)(n_tiles * 256) + (j - head);
+                float g = GRAD_HALF ? half_bits_to_float(static_cast<const uint16_t*>(grads)[i])
+                                    : static_cast<const float*>(grads)[i];
+                float p = p32[i], m = m32[i], v = v32[i];
+                element_any<PS_ARITH_OPERATOR, WD, UNSCALE_RUNTIME>(c, g, p, m, v);
+                p32[i] = p;
+                m32[i] = m;
+                v32[i] = v;
+                if (out16) out16[i] = (uint16_t)float_to_half_bits(p);
+            }
+            break;
+        }
         const size_t i = (t * 64 + threadIdx.x) * 4;
         float g[4];
         if (GRAD_HALF) {
@@ -132,15 +164,13 @@ __global__ void __launch_bounds__(64)
         }
         float4v p = ld_f4(p32 + i), m = ld_f4(m32 + i), v = ld_f4(v32 + i);
         uint32_t h[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            float pe = p[e], me = m[e], ve = v[e];
-            element_any<PS_ARITH_OPERATOR, WD, UNSCALE_RUNTIME>(c, g[e], pe, me, ve);
-            p[e] = pe;
-            m[e] = me;
-            v[e] = ve;
-            h[e] = float_to_half_bits(pe);
-        }
+        // the unscale form is uniform: branch once around the arithmetic, not per element
+        if (c.unscale == UNSCALE_MUL)
+            flat_tile_math<WD, UNSCALE_MUL, GRAD_HALF>(c, g, p, m, v, h);
+        else if (c.unscale == UNSCALE_DIV)
+            flat_tile_math<WD, UNSCALE_DIV, GRAD_HALF>(c, g, p, m, v, h);
+        else
+            flat_tile_math<WD, UNSCALE_NONE, GRAD_HALF>(c, g, p, m, v, h);
         st_f4(p32 + i, p);
         st_f4(m32 + i, m);
         st_f4(v32 + i, v);
