@@ -305,3 +305,42 @@ def test_build_entry_point_compiles_and_loads():
                        text=True, timeout=600)
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
     assert "built" in r.stdout and os.path.exists(_lib.LIB_PATH)
+
+
+def test_chunk_tensor_index_known_answers_of_the_reference_test():
+    """The expectations of unitest/test_chunk_tensor_index.py:82-170: which of 10, 20, 30, 20, 7, 2 fit into a
+    20-element chunk, and the insert / delete / insert sequence on tensor lists (7, 2 | 6, 5 | delete 6 | 8 | 7 | 1, 2, 3)."""
+    idx = ChunkTensorIndex(20)
+    fits = [idx.try_insert_tensor(0, _param(n, f"param_{i}"), AccessType.DATA) for i, n in enumerate([10, 20, 30, 20, 7, 2])]
+    assert fits == [True, False, False, False, True, True]
+    offsets = [i.start_offset for i in idx.generate_tensor_info_in_order(0)]
+    assert offsets == sorted(offsets) == [0, 10, 17]
+
+    idx = ChunkTensorIndex(20)
+    first = [_param(7, "a"), _param(2, "b")]
+    assert idx.try_insert_tensor_list(0, first, AccessType.DATA)
+    second = [_param(6, "c"), _param(5, "d")]
+    assert idx.try_insert_tensor_list(0, second, AccessType.DATA)  # 7, 2, 6, 5
+    idx.delete_tensor(0, second[0], AccessType.DATA)  # 7, 2, (6), 5
+    assert not idx.try_insert_tensor_list(0, [_param(8, "e")], AccessType.DATA)
+    assert not idx.try_insert_tensor_list(0, [_param(7, "f")], AccessType.DATA)
+    assert idx.try_insert_tensor_list(0, [_param(1, "g"), _param(2, "h"), _param(3, "i")], AccessType.DATA)
+    assert [(t.start_offset, t.numel) for t in idx.generate_tensor_info_in_order(0)] == [(0, 7), (7, 2), (9, 1), (10, 2), (12, 3), (15, 5)]
+
+
+def test_optimizer_state_chunk_map_known_answer():
+    """unitest/test_chunk_tensor_index.py:172-213: two fp16 chunks (10, 5) and (6, 9); the momentum chunk of the first
+    is unknown until registered, then it is the registered id for every parameter of that fp16 chunk only."""
+    idx = ChunkTensorIndex(20)
+    params = []
+    for chunk_id, sizes in ((0, (10, 5)), (1, (6, 9))):
+        for n in sizes:
+            p = _param(n, f"param_{n}")
+            assert idx.try_insert_tensor(chunk_id, p, AccessType.DATA)
+            params.append(p)
+    assert idx.get_optimizer_state_chunk_id(params[0], AccessType.DATA, ChunkType.MOMENTUM) is None
+    idx.register_optimizer_state_chunk_id(params[0], AccessType.DATA, ChunkType.MOMENTUM, 3)
+    assert idx.get_optimizer_state_chunk_id(params[0], AccessType.DATA, ChunkType.MOMENTUM) == 3
+    assert idx.get_optimizer_state_chunk_id(params[1], AccessType.DATA, ChunkType.MOMENTUM) == 3
+    assert idx.get_optimizer_state_chunk_id(params[2], AccessType.DATA, ChunkType.MOMENTUM) is None
+    assert idx.get_optimizer_state_chunk_id(params[0], AccessType.DATA, ChunkType.VARIANCE) is None
