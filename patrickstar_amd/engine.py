@@ -13,6 +13,7 @@ is the state ``optimizer.step()`` expects.
 import torch
 
 from . import _lib
+from .chunk_layout import is_param_registered
 from .client import PatrickStarClient
 from .fp16_adam import FP16Adam
 from .loss_scaler import DynamicLossScaler, LossScaler
@@ -149,6 +150,46 @@ class PatrickStarEngine(torch.nn.Module):
             loss.backward()
         self._finish_gradients()
         self.iteration_cnt_ += 1
+
+
+    # -- model checkpoint -------------------------------------------------------------------
+    def state_dict(self, destination=None, prefix="", keep_vars=False):
+        """The model's checkpoint under the module's own parameter names, as the reference writes it
+        (``patrickstar/runtime/checkpoint.py:39-88``): for every chunk-based parameter the fp32 MASTER copy (which
+        is what training continues from), not the fp16 working copy; buffers as they are.  Values are CPU clones."""
+        out = self.module.state_dict(prefix=prefix, keep_vars=False) if destination is None else destination
+        if destination is not None:
+            self.module.state_dict(destination=out, prefix=prefix, keep_vars=False)
+        for key in list(out.keys()):
+            out[key] = out[key].detach().to("cpu", copy=True)
+        for name, p in self.module.named_parameters():
+            if is_param_registered(p) and p in self.client.param_fp16_to_param_fp32_map:
+                master = self.client.access_data(self.client.param_fp16_to_param_fp32_map[p])
+                out[prefix + name] = master.detach().to("cpu", copy=True)
+        return out
+
+    def load_state_dict(self, state_dict, strict=False):
+        """Load a checkpoint written by ``state_dict``: fp32 masters are restored and the fp16 working copies are
+        refreshed from them (round to nearest even); buffers go through ``nn.Module``.  ``strict`` raises on missing
+        or unexpected keys, as ``patrickstar/runtime/checkpoint.py:198-262`` does."""
+        named = dict(self.module.named_parameters())
+        rest = {}
+        missing = [k for k in named if k not in state_dict]
+        with torch.no_grad():
+            for key, value in state_dict.items():
+                p = named.get(key)
+                if p is not None and is_param_registered(p) and p in self.client.param_fp16_to_param_fp32_map:
+                    master = self.client.access_data(self.client.param_fp16_to_param_fp32_map[p])
+                    master.copy_(value.to(master.device, torch.float).view(master.shape))
+                    self.client.access_data(p).copy_(master)
+                else:
+                    rest[key] = value
+        result = self.module.load_state_dict(rest, strict=False)
+        unexpected = list(result.unexpected_keys)
+        missing += [k for k in result.missing_keys if k not in named]
+        if strict and (unexpected or missing):
+            raise RuntimeError(f"Failed to load model strictly. missing: {missing} unexpected: {unexpected}")
+        return result
 
 
 def initialize_engine(model_func, local_rank, config=None, client=None):

@@ -105,3 +105,64 @@ def test_bert_base_at_the_reference_chunk_size_matches_the_oracle():
                 assert_bits_equal(snap(cl[cid].payload), c[key], f"iteration {it} position {i} {key}")
         assert optimizer.loss_scaler.loss_scale == oscaler.loss_scale
     assert np.isfinite(float(loss.detach()))
+
+
+def test_checkpoint_reload_reproduces_the_losses_exactly():
+    """The reference's checkpoint test (unitest/test_checkpoint.py:95-181) on a small BERT: train 5 steps, save model and
+    optimizer, train 5 more on recorded batches, reload, and require (a) the loss right after reloading to EQUAL the
+    loss at the save point and (b) the loss after re-training on the same 5 batches to EQUAL the loss of the first
+    run.  Both need the fp32 masters, m, v, the step counter and the loss-scaler state to come back bit for bit."""
+    transformers = pytest.importorskip("transformers")
+    cfg = transformers.BertConfig(
+        vocab_size=256, hidden_size=64, num_hidden_layers=2, num_attention_heads=4, intermediate_size=128,
+        max_position_embeddings=64, num_labels=2, hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0,
+    )
+    torch.manual_seed(0)
+    config = {
+        "optimizer": {"type": "Adam", "params": {"lr": 1e-3, "betas": (0.9, 0.999), "eps": 1e-6, "weight_decay": 0, "use_hybrid_adam": True}},
+        "fp16": {"enabled": True, "loss_scale": 0, "initial_scale_power": 10, "loss_scale_window": 4, "hysteresis": 2, "min_loss_scale": 1},
+        "default_chunk_size": 32 * 1024,
+    }
+    model, optimizer = ps.initialize_engine(
+        model_func=lambda: transformers.BertForSequenceClassification(cfg), local_rank=0, config=config
+    )
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1)
+
+    def batch():
+        return (torch.randint(0, 256, (4, 32), device="cuda", generator=gen), torch.randint(0, 2, (4,), device="cuda", generator=gen))
+
+    def train_one_step(b):
+        loss = model(input_ids=b[0], labels=b[1])[0]
+        model.backward(loss)
+        optimizer.step()
+
+    def evaluate(b):
+        model.eval()
+        with torch.no_grad():
+            out = model(input_ids=b[0], labels=b[1])[0].item()
+        model.train()
+        return out
+
+    batch0 = batch()
+    for _ in range(5):
+        train_one_step(batch())
+    loss0 = evaluate(batch0)
+    model_sd = model.state_dict()
+    opt_sd = optimizer.state_dict()
+    assert all(v.dtype == torch.float for k, v in model_sd.items() if "weight" in k or "bias" in k)  # the masters
+    later = [batch() for _ in range(5)]
+    for b in later:
+        train_one_step(b)
+    loss1 = evaluate(batch0)
+    assert loss1 != loss0
+    model.load_state_dict(model_sd)
+    optimizer.load_state_dict(opt_sd)
+    loss2 = evaluate(batch0)
+    assert loss0 == loss2, f"Model checkpoint error. {loss0} vs {loss2}"
+    for b in later:
+        train_one_step(b)
+    loss3 = evaluate(batch0)
+    assert loss1 == loss3, f"Optimizer checkpoint error. {loss1} vs {loss3}"
+    with pytest.raises(RuntimeError, match="strictly"):
+        model.load_state_dict({"no.such.key": torch.zeros(1)}, strict=True)
