@@ -201,7 +201,8 @@ class PatrickStarClient:
             return chunk_id
         if ctype == ChunkType.PARAM_FP32:
             ids32 = self.chunk_tensor_index.chunk_type_to_chunk_id_list_map[ChunkType.PARAM_FP32]
-            return ids16[ids32.index(chunk_id)]
+            pos = ids32.index(chunk_id)
+            return ids16[pos] if pos < len(ids16) else None  # an fp32 list driven on its own has no fp16 twin
         for ref_id, os_map in self.chunk_tensor_index.param_chunk_id_to_os_chunk_id_map.items():
             if os_map.get(ctype) == chunk_id:
                 return ref_id
@@ -225,7 +226,7 @@ class PatrickStarClient:
         for chunk_id, chunk in self.chunk_list.generate_chunk():
             if chunk.payload is not None:
                 continue
-            on_host = self._fp16_chunk_of_position(chunk_id) in self.host_fp16_chunk_ids
+            on_host = bool(self.host_fp16_chunk_ids) and self._fp16_chunk_of_position(chunk_id) in self.host_fp16_chunk_ids
             if on_host and (self.host_keeps_fp16 or chunk.chunk_type != ChunkType.PARAM_FP16):
                 chunk.allocate_payload("cpu", pin_memory=True)
             else:
@@ -273,7 +274,10 @@ class PatrickStarClient:
         info = self.chunk_tensor_index.get_tensor_info(param.ps_attr.data_id())
         payload = self.chunk_list[info.chunk_id].payload
         if payload is None:
-            raise RuntimeError(f"chunk {info.chunk_id} has no payload; call allocate_payloads() first")
+            # first access: give every chunk that has none its (zero-filled) payload, as the reference does
+            # on the first access of a chunk (patrickstar/core/client.py:350-420)
+            self.allocate_payloads()
+            payload = self.chunk_list[info.chunk_id].payload
         view = payload.narrow(0, info.start_offset, info.numel).view(param.ps_attr.shape)
         if device is not None and torch.device(device).type != view.device.type:
             # a copy would silently detach the caller from the chunk

@@ -344,3 +344,24 @@ def test_optimizer_state_chunk_map_known_answer():
     assert idx.get_optimizer_state_chunk_id(params[1], AccessType.DATA, ChunkType.MOMENTUM) == 3
     assert idx.get_optimizer_state_chunk_id(params[2], AccessType.DATA, ChunkType.MOMENTUM) is None
     assert idx.get_optimizer_state_chunk_id(params[0], AccessType.DATA, ChunkType.VARIANCE) is None
+
+
+def test_client_append_and_access_known_answer():
+    """unitest/test_client.py:45-78: tensors of 10, 11, 12, 13 elements appended one by one to 40-element chunks
+    (the fourth opens a second chunk), written through access_data and read back later."""
+    client = ps.PatrickStarClient(rank=0, default_chunk_size=40, device="cpu")
+    params, refs = [], []
+    for i, n in enumerate([10, 11, 12, 13]):
+        param = torch.nn.Parameter(torch.rand(n))
+        refs.append(param.data.clone())
+        register_param(param, ParamType.CHUNK_BASED, torch.float, f"param_{i}")
+        client.append_tensor([param], torch.float, AccessType.DATA, ChunkType.PARAM_FP32)
+        client.access_data(param, torch.device("cpu:0")).copy_(param.data)
+        client.release_data(param)
+        params.append(param)
+    idx = client.chunk_tensor_index
+    infos = [idx.get_tensor_info(p.ps_attr.data_id()) for p in params]
+    assert [(t.chunk_id, t.start_offset) for t in infos] == [(0, 0), (0, 10), (0, 21), (1, 0)]
+    for param, ref in zip(params, refs):
+        assert torch.max(client.access_data(param, torch.device("cpu:0")) - ref) == 0
+        client.release_data(param)
