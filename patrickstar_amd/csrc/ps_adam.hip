@@ -13,19 +13,27 @@
 //     for writing, and HBM efficiency drops when the set of in-flight cache
 //     lines gets wide; a narrow, steadily advancing window per array gave
 //     6.3 TB/s where the fully occupied machine gave 5.3 TB/s (a plain
-//     1-read-1-write copy peaks at 6.2-6.3 TB/s on the same GPU);
+//     1-read-1-write copy peaks at 6.3-6.4 TB/s on the same GPU);
 //   * chunk descriptors travel in the kernel-argument segment (64 per launch),
 //     so a wave's first data load depends on one scalar load, not two;
 //   * plain (temporal) loads/stores: non-temporal loads cost 6 % at this
 //     operating point (20-25 % with fully occupied CUs), non-temporal stores
 //     change nothing.
 //
-// Arithmetic contract (bit-exact with the explicit-intrinsic body of the
-// reference operator, patrickstar/ops/csrc/adam/cpu_adam.cpp:91-141): every
-// a*b+c the reference writes as SIMD_FMA is one __builtin_fmaf; every other
-// operation is an individually rounded IEEE binary32 op.  The file must be
-// compiled with -ffp-contract=off and with correctly rounded fp32 divide and
-// sqrt (hipcc's default), denormals preserved.
+// Arithmetic contract (ps_arith.h).  Operator arithmetic: bit-exact with the
+// explicit-intrinsic body of the reference operator
+// (patrickstar/ops/csrc/adam/cpu_adam.cpp:91-141): every a*b+c the reference
+// writes as SIMD_FMA is one __builtin_fmaf; every other operation is an
+// individually rounded IEEE binary32 op.  Torch arithmetic: one rounding step
+// per torch kernel of FP16Adam.torch_adam_update
+// (patrickstar/ops/fp16_cpu_adam.py:259-277), as torch's GPU kernels round.
+// Everything must be compiled with -ffp-contract=off and with correctly rounded
+// fp32 divide and sqrt (hipcc's default), denormals preserved.
+//
+// Layout of the sources: ps_config.h (tuning knobs), ps_arith.h (step constants
+// and per-element arithmetic), ps_tile.h (vector accesses, one tile per wave),
+// ps_kernels.h (the kernels), this file (host state, launches, streaming of
+// host-resident chunks, the C ABI).
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 
