@@ -521,3 +521,59 @@ def test_chunk_step_with_unaligned_payload_bases(offsets):
         assert_bits_equal(d[0].cpu().numpy()[:op], p[:op], "before")
         assert_bits_equal(d[0].cpu().numpy()[op + n:], p[op + n:], "after")
         assert_bits_equal(d[3].cpu().numpy()[oh + n:], g[oh + n:], "after fp16")
+
+
+def test_randomised_shapes_hyperparameters_and_arithmetics():
+    """Forty seeded random cases through ps_adam_step_chunks: list length, chunk length (down to one element),
+    per-list base misalignment, step number, betas, decay form, scale kind and arithmetic all vary.  Each case is one
+    cold step compared bit for bit with the matching CPU restatement."""
+    lib = _lib.load()
+    rng = np.random.default_rng(20240612)
+    for case in range(40):
+        C = int(rng.integers(1, 6))
+        n = int(rng.choice([1, 3, 64, 255, 256, 257, 1000, int(rng.integers(300, 3000))]))
+        offs = [int(o) for o in (rng.integers(0, 4, 4) if rng.random() < 0.5 else np.zeros(4, int))]
+        offs[3] *= 2  # keep the fp16 list's phase comparable now and then
+        step = int(rng.choice([1, 2, 17, 100, 5000]))
+        b1, b2 = float(rng.choice([0.9, 0.8, 0.95])), float(rng.choice([0.999, 0.98, 0.95]))
+        lr, eps = float(rng.choice([1e-3, 1e-4, 3e-5])), float(rng.choice([1e-8, 1e-6]))
+        wd = float(rng.choice([0.0, 0.01, 0.1]))
+        adamw = bool(rng.integers(0, 2))
+        scale = [None, 8, 2**12, 2**16, 1000.0, 12345.678][int(rng.integers(0, 6))]
+        torch_arith = bool(rng.integers(0, 2))
+        what = f"case {case}: C={C} n={n} offs={offs} step={step} betas=({b1},{b2}) lr={lr} eps={eps} wd={wd} adamw={adamw} scale={scale} torch={torch_arith}"
+        host, dev, rows = [], [], []
+        for _ in range(C):
+            p = rng.normal(0, 0.02, n + 16).astype(np.float32)
+            m = rng.normal(0, 1e-4, n + 16).astype(np.float32)
+            v = np.abs(rng.normal(0, 1e-6, n + 16)).astype(np.float32)
+            g = (rng.normal(0, 1e-3, n + 16) * (scale or 1.0)).astype(np.float16)
+            host.append((p, m, v, g))
+            d = tuple(_dev(x.copy()) for x in (p, m, v, g))
+            dev.append(d)
+            rows.append([d[k][offs[k]:].data_ptr() for k in range(4)])
+        oid = 3000 + case
+        _lib.check(lib.ps_adam_create(oid, lr, b1, b2, eps, wd, int(adamw), 0), "create")
+        if torch_arith:
+            _lib.check(lib.ps_adam_set_arithmetic(oid, _lib.PS_ARITH_TORCH), "set_arithmetic")
+        _lib.check(
+            lib.ps_adam_step_chunks(oid, step, lr, b1, b2, eps, wd, 1, _lib.chunk_array(rows), C, n,
+                                    float(scale) if scale is not None else -1.0, _lib.current_stream_handle()),
+            what,
+        )
+        torch.cuda.synchronize()
+        lib.ps_adam_destroy(oid)
+        for (p, m, v, g), d in zip(host, dev):
+            po, mo, vo, go = (np.ascontiguousarray(x[o:o + n]) for x, o in zip((p, m, v, g), offs))
+            if torch_arith:
+                oracle.torch_formula_update(po, go, mo, vo, step, lr, b1, b2, eps, wd, adamw, scale)
+            else:
+                oracle.AdamOracle(lr, b1, b2, eps, wd, adamw).update(
+                    step, lr, b1, b2, eps, wd, True, po, go, mo, vo, float(scale) if scale is not None else -1.0)
+            for k, (want, name) in enumerate(((po, "param"), (mo, "exp_avg"), (vo, "exp_avg_sq"), (oracle.cast_fp32_to_fp16(po), "fp16"))):
+                got = d[k].cpu().numpy()
+                assert_bits_equal(got[offs[k]:offs[k] + n], want, f"{what} {name}")
+                # nothing outside the view was touched
+                src = (p, m, v, g)[k]
+                assert_bits_equal(got[:offs[k]], src[:offs[k]], f"{what} {name} before")
+                assert_bits_equal(got[offs[k] + n:], src[offs[k] + n:], f"{what} {name} after")
