@@ -27,6 +27,7 @@ HIPCC_FLAGS = [
     "-Xclang",
     "-packed-fp32-ops",
     "-Wall",
+    "-Wextra",
     "-Wno-unused-function",
 ]
 
