@@ -1,6 +1,6 @@
 // TEST INFRASTRUCTURE.  A program without Python or PyTorch that drives the C ABI of include/ps_adam.h the way a
 // host application written in C or C++ would: device memory from hipMalloc, a stream from hipStreamCreate, chunk
-// descriptors as a plain host array.  Every result is compared bit for bit with the CPU restatement of the
+// descriptors as a plain host array, pinned host memory from hipHostMalloc for host-resident chunks.  Every result is compared bit for bit with the CPU restatement of the
 // reference operator (oracle/adam_oracle.c, linked as liboracle_adam.so) and, for the loss-scale decisions, with
 // the rules of patrickstar/fp16/loss_scaler.py:158-182 written out below.
 //
@@ -215,7 +215,88 @@ int main()
     }
     PS_OK(ps_adam_destroy(31));
     PS_OK(ps_adam_destroy(32));
-    printf("c abi gpu check ok: 3 host-decided and 8 device-decided steps (2 skipped) over %d x %zu elements, loss scale %g\n",
-           C, n, st.cur_scale);
+
+    // ---- host-resident chunk positions: fp32 param / m / v in pinned host memory, streamed through two staging
+    //      slots; position 0 stays resident, position 1 keeps its fp16 payload in HBM, position 2 has it on the host
+    struct PinnedChunk {
+        float *p = nullptr, *m = nullptr, *v = nullptr;
+        uint16_t* h = nullptr;  // pinned host memory, or NULL when the fp16 payload stays in HBM
+    };
+    PinnedChunk pinned[C];
+    ps_chunk host_table[2], staging[2];
+    for (int c = 1; c < C; ++c) {
+        HIP_OK(hipHostMalloc((void**)&pinned[c].p, n * 4, hipHostMallocDefault));
+        HIP_OK(hipHostMalloc((void**)&pinned[c].m, n * 4, hipHostMallocDefault));
+        HIP_OK(hipHostMalloc((void**)&pinned[c].v, n * 4, hipHostMallocDefault));
+        if (c == 2) HIP_OK(hipHostMalloc((void**)&pinned[c].h, n * 2, hipHostMallocDefault));
+        host_table[c - 1].param_fp32 = pinned[c].p;
+        host_table[c - 1].exp_avg = pinned[c].m;
+        host_table[c - 1].exp_avg_sq = pinned[c].v;
+        host_table[c - 1].param_fp16 = c == 2 ? pinned[c].h : dev[c].h;
+    }
+    for (int s = 0; s < 2; ++s) {
+        HIP_OK(hipMalloc((void**)&staging[s].param_fp32, n * 4));
+        HIP_OK(hipMalloc((void**)&staging[s].exp_avg, n * 4));
+        HIP_OK(hipMalloc((void**)&staging[s].exp_avg_sq, n * 4));
+        HIP_OK(hipMalloc((void**)&staging[s].param_fp16, n * 2));
+    }
+    PS_OK(ps_adam_create(33, lr, b1, b2, eps, wd, 1, 0));
+    oracle_adam_init(&native, lr, b1, b2, eps, wd, 1);
+    for (uint64_t step = 1; step < 4; ++step) {
+        for (int c = 0; c < C; ++c) {
+            new_gradients(rng, host[c], scale);
+            if (c == 0) {
+                if (upload(host[c], dev[c], n)) return 2;
+            } else {
+                memcpy(pinned[c].p, host[c].p.data(), n * 4);
+                memcpy(pinned[c].m, host[c].m.data(), n * 4);
+                memcpy(pinned[c].v, host[c].v.data(), n * 4);
+                if (c == 2)
+                    memcpy(pinned[c].h, host[c].h.data(), n * 2);
+                else
+                    HIP_OK(hipMemcpy(dev[c].h, host[c].h.data(), n * 2, hipMemcpyHostToDevice));
+            }
+        }
+        PS_OK(ps_adam_step_hybrid(33, step, lr, b1, b2, eps, wd, 1, table, 1, host_table, 2, n, staging, 2, scale, NULL,
+                                  stream));
+        HIP_OK(hipStreamSynchronize(stream));
+        oracle_adam_advance(&native, step, b1, b2);
+        oracle_adam_set(&native, lr, eps, wd, 1);
+        for (int c = 0; c < C; ++c) {
+            if (oracle_adam_span(&native, host[c].p.data(), host[c].h.data(), 1, host[c].m.data(), host[c].v.data(),
+                                 n, (float)scale, 0) <= 0)
+                return 5;
+            oracle_cast_f32_to_f16(host[c].p.data(), host[c].h.data(), n);
+        }
+        if (int rc = compare(host[0], dev[0], n, "hybrid step, resident", 0)) return rc;
+        for (int c = 1; c < C; ++c) {
+            bool same = memcmp(pinned[c].p, host[c].p.data(), n * 4) == 0 && memcmp(pinned[c].m, host[c].m.data(), n * 4) == 0 &&
+                        memcmp(pinned[c].v, host[c].v.data(), n * 4) == 0;
+            if (c == 2) {
+                same = same && memcmp(pinned[c].h, host[c].h.data(), n * 2) == 0;
+            } else {
+                std::vector<uint16_t> h16(n);
+                HIP_OK(hipMemcpy(h16.data(), dev[c].h, n * 2, hipMemcpyDeviceToHost));
+                same = same && memcmp(h16.data(), host[c].h.data(), n * 2) == 0;
+            }
+            if (!same) {
+                fprintf(stderr, "hybrid step %llu: host-resident chunk %d differs from the CPU restatement\n",
+                        (unsigned long long)step, c);
+                return 4;
+            }
+        }
+    }
+    // the probe over host-resident positions: an inf in the pinned fp16 payload must reach the device flag
+    PS_OK(ps_state_init(d_state, 1024.0, 1, 2.0, 1, 1000, 1.0, 1, 1, 0, b1, b2, stream));
+    pinned[2].h[n / 2] = 0xFC00;  // -inf
+    PS_OK(ps_overflow_scan_host_chunks(host_table, 2, n, staging, 2, d_state, stream));
+    PS_OK(ps_state_read(d_state, &st, stream));
+    if (st.overflow != 1) {
+        fprintf(stderr, "the probe of host-resident chunks missed an inf\n");
+        return 6;
+    }
+    PS_OK(ps_adam_destroy(33));
+    printf("c abi gpu check ok: 3 host-decided and 8 device-decided steps (2 skipped), 3 steps with host-resident chunks, "
+           "over %d x %zu elements\n", C, n);
     return 0;
 }
