@@ -577,3 +577,57 @@ def test_randomised_shapes_hyperparameters_and_arithmetics():
                 src = (p, m, v, g)[k]
                 assert_bits_equal(got[:offs[k]], src[:offs[k]], f"{what} {name} before")
                 assert_bits_equal(got[offs[k] + n:], src[offs[k] + n:], f"{what} {name} after")
+
+
+def test_two_host_threads_step_their_own_optimizers_concurrently():
+    """Entry points may be called from any host thread: two threads, each with its own optimizer id, chunk list and
+    stream, step at the same time (ctypes drops the GIL during the calls); both must match the oracle."""
+    import threading
+
+    lib = _lib.load()
+    n, C, steps = 256 * 30 + 11, 4, 25
+    results, errors = {}, []
+
+    def worker(tid):
+        try:
+            rng = np.random.default_rng(100 + tid)
+            stream = torch.cuda.Stream()
+            lr, wd = (1e-3, 0.0) if tid == 0 else (1e-4, 0.01)
+            host = [(rng.normal(0, 0.02, n).astype(np.float32), np.zeros(n, np.float32), np.zeros(n, np.float32)) for _ in range(C)]
+            grads = [[(rng.normal(0, 1e-3, n) * 8).astype(np.float16) for _ in range(C)] for _ in range(steps)]
+            with torch.cuda.stream(stream):
+                dev = [tuple(_dev(x.copy()) for x in h) + (torch.zeros(n, dtype=torch.half, device="cuda"),) for h in host]
+                rows = _lib.chunk_array([[d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr()] for d in dev])
+                oid = 700 + tid
+                lib.ps_adam_create(oid, lr, 0.9, 0.999, 1e-8, wd, tid, 0)
+                handle = _lib.current_stream_handle()
+                for s in range(steps):
+                    for c in range(C):
+                        dev[c][3].copy_(torch.from_numpy(grads[s][c]), non_blocking=False)
+                    assert lib.ps_adam_step_chunks(oid, s + 1, lr, 0.9, 0.999, 1e-8, wd, 1, rows, C, n, 8.0, handle) == 0
+                stream.synchronize()
+                lib.ps_adam_destroy(oid)
+            o = oracle.AdamOracle(lr, 0.9, 0.999, 1e-8, wd, bool(tid))
+            for s in range(steps):
+                o.advance(s + 1, 0.9, 0.999)
+                o.set(lr, 1e-8, wd, True)
+                for c in range(C):
+                    p, m, v = host[c]
+                    assert oracle.lib().oracle_adam_span(o._buf, p.ctypes.data, grads[s][c].ctypes.data, 1, m.ctypes.data, v.ctypes.data, n, 8.0, 0) > 0
+            results[tid] = (host, [tuple(t.cpu().numpy() for t in d) for d in dev])
+        except Exception as e:  # surfaced by the main thread
+            errors.append((tid, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for tid in range(2):
+        host, got = results[tid]
+        for c in range(C):
+            assert_bits_equal(got[c][0], host[c][0], f"thread {tid} chunk {c} param")
+            assert_bits_equal(got[c][1], host[c][1], f"thread {tid} chunk {c} exp_avg")
+            assert_bits_equal(got[c][2], host[c][2], f"thread {tid} chunk {c} exp_avg_sq")
+            assert_bits_equal(got[c][3], oracle.cast_fp32_to_fp16(host[c][0]), f"thread {tid} chunk {c} fp16")
