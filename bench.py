@@ -398,6 +398,7 @@ def main():
             "traffic": traffic_from_profile(args.mode, args.arithmetic) if (C, N) == (24, N_CHUNK) else None,
             "algorithmic_bytes_per_launch": algorithmic,
             "avg_kernel_ms": avg_kernel_ms,
+            "median_kernel_ms": sorted(kernel_ms)[len(kernel_ms) // 2],
             "min_kernel_ms": min(kernel_ms),
         },
     }
