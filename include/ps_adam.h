@@ -190,6 +190,21 @@ int ps_adam_step_chunks_gated(int optimizer_id, double lr, double epsilon, doubl
                               size_t chunk_numel, const ps_step_state* d_state,
                               ps_stream_t stream);
 
+/* The per-tensor loop of FP16Adam.fp16_chunk_adam_ops (fp16_cpu_adam.py:336-468) as ONE call, for chunk layouts
+ * in which a parameter's exp_avg / exp_avg_sq do not sit at the parameter's own offset inside their chunks (the
+ * reference packs optimizer-state tensors first-fit in parameters() order, patrickstar/core/client.py:282-309,
+ * which can permute them inside a chunk), so that the whole-chunk pass of ps_adam_step_chunks does not apply.
+ *   tensors[i]  the four DEVICE addresses of parameter i: fp32 param, exp_avg, exp_avg_sq and its fp16 slot
+ *               (gradient in, fp16 parameter out), numels[i] elements each; both are host arrays
+ *   d_state     NULL: host-decided step with loss_scale; else device-gated like ps_adam_step_chunks_gated
+ *               (step, betas and loss_scale ignored; a flagged step restores the fp16 slots from fp32)
+ * Same arithmetic, clamp and 28 B/element as the chunk-list form; the operator's step scalars advance once
+ * for the call.  Up to 48 tensors go into one launch. */
+int ps_adam_step_tensors(int optimizer_id, size_t step, double lr, double beta1, double beta2,
+                         double epsilon, double weight_decay, int bias_correction,
+                         const ps_chunk* tensors, const size_t* numels, int n_tensors,
+                         double loss_scale, const ps_step_state* d_state, ps_stream_t stream);
+
 /* Unconditional restore p16 = RNE(p32) of a chunk list (FP16ChunkWriteBuffer,
  * chunk_io_buff.py:85-151), or only when d_state->overflow is set if d_state != NULL. */
 int ps_restore_fp16_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_numel,

@@ -85,6 +85,7 @@ SIGNATURES = {
     "ps_adam_update": (_i, [_i, _sz, _f, _f, _f, _f, _f, _i, _vp, _vp, _i, _vp, _vp, _sz, _f, _vp, _vp]),
     "ps_adam_step_chunks": (_i, [_i, _sz, _d, _d, _d, _d, _d, _i, _vp, _i, _sz, _d, _vp]),
     "ps_adam_step_chunks_gated": (_i, [_i, _d, _d, _d, _i, _vp, _i, _sz, _vp, _vp]),
+    "ps_adam_step_tensors": (_i, [_i, _sz, _d, _d, _d, _d, _d, _i, _vp, _vp, _i, _d, _vp, _vp]),
     "ps_adam_step_hybrid": (_i, [_i, _sz, _d, _d, _d, _d, _d, _i, _vp, _i, _vp, _i, _sz, _vp, _i, _d, _vp, _vp]),
     "ps_overflow_scan_host_chunks": (_i, [_vp, _i, _sz, _vp, _i, _vp, _vp]),
     "ps_restore_fp16_chunks": (_i, [_vp, _i, _sz, _vp, _vp]),

@@ -244,6 +244,43 @@ void launch_gated_batch(int arith, const ChunkBatch& b, dim3 grid, size_t chunk_
         launch_gated_batch_arith<PS_ARITH_OPERATOR>(b, grid, chunk_numel, ga, d_state, s);
 }
 
+template <int ARITH, int WD>
+void launch_tensors_wd(const TensorBatch& b, unsigned n_tiles, const StepConsts& c, hipStream_t s)
+{
+    dim3 grid(n_tiles), block(kBlock);
+    if (c.unscale == UNSCALE_MUL)
+        hipLaunchKernelGGL((adam_tensors_kernel<ARITH, WD, UNSCALE_MUL>), grid, block, kTensorLdsBytes, s, b, c);
+    else if (ARITH == PS_ARITH_OPERATOR && c.unscale == UNSCALE_DIV)
+        hipLaunchKernelGGL((adam_tensors_kernel<ARITH, WD, UNSCALE_DIV>), grid, block, kTensorLdsBytes, s, b, c);
+    else
+        hipLaunchKernelGGL((adam_tensors_kernel<ARITH, WD, UNSCALE_NONE>), grid, block, kTensorLdsBytes, s, b, c);
+}
+
+template <int ARITH>
+void launch_tensors_arith(const TensorBatch& b, unsigned n_tiles, const StepConsts& c, hipStream_t s)
+{
+    if (c.wd_mode == WD_DECOUPLED)
+        launch_tensors_wd<ARITH, WD_DECOUPLED>(b, n_tiles, c, s);
+    else if (c.wd_mode == WD_L2)
+        launch_tensors_wd<ARITH, WD_L2>(b, n_tiles, c, s);
+    else
+        launch_tensors_wd<ARITH, WD_NONE>(b, n_tiles, c, s);
+}
+
+template <int ARITH>
+void launch_tensors_gated_arith(const TensorBatch& b, unsigned n_tiles, const GatedArgs& ga,
+                                const ps_step_state* d_state, hipStream_t s)
+{
+    dim3 grid(n_tiles), block(kBlock);
+    const bool decay = ARITH == PS_ARITH_OPERATOR ? (float)ga.wd > 0.0f : ga.wd != 0.0;
+    if (decay && ga.adamw)
+        hipLaunchKernelGGL((adam_tensors_gated_kernel<ARITH, WD_DECOUPLED>), grid, block, kTensorLdsBytes, s, b, ga, d_state);
+    else if (decay)
+        hipLaunchKernelGGL((adam_tensors_gated_kernel<ARITH, WD_L2>), grid, block, kTensorLdsBytes, s, b, ga, d_state);
+    else
+        hipLaunchKernelGGL((adam_tensors_gated_kernel<ARITH, WD_NONE>), grid, block, kTensorLdsBytes, s, b, ga, d_state);
+}
+
 // The Python numbers of one step as they cross the boundary.
 struct HyperParams {
     double lr, beta1, beta2, eps, wd;
@@ -583,6 +620,67 @@ int ps_adam_step_chunks_gated(int optimizer_id, double lr, double epsilon, doubl
     return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid) {
         launch_gated_batch(arith, b, grid, chunk_numel, ga, d_state, s);
     });
+}
+
+int ps_adam_step_tensors(int optimizer_id, size_t step, double lr, double beta1, double beta2,
+                         double epsilon, double weight_decay, int bias_correction,
+                         const ps_chunk* tensors, const size_t* numels, int n_tensors,
+                         double loss_scale, const ps_step_state* d_state, ps_stream_t stream)
+{
+    auto o = find_opt(optimizer_id);
+    if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
+    if (n_tensors < 0) return fail(PS_ERR_BAD_ARG, "n_tensors = %d is negative", n_tensors);
+    if (n_tensors > 0 && (!tensors || !numels)) return fail(PS_ERR_BAD_ARG, "tensors or numels is NULL");
+    for (int i = 0; i < n_tensors; ++i) {
+        const ps_chunk& t = tensors[i];
+        if (numels[i] > 0 && (!t.param_fp32 || !t.exp_avg || !t.exp_avg_sq || !t.param_fp16))
+            return fail(PS_ERR_BAD_ARG, "tensor %d has a NULL address", i);
+        if ((numels[i] + kTile - 1) / kTile > kMaxGridX)
+            return fail(PS_ERR_BAD_ARG, "tensor %d: numel = %zu is beyond the launch grid", i, numels[i]);
+    }
+    const int arith = o->arith;
+    StepConsts c;
+    GatedArgs ga = gated_args(*o, lr, epsilon, weight_decay, bias_correction);
+    if (d_state == nullptr) {
+        const HyperParams hp{lr, beta1, beta2, epsilon, weight_decay, loss_scale, bias_correction != 0};
+        c = arith == PS_ARITH_TORCH ? torch_step_consts(*o, step, hp) : operator_step_consts(*o, step, hp);
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    TensorBatch b;
+    int in_batch = 0;
+    size_t tiles = 0;
+    auto flush = [&]() -> int {
+        if (in_batch == 0) return 0;
+        for (int i = in_batch; i < 64; ++i) b.first_tile[i] = 0xFFFFFFFFu;
+        if (d_state == nullptr) {
+            if (arith == PS_ARITH_TORCH)
+                launch_tensors_arith<PS_ARITH_TORCH>(b, (unsigned)tiles, c, s);
+            else
+                launch_tensors_arith<PS_ARITH_OPERATOR>(b, (unsigned)tiles, c, s);
+        } else {
+            if (arith == PS_ARITH_TORCH)
+                launch_tensors_gated_arith<PS_ARITH_TORCH>(b, (unsigned)tiles, ga, d_state, s);
+            else
+                launch_tensors_gated_arith<PS_ARITH_OPERATOR>(b, (unsigned)tiles, ga, d_state, s);
+        }
+        PS_HIP(hipGetLastError());
+        in_batch = 0;
+        tiles = 0;
+        return 0;
+    };
+    memset(&b, 0, sizeof(b));
+    for (int i = 0; i < n_tensors; ++i) {
+        if (numels[i] == 0) continue;
+        const size_t t_i = (numels[i] + kTile - 1) / kTile;
+        if (in_batch == kTensorBatch || tiles + t_i > kMaxGridX)
+            if (int rc = flush()) return rc;
+        b.t[in_batch] = tensors[i];
+        b.numel[in_batch] = numels[i];
+        b.first_tile[in_batch] = (uint32_t)tiles;
+        tiles += t_i;
+        in_batch += 1;
+    }
+    return flush();
 }
 
 int ps_restore_fp16_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_numel,

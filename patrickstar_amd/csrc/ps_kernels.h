@@ -38,17 +38,10 @@ struct GatedArgs {
 // device-resident state; a flagged step restores fp16 from fp32 instead.
 // The weight-decay form is known to the host; the unscale form depends on
 // the device-resident scale and is a uniform branch around the arithmetic.
-template <int ARITH, int WD>
-__global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
-    adam_chunks_gated_kernel(ChunkBatch b, size_t chunk_numel, GatedArgs ga,
-                             const ps_step_state* __restrict__ st)
+// Step constants of a device-decided step, formed by every wave from the device-resident state.
+template <int ARITH>
+__device__ __forceinline__ StepConsts gated_consts(const GatedArgs& ga, const ps_step_state* __restrict__ st)
 {
-    const ps_chunk& ch = b.c[blockIdx.y];
-    const size_t base = (size_t)blockIdx.x * kTile;
-    if (st->overflow) {
-        restore_tile(ch.param_fp32, ch.param_fp16, base, chunk_numel);
-        return;
-    }
     StepConsts c;
     const float clip = clamp_bound(ga.grad_clamp, st->cur_scale);
     if (ARITH == PS_ARITH_OPERATOR) {
@@ -62,7 +55,78 @@ __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
                      bc ? st->bias_correction1_next : 1.0, bc ? st->bias_correction2_next : 1.0,
                      st->cur_scale, clip);
     }
+    return c;
+}
+
+template <int ARITH, int WD>
+__global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
+    adam_chunks_gated_kernel(ChunkBatch b, size_t chunk_numel, GatedArgs ga,
+                             const ps_step_state* __restrict__ st)
+{
+    const ps_chunk& ch = b.c[blockIdx.y];
+    const size_t base = (size_t)blockIdx.x * kTile;
+    if (st->overflow) {
+        restore_tile(ch.param_fp32, ch.param_fp16, base, chunk_numel);
+        return;
+    }
+    const StepConsts c = gated_consts<ARITH>(ga, st);
     adam_tile<ARITH, WD, UNSCALE_RUNTIME>(c, ch, base, chunk_numel);
+}
+
+// ------------------------------------------------------- tensor-list kernels
+//
+// The same tiles over a list of TENSORS of different lengths, for chunk layouts in which a
+// parameter's momentum and variance do not sit at the parameter's own offset (the reference packs
+// optimizer-state tensors first-fit in parameters() order, patrickstar/core/client.py:282-309, so the
+// whole-chunk pass does not apply and the reference loops over tensors, fp16_cpu_adam.py:336-468).
+// Grid: x = tile of the batch; tiles are numbered tensor by tensor.  A wave finds its tensor with one
+// 64-lane load of the batch's first-tile table, a ballot and a population count.
+
+// A wave of the tensor-list kernels starts with one more dependent load (the lookup) than a wave of the
+// chunk-list kernels; 13 resident workgroups per CU (12 KiB each) instead of 9 make up for it
+// (GPT-2 XL's 580 tensors, 1.56 G elements: 7.42 ms with 12 KiB, 7.97 ms with 17 KiB, 7.05 ms as one chunk).
+#ifndef PS_TENSOR_LDS_KB
+#define PS_TENSOR_LDS_KB 12
+#endif
+constexpr unsigned kTensorLdsBytes = PS_TENSOR_LDS_KB * 1024u;
+#ifndef PS_TENSOR_BATCH
+#define PS_TENSOR_BATCH 48
+#endif
+constexpr int kTensorBatch = PS_TENSOR_BATCH;
+static_assert(kTensorBatch <= 64, "the first-tile table is read by one wave");
+struct TensorBatch {
+    ps_chunk t[kTensorBatch];          // fp32 param, exp_avg, exp_avg_sq, fp16 slot of each tensor
+    uint64_t numel[kTensorBatch];
+    uint32_t first_tile[64];           // of tensor i; 0xFFFFFFFF beyond the last tensor
+};
+
+__device__ __forceinline__ int tensor_of_tile(const TensorBatch& b, uint32_t tile)
+{
+    const uint32_t first = b.first_tile[threadIdx.x & 63];
+    // the same in every lane: say so, and descriptor and length come through scalar loads
+    return __builtin_amdgcn_readfirstlane(__popcll(__ballot(tile >= first)) - 1);
+}
+
+template <int ARITH, int WD, int UNS>
+__global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
+    adam_tensors_kernel(TensorBatch b, StepConsts c)
+{
+    const int k = tensor_of_tile(b, blockIdx.x);
+    adam_tile<ARITH, WD, UNS>(c, b.t[k], (size_t)(blockIdx.x - b.first_tile[k]) * kTile, (size_t)b.numel[k]);
+}
+
+template <int ARITH, int WD>
+__global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
+    adam_tensors_gated_kernel(TensorBatch b, GatedArgs ga, const ps_step_state* __restrict__ st)
+{
+    const int k = tensor_of_tile(b, blockIdx.x);
+    const size_t base = (size_t)(blockIdx.x - b.first_tile[k]) * kTile;
+    if (st->overflow) {
+        restore_tile(b.t[k].param_fp32, b.t[k].param_fp16, base, (size_t)b.numel[k]);
+        return;
+    }
+    const StepConsts c = gated_consts<ARITH>(ga, st);
+    adam_tile<ARITH, WD, UNSCALE_RUNTIME>(c, b.t[k], base, (size_t)b.numel[k]);
 }
 
 __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY

@@ -1,0 +1,183 @@
+"""GPU parity of ps_adam_step_tensors: the per-tensor loop of the reference as one call, for chunk layouts in which
+momentum and variance tensors are NOT at their parameter's own offset (the reference's own packing of optimizer-state
+tensors, patrickstar/core/client.py:282-309).  Bit-exact against the CPU restatements, both arithmetics, host-decided
+and device-gated."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import patrickstar_amd as ps
+from patrickstar_amd import _lib
+from _harness import assert_bits_equal
+
+pytestmark = pytest.mark.gpu
+
+SIZES = [1, 3, 255, 256, 257, 768, 1000, 4096 + 3, 2304 * 64, 100_000, 5, 64] * 5 + [300_001]  # 61 tensors: two launches
+
+
+class PermutedLayout:
+    """Parameters packed in order into an fp16 and an fp32 payload; momentum packed in REVERSE order and variance
+    in a rotated order into theirs, so no two lists share offsets."""
+
+    def __init__(self, sizes, seed, scale):
+        rng = np.random.default_rng(seed)
+        self.sizes = sizes
+        total = sum(sizes)
+        order = {"p": list(range(len(sizes))), "m": list(reversed(range(len(sizes)))),
+                 "v": list(range(7, len(sizes))) + list(range(7))}
+        self.off = {}
+        for key, seq in order.items():
+            cur, offs = 0, {}
+            for i in seq:
+                offs[i] = cur
+                cur += sizes[i]
+            self.off[key] = offs
+        self.host = {
+            "p": rng.normal(0, 0.02, total).astype(np.float32),
+            "m": rng.normal(0, 1e-4, total).astype(np.float32),
+            "v": np.abs(rng.normal(0, 1e-6, total)).astype(np.float32),
+            "h": (rng.normal(0, 1e-3, total) * scale).astype(np.float16),
+        }
+        self.dev = {k: torch.from_numpy(a.copy()).cuda() for k, a in self.host.items()}
+        rows = []
+        for i, n in enumerate(sizes):
+            rows.append([
+                self.dev["p"][self.off["p"][i]:].data_ptr(), self.dev["m"][self.off["m"][i]:].data_ptr(),
+                self.dev["v"][self.off["v"][i]:].data_ptr(), self.dev["h"][self.off["p"][i]:].data_ptr(),
+            ])
+        self.table = _lib.chunk_array(rows)
+        self.numels = (ctypes.c_size_t * len(sizes))(*sizes)
+
+    def views(self, i):
+        n = self.sizes[i]
+        return (self.host["p"][self.off["p"][i]:][:n], self.host["h"][self.off["p"][i]:][:n],
+                self.host["m"][self.off["m"][i]:][:n], self.host["v"][self.off["v"][i]:][:n])
+
+    def new_grads(self, rng, scale):
+        g = (rng.normal(0, 1e-3, self.host["h"].size) * scale).astype(np.float16)
+        self.host["h"][...] = g
+        self.dev["h"].copy_(torch.from_numpy(g))
+
+    def compare(self, what):
+        for k in "pmvh":
+            assert_bits_equal(self.dev[k].cpu().numpy(), self.host[k], f"{what}: {k}")
+
+
+@pytest.mark.parametrize("arithmetic", ["operator", "torch"])
+@pytest.mark.parametrize("adamw,wd,scale", [(True, 0.01, 2**12), (False, 0.01, 1000.0), (False, 0.0, None)])
+def test_host_decided_steps_over_a_permuted_layout(arithmetic, adamw, wd, scale):
+    lib = _lib.load()
+    lr, b1, b2, eps = 1e-4, 0.9, 0.999, 1e-8
+    L = PermutedLayout(SIZES, seed=len(arithmetic) + int(adamw), scale=scale or 1.0)
+    rng = np.random.default_rng(9)
+    oid = 820
+    _lib.check(lib.ps_adam_create(oid, lr, b1, b2, eps, wd, int(adamw), 0), "create")
+    if arithmetic == "torch":
+        _lib.check(lib.ps_adam_set_arithmetic(oid, _lib.PS_ARITH_TORCH), "arith")
+    native = oracle.AdamOracle(lr, b1, b2, eps, wd, adamw)
+    for step in (100, 101, 102):
+        if step > 100:
+            L.new_grads(rng, scale or 1.0)
+        _lib.check(
+            lib.ps_adam_step_tensors(oid, step, lr, b1, b2, eps, wd, 1, L.table, L.numels, len(SIZES),
+                                     float(scale) if scale is not None else -1.0, None, _lib.current_stream_handle()),
+            "ps_adam_step_tensors",
+        )
+        torch.cuda.synchronize()
+        native.advance(step, b1, b2)
+        native.set(lr, eps, wd, True)
+        for i, n in enumerate(SIZES):
+            p, h, m, v = L.views(i)
+            if arithmetic == "torch":
+                pc, mc, vc, hc = p.copy(), m.copy(), v.copy(), h.copy()
+                oracle.torch_formula_update(pc, hc, mc, vc, step, lr, b1, b2, eps, wd, adamw, scale)
+                p[...], m[...], v[...] = pc, mc, vc
+            else:
+                pc, mc, vc, hc = p.copy(), m.copy(), v.copy(), h.copy()
+                assert oracle.lib().oracle_adam_span(native._buf, pc.ctypes.data, hc.ctypes.data, 1, mc.ctypes.data,
+                                                     vc.ctypes.data, n, float(scale) if scale is not None else -1.0, 0) > 0
+                p[...], m[...], v[...] = pc, mc, vc
+            h[...] = oracle.cast_fp32_to_fp16(np.ascontiguousarray(p))
+        L.compare(f"{arithmetic} step {step}")
+    lib.ps_adam_destroy(oid)
+
+
+@pytest.mark.parametrize("arithmetic", ["operator", "torch"])
+def test_device_gated_steps_over_a_permuted_layout(arithmetic):
+    """Scale, step and flag from the device state; iteration 1 is poisoned and must restore the fp16 slots only."""
+    lib = _lib.load()
+    lr, b1, b2, eps, wd = 1e-3, 0.9, 0.999, 1e-8, 0.01
+    kw = dict(init_scale=2**10, scale_factor=2, scale_window=2, min_scale=1)
+    scaler = ps.DynamicLossScaler(**kw)
+    scaler.materialize("cuda:0", betas=(b1, b2))
+    oscaler = oracle.ScalerOracle(**kw)
+    L = PermutedLayout(SIZES[:50], seed=4, scale=2.0**10)
+    rng = np.random.default_rng(10)
+    oid = 821
+    _lib.check(lib.ps_adam_create(oid, lr, b1, b2, eps, wd, 1, 0), "create")
+    if arithmetic == "torch":
+        _lib.check(lib.ps_adam_set_arithmetic(oid, _lib.PS_ARITH_TORCH), "arith")
+    native = oracle.AdamOracle(lr, b1, b2, eps, wd, True)
+    adam_step = 0
+    for it in range(5):
+        L.new_grads(rng, float(oscaler.loss_scale))
+        if it == 1:
+            L.host["h"][L.off["p"][9] + 2] = np.float16("inf")
+            L.dev["h"].copy_(torch.from_numpy(L.host["h"]))
+        scaler.scan(L.dev["h"])
+        _lib.check(
+            lib.ps_adam_step_tensors(oid, 0, lr, b1, b2, eps, wd, 1, L.table, L.numels, 50, -1.0, scaler.state_ptr,
+                                     _lib.current_stream_handle()),
+            "ps_adam_step_tensors",
+        )
+        scaler.update_scale(None)
+        torch.cuda.synchronize()
+        if it == 1:
+            oscaler.update_scale(True)
+            for i in range(50):
+                p, h, m, v = L.views(i)
+                h[...] = oracle.cast_fp32_to_fp16(np.ascontiguousarray(p))
+        else:
+            adam_step += 1
+            scale = oscaler.loss_scale
+            native.advance(adam_step, b1, b2)
+            native.set(lr, eps, wd, True)
+            for i, n in enumerate(SIZES[:50]):
+                p, h, m, v = L.views(i)
+                pc, mc, vc, hc = p.copy(), m.copy(), v.copy(), h.copy()
+                if arithmetic == "torch":
+                    oracle.torch_formula_update(pc, hc, mc, vc, adam_step, lr, b1, b2, eps, wd, True, scale)
+                else:
+                    assert oracle.lib().oracle_adam_span(native._buf, pc.ctypes.data, hc.ctypes.data, 1, mc.ctypes.data,
+                                                         vc.ctypes.data, n, float(scale), 0) > 0
+                p[...], m[...], v[...] = pc, mc, vc
+                h[...] = oracle.cast_fp32_to_fp16(pc)
+            oscaler.update_scale(False)
+        L.compare(f"{arithmetic} iteration {it}")
+        assert scaler.loss_scale == oscaler.loss_scale
+    assert scaler.adam_step == 4
+    lib.ps_adam_destroy(oid)
+
+
+def test_tensor_list_argument_checks_and_empty_lists():
+    lib = _lib.load()
+    lib.ps_adam_create(822, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, 0)
+    s = _lib.current_stream_handle()
+    assert lib.ps_adam_step_tensors(822, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, None, 0, -1.0, None, s) == 0
+    assert lib.ps_adam_step_tensors(822, 2, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, None, 3, -1.0, None, s) == _lib.PS_ERR_BAD_ARG
+    assert lib.ps_adam_step_tensors(822, 2, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, None, -1, -1.0, None, s) == _lib.PS_ERR_BAD_ARG
+    x = torch.ones(8, device="cuda")
+    h = torch.zeros(8, dtype=torch.half, device="cuda")
+    rows = _lib.chunk_array([[x.data_ptr(), x.data_ptr(), 0, h.data_ptr()], [x.data_ptr(), 0, 0, 0]])
+    numels = (ctypes.c_size_t * 2)(8, 0)
+    assert lib.ps_adam_step_tensors(822, 2, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, rows, numels, 2, -1.0, None, s) == _lib.PS_ERR_BAD_ARG
+    assert b"tensor 0" in lib.ps_last_error()
+    numels = (ctypes.c_size_t * 2)(0, 0)  # zero-length tensors may carry NULL addresses and are skipped
+    assert lib.ps_adam_step_tensors(822, 2, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, rows, numels, 2, -1.0, None, s) == 0
+    assert lib.ps_adam_step_tensors(4711, 2, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, rows, numels, 2, -1.0, None, s) == _lib.PS_ERR_UNKNOWN_ID
+    torch.cuda.synchronize()
+    assert torch.equal(x, torch.ones(8, device="cuda"))
+    lib.ps_adam_destroy(822)
