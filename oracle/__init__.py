@@ -19,7 +19,7 @@ Contents
 ``StaticScalerOracle``    ``patrickstar/fp16/loss_scaler.py:46-76``.
 ``scaler_from_config``    ``patrickstar/runtime/engine.py:79-99`` wiring (``hysteresis`` feeds
                           ``scale_factor``; ``delayed_shift`` is always 1 through the engine).
-``optimizer_step_oracle`` sequencing of ``patrickstar/ops/fp16_cpu_adam.py:472-628`` over a
+``OptimizerStepOracle``   sequencing of ``patrickstar/ops/fp16_cpu_adam.py:472-628`` over a
                           chunk list held as numpy arrays.
 
 Pinning: see the header of ``adam_oracle.c`` for the Adam arithmetic and
@@ -322,26 +322,41 @@ def scaler_from_config(fp16_config):
 
 
 class OptimizerStepOracle:
-    """``FP16Adam.step`` over a chunk list, one native call per step over each chunk.
+    """``FP16Adam.step`` over a chunk list, one ``adam_update`` per TENSOR as the reference makes them.
 
     Each chunk is a dict of flat numpy arrays ``p32``, ``m``, ``v`` (float32)
     and ``p16`` (float16; holds the gradients on entry to ``step`` and the
     refreshed fp16 parameters on exit, as in the reference where backward
     overwrites the fp16 parameter slot with the gradient).
 
+    ``tensors`` lists the trainable parameters in ``param_groups`` order as
+    ``(chunk index, element offset, numel)``; by default every chunk is one
+    tensor, in chunk order (what a synthetic chunk list of one flat parameter
+    per chunk is).  Parameters that are not listed (``requires_grad=False``)
+    are skipped like ``fp16_cpu_adam.py:566-569`` skips them.
+
     Sequencing restated from ``fp16_cpu_adam.py``: overflow gate first
     (``:549-558``: on overflow restore fp16 from fp32, ``update_scale(True)``,
-    leave ``step`` alone), else ``step += 1`` (``:574``), update every chunk
-    with the scaler's current scale or -1 (``:227``), cast fp32 -> fp16
-    (``chunk_io_buff.py:116-126``), ``update_scale(False)`` (``:624-625``).
-    The native object sees one ``adam_update`` per step (the whole chunk list
-    is one flat tensor for it), so consecutive steps take the running-product
-    branch of ``cpu_adam.h:143-162``.
+    leave ``step`` alone), else ``step += 1`` (``:574``), then the loop of
+    ``fp16_chunk_adam_ops`` (``:336-468``): for every tensor in turn clamp its
+    gradient (``:364-379``), run the operator (``:415-428``) or the torch
+    formula (``:430-443``) with the scaler's current scale or -1 (``:227``);
+    whole-chunk cast fp32 -> fp16 of every chunk that was visited
+    (``chunk_io_buff.py:116-126,143-146``); ``update_scale(False)`` (``:624-625``).
+
+    Every operator call carries the same ``step``, so inside
+    ``Adam_Optimizer::IncrementStep`` (``cpu_adam.h:143-162``) only the FIRST
+    call of a step can find ``_step + 1 == step`` and multiply the running
+    float product; every later call of the step sees ``_step + 1 != step`` and
+    evaluates ``pow``.  With two or more tensors the first tensor of step t is
+    therefore updated with ``float(pow(beta, t-1)) * beta`` and all others
+    with ``float(pow(beta, t))``.  ``AdamOracle.update`` is that call, state
+    machine included; nothing about the branch is decided here.
     """
 
     def __init__(self, chunks, loss_scaler=None, lr=1e-3, betas=(0.9, 0.999), eps=1e-8,
                  weight_decay=0.0, use_adamw=False, isa=ISA_AUTO, gradient_clipping=-1, arithmetic="operator",
-                 operator_chunks=()):
+                 operator_chunks=(), tensors=None):
         self.chunks = chunks
         self.loss_scaler = loss_scaler
         self.lr, self.betas, self.eps, self.weight_decay = lr, betas, eps, weight_decay
@@ -351,12 +366,17 @@ class OptimizerStepOracle:
         self.isa = isa
         self.gradient_clipping = gradient_clipping
         # The reference picks per tensor by where its optimizer state lives (:415-443):
-        # "operator": every chunk through the native operator (state in host memory);
-        # "torch": chunks through torch_adam_update (state in GPU memory), except those listed
-        # in operator_chunks (indices of chunks whose state is in host memory).
+        # "operator": every tensor through the native operator (state in host memory);
+        # "torch": tensors through torch_adam_update (state in GPU memory), except those of the chunks
+        # listed in operator_chunks (indices of chunks whose state is in host memory).
         assert arithmetic in ("operator", "torch")
         self.arithmetic = arithmetic
         self.operator_chunks = set(operator_chunks)
+        if tensors is None:
+            tensors = [(i, 0, c["p32"].size) for i, c in enumerate(chunks)]
+        for ci, off, numel in tensors:
+            assert 0 <= ci < len(chunks) and 0 <= off and off + numel <= chunks[ci]["p32"].size, (ci, off, numel)
+        self.tensors = list(tensors)
         self.native = AdamOracle(lr, betas[0], betas[1], eps, weight_decay, use_adamw)
 
     def check_overflow(self):
@@ -369,6 +389,17 @@ class OptimizerStepOracle:
             if self.loss_scaler.has_overflow(c["p16"]):
                 self.has_overflow = True
 
+    def _clamp(self, g):
+        # fp16_cpu_adam.py:364-379, GPU branch: clamp_ of the fp16 gradient tensor to
+        # +-min(65504, clipping * loss_scale); the Python float bound narrows to float, then to half
+        bound = self.gradient_clipping
+        if self.loss_scaler is not None:
+            bound = bound * self.loss_scaler.loss_scale
+        bound = min(65504.0, bound)
+        b16 = np.float16(np.float32(bound))
+        g[g < -b16] = -b16
+        g[g > b16] = b16
+
     def step(self):
         """Returns True when the step was skipped."""
         if self.has_overflow:
@@ -379,38 +410,28 @@ class OptimizerStepOracle:
             return True
         self.step_count += 1
         scaler_scale = self.loss_scaler.loss_scale if self.loss_scaler is not None else None
-        via_torch = [
-            self.arithmetic == "torch" and i not in self.operator_chunks for i in range(len(self.chunks))
-        ]
-        if not all(via_torch):
-            # the native object is only touched when the operator runs at all
-            self.native.advance(self.step_count, self.betas[0], self.betas[1])
-            self.native.set(self.lr, self.eps, self.weight_decay, True)
-        L = lib()
-        if self.gradient_clipping > 0:
-            # fp16_cpu_adam.py:364-379, GPU branch: clamp_ of the fp16 gradient tensor to
-            # +-min(65504, clipping * loss_scale); the Python float bound narrows to float, then to half
-            bound = self.gradient_clipping
-            if self.loss_scaler is not None:
-                bound = bound * self.loss_scaler.loss_scale
-            bound = min(65504.0, bound)
-            b16 = np.float16(np.float32(bound))
-            for c in self.chunks:
-                g = c["p16"]
-                g[g < -b16] = -b16
-                g[g > b16] = b16
-        for c, torch_branch in zip(self.chunks, via_torch):
-            if torch_branch:
+        visited = []
+        for ci, off, numel in self.tensors:
+            c = self.chunks[ci]
+            p, g, m, v = (c[k][off : off + numel] for k in ("p32", "p16", "m", "v"))
+            if self.gradient_clipping > 0:
+                self._clamp(g)
+            if self.arithmetic == "torch" and ci not in self.operator_chunks:
                 torch_formula_update(
-                    c["p32"], c["p16"], c["m"], c["v"], self.step_count, self.lr, self.betas[0], self.betas[1],
+                    p, g, m, v, self.step_count, self.lr, self.betas[0], self.betas[1],
                     self.eps, self.weight_decay, self.use_adamw, scaler_scale,
                 )
             else:
-                took = L.oracle_adam_span(
-                    self.native._buf, _ptr(c["p32"]), _ptr(c["p16"]), 1, _ptr(c["m"]), _ptr(c["v"]),
-                    c["p32"].size, float(scaler_scale if scaler_scale is not None else -1), self.isa,
+                # one adam_update of the native operator: IncrementStep, update_state, Step
+                self.native.update(
+                    self.step_count, self.lr, self.betas[0], self.betas[1], self.eps, self.weight_decay, True,
+                    p, g, m, v, float(scaler_scale if scaler_scale is not None else -1), self.isa,
                 )
-                assert took > 0
+            if ci not in visited:
+                visited.append(ci)
+        # the gradients of a chunk have all been read by now: whole-chunk write-back, padding included
+        for ci in visited:
+            c = self.chunks[ci]
             c["p16"][...] = cast_fp32_to_fp16(c["p32"])
         if self.loss_scaler:
             self.loss_scaler.update_scale(False)

@@ -1,5 +1,7 @@
 """Pins the oracle's restatement of FP16Adam.step's sequencing (patrickstar/ops/fp16_cpu_adam.py:472-628) and of the
 element-wise gradient clamp (:364-379) through invariants and a library routine; CPU only."""
+import math
+
 import numpy as np
 import torch
 
@@ -86,3 +88,177 @@ def test_clamp_restatement_equals_tensor_clamp():
             assert np.array_equal(nan, np.isnan(y.astype(np.float32)))
             assert np.array_equal(x[~nan], y[~nan]), (clipping, scale, k)
         assert 0 < (np.abs(g[3:].astype(np.float32)) > bound).mean() < 1
+
+
+# ---- the per-tensor call pattern of one step (fp16_cpu_adam.py:336-428 -> cpu_adam.h:143-162) -----------------
+#
+# The reference calls adam_update once per tensor with the same `step`.  IncrementStep does `_step++` and
+# compares: only the first call of a step can continue the running float product; every later call of the
+# step finds `_step + 1 != step` and evaluates pow.  Expected values below are built WITHOUT the step-level
+# oracle: from math.pow / numpy float32 arithmetic and from fresh single-call operator objects whose branch
+# is forced by hand (those branches are pinned in test_oracle_adam.py::test_beta_power_state_machine).
+
+B1, B2 = np.float32(0.9), np.float32(0.999)
+
+
+def _beta_powers(t, first, single_tensor_history=False):
+    """float32 beta^t as IncrementStep leaves it for the first / a later call of step t (steps 1..t-1 all ran)."""
+    if first:
+        if single_tensor_history:
+            r1 = r2 = np.float32(1.0)
+            for _ in range(t):
+                r1, r2 = np.float32(r1 * B1), np.float32(r2 * B2)
+            return r1, r2
+        return (np.float32(np.float32(math.pow(float(B1), t - 1)) * B1),
+                np.float32(np.float32(math.pow(float(B2), t - 1)) * B2))
+    return np.float32(math.pow(float(B1), t)), np.float32(math.pow(float(B2), t))
+
+
+def _probe_update_f64(g, m, v, lr, eps, b1t, b2t):
+    """Textbook Adam on a zero parameter in float64 with the given float32 beta powers: p' = -lr/bc1 * m'/(sqrt(v')*bc2inv + eps)."""
+    b1, b2 = float(B1), float(B2)
+    m1 = b1 * m + (1.0 - b1) * g
+    v1 = b2 * v + (1.0 - b2) * g * g
+    bc1 = float(np.float32(1.0) - b1t)
+    bc2inv = float(np.float32(1.0) / np.sqrt(np.float32(1.0) - b2t, dtype=np.float32))
+    return -(lr / bc1) * m1 / (math.sqrt(v1) * bc2inv + eps)
+
+
+def _three_tensor_layout():
+    # two chunks of 600 elements: tensors at (0, 0, 250), (0, 250, 300), (1, 0, 400); the tails are padding
+    return [(0, 0, 250), (0, 250, 300), (1, 0, 400)]
+
+
+def test_first_tensor_of_a_step_multiplies_and_every_later_tensor_takes_pow():
+    lr, eps = 1e-3, 1e-8
+    tensors = _three_tensor_layout()
+    cs = _chunks(n_chunks=2, n=600, seed=21)
+    for c in cs:
+        c["p16"][...] = 0
+    opt = oracle.OptimizerStepOracle(cs, None, lr=lr, betas=(0.9, 0.999), eps=eps, tensors=tensors)
+    rng = np.random.default_rng(22)
+    differing = 0
+    for t in range(1, 21):
+        # element 0 of every tensor is a probe: parameter and moments 0, so the new parameter IS
+        # step_size * m'/denominator with no cancellation anywhere
+        probes = []
+        for ci, off, numel in tensors:
+            g = rng.normal(0, 1e-2, numel).astype(np.float16)
+            g[0] = np.float16(0.0123)
+            cs[ci]["p16"][off : off + numel] = g
+            cs[ci]["p32"][off] = cs[ci]["m"][off] = cs[ci]["v"][off] = 0.0
+            probes.append((float(g[0]), 0.0, 0.0))
+        assert opt.step() is False
+        for k, ((ci, off, _), (g, m, v)) in enumerate(zip(tensors, probes)):
+            got = float(cs[ci]["p32"][off])
+            right = _probe_update_f64(g, m, v, lr, eps, *_beta_powers(t, first=(k == 0)))
+            wrong = _probe_update_f64(g, m, v, lr, eps, *_beta_powers(t, first=(k != 0)))
+            assert abs(got - right) <= 4e-7 * abs(right), (t, k, got, right)
+            if abs(right - wrong) > 2e-6 * abs(right):
+                differing += 1
+                assert abs(got - wrong) > 1e-6 * abs(right), (t, k, "took the other branch of IncrementStep")
+    # the two branches really are different numbers on most early steps (bc2inv differs by up to 1e-5)
+    assert differing >= 8
+
+
+def test_step_oracle_equals_hand_sequenced_operator_calls():
+    """Bit-exact: every tensor against a FRESH operator object driven into the branch the reference takes."""
+    kw = dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
+    tensors = _three_tensor_layout()
+    cs = _chunks(n_chunks=2, n=600, seed=31)
+    s = oracle.StaticScalerOracle(64)
+    opt = oracle.OptimizerStepOracle(cs, s, tensors=tensors, **kw)
+    rng = np.random.default_rng(32)
+
+    def hand(t, k, ref_chunk, off, numel):
+        o = oracle.AdamOracle(1e-3, 0.9, 0.999, 1e-8, 0.01, True)
+        if k == 0 and t > 1:
+            o.advance(t - 1, 0.9, 0.999)  # a cold call: pow(beta, t-1), as the LAST tensor of step t-1 left it
+        elif k > 0:
+            o.advance(t, 0.9, 0.999)  # the first tensor of this step came before: _step is already t
+        sl = slice(off, off + numel)
+        o.update(t, 1e-3, 0.9, 0.999, 1e-8, 0.01, True, ref_chunk["p32"][sl], ref_chunk["p16"][sl],
+                 ref_chunk["m"][sl], ref_chunk["v"][sl], 64.0)
+
+    steps = list(range(1, 13))
+    for t in steps:
+        for c in cs:
+            c["p16"][...] = (rng.normal(0, 1e-3, c["p16"].size) * 64).astype(np.float16)
+        ref = _copy(cs)
+        opt.step()
+        for k, (ci, off, numel) in enumerate(tensors):
+            hand(t, k, ref[ci], off, numel)
+        for c, r in zip(cs, ref):
+            for key in ("p32", "m", "v"):
+                assert np.array_equal(c[key].view(np.uint32), r[key].view(np.uint32)), (t, key)
+            assert np.array_equal(c["p16"].view(np.uint16), oracle.cast_fp32_to_fp16(r["p32"]).view(np.uint16))
+    assert opt.step_count == 12
+
+    # a jump (optimizer reloaded at step 99 with a fresh native object): the first tensor of step 100 finds
+    # _step + 1 = 1 != 100 and takes pow like the others; step 101 then multiplies for its first tensor again
+    opt2 = oracle.OptimizerStepOracle(cs, s, tensors=tensors, **kw)
+    opt2.step_count = 99
+    for t in (100, 101):
+        for c in cs:
+            c["p16"][...] = (rng.normal(0, 1e-3, c["p16"].size) * 64).astype(np.float16)
+        ref = _copy(cs)
+        opt2.step()
+        for k, (ci, off, numel) in enumerate(tensors):
+            o = oracle.AdamOracle(1e-3, 0.9, 0.999, 1e-8, 0.01, True)
+            if t == 101 and k == 0:
+                o.advance(100, 0.9, 0.999)
+            elif t == 101:
+                o.advance(101, 0.9, 0.999)
+            sl = slice(off, off + numel)
+            o.update(t, 1e-3, 0.9, 0.999, 1e-8, 0.01, True, ref[ci]["p32"][sl], ref[ci]["p16"][sl], ref[ci]["m"][sl],
+                     ref[ci]["v"][sl], 64.0)
+        for c, r in zip(cs, ref):
+            for key in ("p32", "m", "v"):
+                assert np.array_equal(c[key].view(np.uint32), r[key].view(np.uint32)), (t, key)
+
+
+def test_a_skipped_step_does_not_touch_the_native_object_and_single_tensor_lists_keep_the_running_product():
+    # one tensor per step: the running float product on every step (the one-chunk reference configuration)
+    cs = _chunks(n_chunks=1, n=64, seed=41)
+    opt = oracle.OptimizerStepOracle(cs, None, lr=1e-3)
+    for t in range(1, 31):
+        cs[0]["p16"][...] = np.float16(0.01)
+        opt.step()
+        b1t, _ = _beta_powers(t, first=True, single_tensor_history=True)
+        assert opt.native.consts()[5] == np.float32(1.0) - b1t
+    # two tensors, dynamic scaler, step 3 poisoned: the skipped step makes no operator call, so step 3 is retried
+    # and its first tensor multiplies from pow(beta, 2)
+    cs = _chunks(n_chunks=2, n=64, seed=42)
+    s = oracle.ScalerOracle(init_scale=4, scale_factor=2, scale_window=1000)
+    opt = oracle.OptimizerStepOracle(cs, s, lr=1e-3)
+    skipped = []
+    for i in range(5):
+        for c in cs:
+            c["p16"][...] = np.float16(0.01)
+        if i == 2:
+            cs[1]["p16"][5] = np.nan
+        cs[0]["p32"][0] = cs[0]["m"][0] = cs[0]["v"][0] = 0.0
+        m0, v0 = 0.0, 0.0
+        scale = s.loss_scale
+        opt.check_overflow()
+        skipped.append(opt.step())
+        if not skipped[-1]:
+            t = opt.step_count
+            right = _probe_update_f64(float(np.float16(0.01)) / scale, m0, v0, 1e-3, 1e-8, *_beta_powers(t, first=True))
+            assert abs(float(cs[0]["p32"][0]) - right) <= 4e-7 * abs(right), (i, t)
+    assert skipped == [False, False, True, False, False] and opt.step_count == 4
+
+
+def test_frozen_tensors_are_not_listed_and_not_touched():
+    cs = _chunks(n_chunks=1, n=500, seed=51)
+    cs[0]["p16"][...] = cs[0]["p32"].astype(np.float16)  # the slot of a frozen parameter holds the parameter
+    before = _copy(cs)
+    live = [(0, 0, 100), (0, 300, 200)]  # elements 100..299 belong to a frozen parameter
+    cs[0]["p16"][:100] = np.float16(0.5)
+    cs[0]["p16"][300:] = np.float16(-0.5)
+    opt = oracle.OptimizerStepOracle(cs, None, lr=1e-2, weight_decay=0.1, use_adamw=True, tensors=live)
+    opt.step()
+    for key in ("p32", "m", "v"):
+        assert np.array_equal(cs[0][key][100:300], before[0][key][100:300])
+        assert not np.array_equal(cs[0][key][:100], before[0][key][:100])
+    assert np.array_equal(cs[0]["p16"][100:300].view(np.uint16), before[0]["p32"][100:300].astype(np.float16).view(np.uint16))
