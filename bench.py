@@ -213,9 +213,9 @@ def run_hybrid(args):
     def kernels():
         s = _lib.current_stream_handle()
         if res_rows:
-            lib.ps_adam_step_chunks(991, 1, 1e-4, 0.9, 0.999, 1e-8, 0.01, 1, res, len(res_rows), N, 4096.0, s)
+            lib.ps_adam_step_chunks(991, 1, 1e-4, 0.9, 0.999, 1e-8, 0.01, 1, res, len(res_rows), N, None, 4096.0, s)
         for _ in host_pos:
-            lib.ps_adam_step_chunks(991, 1, 1e-4, 0.9, 0.999, 1e-8, 0.01, 1, one, 1, N, 4096.0, s)
+            lib.ps_adam_step_chunks(991, 1, 1e-4, 0.9, 0.999, 1e-8, 0.01, 1, one, 1, N, None, 4096.0, s)
 
     t_h2d, t_d2h = timed(h2d), timed(d2h)
     h2d()  # leave finite data in the slot for the kernel leg

@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define PS_ABI_VERSION 2
+#define PS_ABI_VERSION 3
 
 #define PS_ERR_BAD_ARG (-10001)     /* null pointer, negative count, unknown mode */
 #define PS_ERR_UNKNOWN_ID (-10002)  /* optimizer id was never created (the reference dereferences null here) */
@@ -65,7 +65,7 @@ typedef struct ps_chunk {
  * (fp16_cpu_adam.py:279-285) and the Adam step counter with its float
  * beta^t running products (cpu_adam.h:143-162).  It lives in device memory
  * so that "was there an overflow -> skip, restore, halve" needs no host
- * round trip.  160 bytes, 16-byte aligned.
+ * round trip.  192 bytes, 16-byte aligned.
  */
 typedef struct ps_step_state {
     double cur_scale;           /* loss_scale; Python float semantics (binary64) */
@@ -86,7 +86,7 @@ typedef struct ps_step_state {
     uint32_t last_skipped;      /* what the latest ps_scaler_update decided */
     float beta1;
     float beta2;
-    float beta1_t_next;         /* beta1^t for t = adam_step + 1 */
+    float beta1_t_next;         /* beta1^t that the FIRST operator call of step t = adam_step + 1 uses */
     float beta2_t_next;
     uint32_t reserved[4];
     /* torch-formula arithmetic (PS_ARITH_TORCH): the Python floats behind the betas and the
@@ -95,7 +95,34 @@ typedef struct ps_step_state {
     double beta2_f64;
     double bias_correction1_next;
     double bias_correction2_next;
+    /* The native operator object as Adam_Optimizer::IncrementStep (cpu_adam.h:143-162) leaves it.  The
+     * reference calls the operator once per tensor with the same step number; only the first call of a
+     * step can continue the running float product (`_step + 1 == step`), every later call of the step
+     * evaluates pow. */
+    int64_t operator_step;      /* its _step: the step number of its latest call (0: never called) */
+    float beta1_t_cur;          /* its _betta1_t / _betta2_t after that call */
+    float beta2_t_cur;
+    float beta1_t_rest;         /* (float)pow((double)beta, adam_step + 1): what every operator call */
+    float beta2_t_rest;         /* of step adam_step + 1 after the first one uses */
+    uint32_t reserved2[2];
 } ps_step_state;
+
+/*
+ * How the reference would have cut one step over a chunk list into operator calls.  FP16Adam calls
+ * adam_update once per trainable tensor, in param_groups order, all with the same step number
+ * (patrickstar/ops/fp16_cpu_adam.py:336-428), and Adam_Optimizer::IncrementStep (cpu_adam.h:143-162)
+ * gives the first of those calls the running float product beta^t and every later one
+ * (float)pow(beta, t).  The two differ in the last bits (1 / sqrt(1 - beta2^t) by up to 1e-5
+ * relative at small t), so a fused pass over whole chunks has to know which elements the first call
+ * covered.  Only the operator's arithmetic looks at this; the torch formula has no such state.
+ */
+typedef struct ps_call_pattern {
+    int64_t n_calls;       /* operator calls of the step over this list = its trainable tensors (>= 1) */
+    int64_t first_chunk;   /* index of the chunk that holds the first call's tensor (ps_adam_step_hybrid:
+                              chunks[] counted first, host_chunks[] after them) */
+    uint64_t first_offset; /* element offset of that tensor inside its chunk */
+    uint64_t first_numel;  /* its length in elements */
+} ps_call_pattern;
 
 /* One entry of the optional per-iteration log written by ps_scaler_update. */
 typedef struct ps_scale_record {
@@ -177,18 +204,18 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
 int ps_adam_step_chunks(int optimizer_id, size_t step, double lr, double beta1, double beta2,
                         double epsilon, double weight_decay, int bias_correction,
                         const ps_chunk* chunks, int n_chunks, size_t chunk_numel,
-                        double loss_scale, ps_stream_t stream);
+                        const ps_call_pattern* calls, double loss_scale, ps_stream_t stream);
 
 /* Same pass, decided on the device: if d_state->overflow is set, every chunk's
  * fp16 payload is restored from the fp32 master copy (fp16_cpu_adam.py:298-309)
  * and nothing else changes; otherwise the Adam update runs with
- * loss_scale = d_state->cur_scale and t = d_state->adam_step + 1 (beta^t, or
- * the binary64 bias corrections of the torch arithmetic, from d_state).  Follow
- * with ps_scaler_update(..., PS_FLAG_FROM_DEVICE). */
+ * loss_scale = d_state->cur_scale and t = d_state->adam_step + 1 (beta^t of the first and of the
+ * later operator calls, or the binary64 bias corrections of the torch arithmetic, from d_state).
+ * Follow with ps_scaler_update(..., PS_FLAG_FROM_DEVICE, ..., calls ? calls->n_calls : 1). */
 int ps_adam_step_chunks_gated(int optimizer_id, double lr, double epsilon, double weight_decay,
                               int bias_correction, const ps_chunk* chunks, int n_chunks,
-                              size_t chunk_numel, const ps_step_state* d_state,
-                              ps_stream_t stream);
+                              size_t chunk_numel, const ps_call_pattern* calls,
+                              const ps_step_state* d_state, ps_stream_t stream);
 
 /* The per-tensor loop of FP16Adam.fp16_chunk_adam_ops (fp16_cpu_adam.py:336-468) as ONE call, for chunk layouts
  * in which a parameter's exp_avg / exp_avg_sq do not sit at the parameter's own offset inside their chunks (the
@@ -198,8 +225,10 @@ int ps_adam_step_chunks_gated(int optimizer_id, double lr, double epsilon, doubl
  *               (gradient in, fp16 parameter out), numels[i] elements each; both are host arrays
  *   d_state     NULL: host-decided step with loss_scale; else device-gated like ps_adam_step_chunks_gated
  *               (step, betas and loss_scale ignored; a flagged step restores the fp16 slots from fp32)
- * Same arithmetic, clamp and 28 B/element as the chunk-list form; the operator's step scalars advance once
- * for the call.  Up to 48 tensors go into one launch. */
+ * Same arithmetic, clamp and 28 B/element as the chunk-list form.  Every tensor is one operator call of the
+ * reference's loop, tensors[0] the first of the step (zero-length tensors included: the reference calls the
+ * operator for them too); follow a device-gated call with ps_scaler_update(..., n_tensors).
+ * Up to 48 tensors go into one launch. */
 int ps_adam_step_tensors(int optimizer_id, size_t step, double lr, double beta1, double beta2,
                          double epsilon, double weight_decay, int bias_correction,
                          const ps_chunk* tensors, const size_t* numels, int n_tensors,
@@ -230,8 +259,10 @@ int ps_restore_fp16_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_nu
  *   staging      host array of n_slots (1..8) descriptors of DEVICE buffers of
  *                chunk_numel elements each, owned by the caller; param_fp16 may be NULL when
  *                every host chunk keeps its fp16 payload in HBM
- *   d_state      NULL: host-decided step with loss_scale, the operator's step scalars
- *                advanced ONCE for both lists; else device-gated exactly like
+ *   calls        as for ps_adam_step_chunks, over chunks[] followed by host_chunks[]; with
+ *                PS_ARITH_TORCH only host_chunks[] reach the operator and the pattern describes those
+ *                (first_chunk >= n_chunks).  NULL: one operator call for everything
+ *   d_state      NULL: host-decided step with loss_scale; else device-gated exactly like
  *                ps_adam_step_chunks_gated (step, betas and loss_scale ignored)
  * Work queued on `stream` before the call is waited for; work queued on it
  * afterwards waits for the last write-back.  The call itself never blocks.
@@ -240,7 +271,8 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, 
                         double epsilon, double weight_decay, int bias_correction,
                         const ps_chunk* chunks, int n_chunks, const ps_chunk* host_chunks,
                         int n_host_chunks, size_t chunk_numel, const ps_chunk* staging, int n_slots,
-                        double loss_scale, const ps_step_state* d_state, ps_stream_t stream);
+                        const ps_call_pattern* calls, double loss_scale, const ps_step_state* d_state,
+                        ps_stream_t stream);
 
 /* The inf/nan probe for host-resident chunks: only the fp16 payloads are
  * streamed (2 B/element) through staging[i].param_fp16; fp16 payloads that
@@ -263,12 +295,18 @@ int ps_state_init(ps_step_state* d_state, double init_scale, int init_is_int, do
                   int delayed_shift, int consecutive_hysteresis, double beta1, double beta2,
                   ps_stream_t stream);
 
-/* Set the Adam step counter (load_state_dict, fp16_cpu_adam.py:660-694) and
- * betas; the operator's beta^t for the next step is pow((float)beta, adam_step + 1)
- * evaluated in double on the host and narrowed, i.e. the reference's cold branch;
- * the torch arithmetic's bias corrections are 1 - pow(beta, adam_step + 1). */
+/* Set the Adam step counter (load_state_dict, fp16_cpu_adam.py:660-694) and betas.
+ *   fresh_operator != 0  a new operator object stands behind them (step 0, beta^t = 1, as create_adam leaves
+ *                        it): its first call, for step adam_step + 1, multiplies only if adam_step is 0 and
+ *                        otherwise evaluates pow((float)beta, adam_step + 1) in double and narrows, i.e. the
+ *                        reference's cold branch;
+ *   fresh_operator == 0  the operator object is the one that has been running (the reference's
+ *                        load_state_dict does not touch it): the first call of step adam_step + 1
+ *                        continues its running product only if its own step is adam_step and the betas are
+ *                        unchanged, as IncrementStep decides (cpu_adam.h:143-162).
+ * The torch arithmetic's bias corrections become 1 - pow(beta, adam_step + 1). */
 int ps_state_seed_step(ps_step_state* d_state, int64_t adam_step, double beta1, double beta2,
-                       ps_stream_t stream);
+                       int fresh_operator, ps_stream_t stream);
 
 /* Overwrite the loss-scaler fields only (restoring a checkpointed scaler). */
 int ps_state_set_scaler(ps_step_state* d_state, double cur_scale, int scale_is_int,
@@ -298,13 +336,16 @@ int ps_grad_to_chunk(const void* d_grad, int grad_is_half, uint16_t* d_slot_fp16
 #define PS_FLAG_FROM_DEVICE 2
 /* DynamicLossScaler.update_scale (loss_scaler.py:158-182) on the device.
  * flag_mode chooses the `overflow` argument: a host-given bool or the sticky
- * device flag.  A clean step also advances adam_step, beta^t (the float
- * running product of cpu_adam.h:158-159) and the binary64 bias corrections of
- * the torch arithmetic.  Clears the sticky flag.  If d_log
+ * device flag.  A clean step also advances adam_step, the operator's beta^t
+ * state (cpu_adam.h:143-162) and the binary64 bias corrections of
+ * the torch arithmetic.  operator_calls says how often the step that was just
+ * queued called the operator in the reference's terms: the n_calls of its
+ * ps_call_pattern (1 without one, the tensor count of ps_adam_step_tensors, 0 if
+ * every chunk took the torch formula).  Clears the sticky flag.  If d_log
  * is not NULL, entry [cur_iter % log_capacity] (cur_iter before the
  * increment) records the decision. */
 int ps_scaler_update(ps_step_state* d_state, int flag_mode, ps_scale_record* d_log,
-                     int64_t log_capacity, ps_stream_t stream);
+                     int64_t log_capacity, int64_t operator_calls, ps_stream_t stream);
 
 /* Copy *d_state to host memory and wait for it: the only synchronising call. */
 int ps_state_read(const ps_step_state* d_state, ps_step_state* host_out, ps_stream_t stream);

@@ -11,7 +11,7 @@ LIB_PATH = os.path.join(PKG_DIR, "libps_adam.so")
 PS_FLAG_FALSE, PS_FLAG_TRUE, PS_FLAG_FROM_DEVICE = 0, 1, 2
 PS_ERR_BAD_ARG, PS_ERR_UNKNOWN_ID, PS_ERR_NO_DEVICE = -10001, -10002, -10003
 PS_ARITH_OPERATOR, PS_ARITH_TORCH = 0, 1
-PS_ABI_VERSION = 2
+PS_ABI_VERSION = 3
 
 
 class ps_chunk(ctypes.Structure):
@@ -50,6 +50,21 @@ class ps_step_state(ctypes.Structure):
         ("beta2_f64", ctypes.c_double),
         ("bias_correction1_next", ctypes.c_double),
         ("bias_correction2_next", ctypes.c_double),
+        ("operator_step", ctypes.c_int64),
+        ("beta1_t_cur", ctypes.c_float),
+        ("beta2_t_cur", ctypes.c_float),
+        ("beta1_t_rest", ctypes.c_float),
+        ("beta2_t_rest", ctypes.c_float),
+        ("reserved2", ctypes.c_uint32 * 2),
+    ]
+
+
+class ps_call_pattern(ctypes.Structure):
+    _fields_ = [
+        ("n_calls", ctypes.c_int64),
+        ("first_chunk", ctypes.c_int64),
+        ("first_offset", ctypes.c_uint64),
+        ("first_numel", ctypes.c_uint64),
     ]
 
 
@@ -62,7 +77,8 @@ class ps_scale_record(ctypes.Structure):
 
 
 assert ctypes.sizeof(ps_chunk) == 32
-assert ctypes.sizeof(ps_step_state) == 160
+assert ctypes.sizeof(ps_step_state) == 192
+assert ctypes.sizeof(ps_call_pattern) == 32
 assert ctypes.sizeof(ps_scale_record) == 16
 
 _f, _d, _i, _i64, _sz, _vp = (
@@ -83,21 +99,21 @@ SIGNATURES = {
     "ps_adam_set_arithmetic": (_i, [_i, _i]),
     "ps_adam_destroy": (_i, [_i]),
     "ps_adam_update": (_i, [_i, _sz, _f, _f, _f, _f, _f, _i, _vp, _vp, _i, _vp, _vp, _sz, _f, _vp, _vp]),
-    "ps_adam_step_chunks": (_i, [_i, _sz, _d, _d, _d, _d, _d, _i, _vp, _i, _sz, _d, _vp]),
-    "ps_adam_step_chunks_gated": (_i, [_i, _d, _d, _d, _i, _vp, _i, _sz, _vp, _vp]),
+    "ps_adam_step_chunks": (_i, [_i, _sz, _d, _d, _d, _d, _d, _i, _vp, _i, _sz, _vp, _d, _vp]),
+    "ps_adam_step_chunks_gated": (_i, [_i, _d, _d, _d, _i, _vp, _i, _sz, _vp, _vp, _vp]),
     "ps_adam_step_tensors": (_i, [_i, _sz, _d, _d, _d, _d, _d, _i, _vp, _vp, _i, _d, _vp, _vp]),
-    "ps_adam_step_hybrid": (_i, [_i, _sz, _d, _d, _d, _d, _d, _i, _vp, _i, _vp, _i, _sz, _vp, _i, _d, _vp, _vp]),
+    "ps_adam_step_hybrid": (_i, [_i, _sz, _d, _d, _d, _d, _d, _i, _vp, _i, _vp, _i, _sz, _vp, _i, _vp, _d, _vp, _vp]),
     "ps_overflow_scan_host_chunks": (_i, [_vp, _i, _sz, _vp, _i, _vp, _vp]),
     "ps_restore_fp16_chunks": (_i, [_vp, _i, _sz, _vp, _vp]),
     "ps_cast_fp32_to_fp16": (_i, [_vp, _vp, _sz, _vp]),
     "ps_state_init": (_i, [_vp, _d, _i, _d, _i, _i64, _d, _i, _i, _i, _d, _d, _vp]),
-    "ps_state_seed_step": (_i, [_vp, _i64, _d, _d, _vp]),
+    "ps_state_seed_step": (_i, [_vp, _i64, _d, _d, _i, _vp]),
     "ps_state_set_scaler": (_i, [_vp, _d, _i, _i64, _i64, _i, _vp]),
     "ps_overflow_scan": (_i, [_vp, _sz, _vp, _vp]),
     "ps_overflow_scan_f32": (_i, [_vp, _sz, _vp, _vp]),
     "ps_overflow_scan_chunks": (_i, [_vp, _i, _sz, _vp, _vp]),
     "ps_grad_to_chunk": (_i, [_vp, _i, _vp, _sz, _vp, _vp]),
-    "ps_scaler_update": (_i, [_vp, _i, _vp, _i64, _vp]),
+    "ps_scaler_update": (_i, [_vp, _i, _vp, _i64, _i64, _vp]),
     "ps_state_read": (_i, [_vp, ctypes.POINTER(ps_step_state), _vp]),
 }
 
@@ -142,6 +158,11 @@ def current_stream_handle():
     import torch
 
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def call_pattern(n_calls, first_chunk=0, first_offset=0, first_numel=0):
+    """A ps_call_pattern, by reference, for the `calls` argument of the step entry points."""
+    return ctypes.byref(ps_call_pattern(int(n_calls), int(first_chunk), int(first_offset), int(first_numel)))
 
 
 def chunk_array(rows):

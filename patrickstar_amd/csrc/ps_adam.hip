@@ -169,7 +169,7 @@ int make_chunk_list(ChunkList& a, const ps_chunk* chunks, int n_chunks, size_t c
     return 0;
 }
 
-// Calls launch(batch, n_in_batch, grid) for every group of up to kBatch chunks.
+// Calls launch(batch, grid, index of the batch's first chunk) for every group of up to kBatch chunks.
 template <typename F>
 int for_each_batch(const ChunkList& a, F launch)
 {
@@ -179,69 +179,111 @@ int for_each_batch(const ChunkList& a, F launch)
         ChunkBatch b;
         memset(&b, 0, sizeof(b));
         for (int i = 0; i < n; ++i) b.c[i] = a.chunks[first + i];
-        launch(b, dim3((unsigned)a.tiles_per_chunk, (unsigned)n));
+        launch(b, dim3((unsigned)a.tiles_per_chunk, (unsigned)n), first);
         PS_HIP(hipGetLastError());
     }
     return 0;
 }
 
+// Validated copy of a ps_call_pattern: how many operator calls the reference makes in the step and
+// which elements its first call covers, as a chunk index over the call's whole list.
+struct Calls {
+    int64_t n_calls = 1;
+    int64_t first_chunk = -1;  // -1: the first call's span is not needed (one call, or no elements)
+    uint64_t lo = 0, hi = 0;
+
+    // The span as the launch of chunks [batch_first, batch_first + n) sees it.
+    FirstCall in_batch(int64_t batch_first, int n) const
+    {
+        FirstCall fc{-1, 0, 0};
+        if (first_chunk >= batch_first && first_chunk < batch_first + n) {
+            fc.chunk = (int)(first_chunk - batch_first);
+            fc.lo = lo;
+            fc.hi = hi;
+        }
+        return fc;
+    }
+};
+
+int make_calls(Calls& out, const ps_call_pattern* calls, int64_t n_chunks_total, size_t chunk_numel)
+{
+    out = Calls();
+    if (calls == nullptr) return 0;
+    if (calls->n_calls < 1) return fail(PS_ERR_BAD_ARG, "calls->n_calls = %lld must be at least 1", (long long)calls->n_calls);
+    out.n_calls = calls->n_calls;
+    if (calls->n_calls == 1 || calls->first_numel == 0) return 0;  // one call, or a first call without elements
+    if (calls->first_chunk < 0 || calls->first_chunk >= n_chunks_total)
+        return fail(PS_ERR_BAD_ARG, "calls->first_chunk = %lld is outside the list of %lld chunks",
+                    (long long)calls->first_chunk, (long long)n_chunks_total);
+    if (calls->first_offset > chunk_numel || calls->first_numel > chunk_numel - calls->first_offset)
+        return fail(PS_ERR_BAD_ARG, "the first call's tensor (offset %llu, %llu elements) does not fit a chunk of %zu",
+                    (unsigned long long)calls->first_offset, (unsigned long long)calls->first_numel, chunk_numel);
+    out.first_chunk = calls->first_chunk;
+    out.lo = calls->first_offset;
+    out.hi = calls->first_offset + calls->first_numel;
+    return 0;
+}
+
 template <int ARITH, int WD>
 void launch_adam_batch_wd(const ChunkBatch& b, dim3 grid, size_t chunk_numel, const StepConsts& c,
-                          hipStream_t s)
+                          const FirstCall& fc, hipStream_t s)
 {
     dim3 block(kBlock);
     if (c.unscale == UNSCALE_MUL)
-        hipLaunchKernelGGL((adam_chunks_kernel<ARITH, WD, UNSCALE_MUL>), grid, block, kLdsBytes, s, b, chunk_numel, c);
+        hipLaunchKernelGGL((adam_chunks_kernel<ARITH, WD, UNSCALE_MUL>), grid, block, kLdsBytes, s, b, chunk_numel, c, fc);
     else if (ARITH == PS_ARITH_OPERATOR && c.unscale == UNSCALE_DIV)  // the torch formula never divides
-        hipLaunchKernelGGL((adam_chunks_kernel<ARITH, WD, UNSCALE_DIV>), grid, block, kLdsBytes, s, b, chunk_numel, c);
+        hipLaunchKernelGGL((adam_chunks_kernel<ARITH, WD, UNSCALE_DIV>), grid, block, kLdsBytes, s, b, chunk_numel, c, fc);
     else
-        hipLaunchKernelGGL((adam_chunks_kernel<ARITH, WD, UNSCALE_NONE>), grid, block, kLdsBytes, s, b, chunk_numel, c);
+        hipLaunchKernelGGL((adam_chunks_kernel<ARITH, WD, UNSCALE_NONE>), grid, block, kLdsBytes, s, b, chunk_numel, c, fc);
 }
 
 template <int ARITH>
 void launch_adam_batch_arith(const ChunkBatch& b, dim3 grid, size_t chunk_numel,
-                             const StepConsts& c, hipStream_t s)
+                             const StepConsts& c, const FirstCall& fc, hipStream_t s)
 {
     if (c.wd_mode == WD_DECOUPLED)
-        launch_adam_batch_wd<ARITH, WD_DECOUPLED>(b, grid, chunk_numel, c, s);
+        launch_adam_batch_wd<ARITH, WD_DECOUPLED>(b, grid, chunk_numel, c, fc, s);
     else if (c.wd_mode == WD_L2)
-        launch_adam_batch_wd<ARITH, WD_L2>(b, grid, chunk_numel, c, s);
+        launch_adam_batch_wd<ARITH, WD_L2>(b, grid, chunk_numel, c, fc, s);
     else
-        launch_adam_batch_wd<ARITH, WD_NONE>(b, grid, chunk_numel, c, s);
+        launch_adam_batch_wd<ARITH, WD_NONE>(b, grid, chunk_numel, c, fc, s);
 }
 
-// `c` must have been built for `arith` (finish_consts / torch_consts).
+// `c` must have been built for `arith` (finish_consts / torch_consts).  `fc`: which elements of the
+// batch the step's first operator call covers; the torch formula has no such distinction.
 void launch_adam_batch(int arith, const ChunkBatch& b, dim3 grid, size_t chunk_numel,
-                       const StepConsts& c, hipStream_t s)
+                       const StepConsts& c, const FirstCall& fc, hipStream_t s)
 {
     if (arith == PS_ARITH_TORCH)
-        launch_adam_batch_arith<PS_ARITH_TORCH>(b, grid, chunk_numel, c, s);
+        launch_adam_batch_arith<PS_ARITH_TORCH>(b, grid, chunk_numel, c, FirstCall{-1, 0, 0}, s);
     else
-        launch_adam_batch_arith<PS_ARITH_OPERATOR>(b, grid, chunk_numel, c, s);
+        launch_adam_batch_arith<PS_ARITH_OPERATOR>(b, grid, chunk_numel, c, fc, s);
 }
 
 template <int ARITH>
 void launch_gated_batch_arith(const ChunkBatch& b, dim3 grid, size_t chunk_numel,
-                              const GatedArgs& ga, const ps_step_state* d_state, hipStream_t s)
+                              const GatedArgs& ga, const FirstCall& fc, const ps_step_state* d_state,
+                              hipStream_t s)
 {
     dim3 block(kBlock);
     // the operator tests its float weight decay "> 0" (cpu_adam.cpp:42), the torch formula "!= 0"
     const bool decay = ARITH == PS_ARITH_OPERATOR ? (float)ga.wd > 0.0f : ga.wd != 0.0;
     if (decay && ga.adamw)
-        hipLaunchKernelGGL((adam_chunks_gated_kernel<ARITH, WD_DECOUPLED>), grid, block, kLdsBytes, s, b, chunk_numel, ga, d_state);
+        hipLaunchKernelGGL((adam_chunks_gated_kernel<ARITH, WD_DECOUPLED>), grid, block, kLdsBytes, s, b, chunk_numel, ga, fc, d_state);
     else if (decay)
-        hipLaunchKernelGGL((adam_chunks_gated_kernel<ARITH, WD_L2>), grid, block, kLdsBytes, s, b, chunk_numel, ga, d_state);
+        hipLaunchKernelGGL((adam_chunks_gated_kernel<ARITH, WD_L2>), grid, block, kLdsBytes, s, b, chunk_numel, ga, fc, d_state);
     else
-        hipLaunchKernelGGL((adam_chunks_gated_kernel<ARITH, WD_NONE>), grid, block, kLdsBytes, s, b, chunk_numel, ga, d_state);
+        hipLaunchKernelGGL((adam_chunks_gated_kernel<ARITH, WD_NONE>), grid, block, kLdsBytes, s, b, chunk_numel, ga, fc, d_state);
 }
 
 void launch_gated_batch(int arith, const ChunkBatch& b, dim3 grid, size_t chunk_numel,
-                        const GatedArgs& ga, const ps_step_state* d_state, hipStream_t s)
+                        const GatedArgs& ga, const FirstCall& fc, const ps_step_state* d_state,
+                        hipStream_t s)
 {
     if (arith == PS_ARITH_TORCH)
-        launch_gated_batch_arith<PS_ARITH_TORCH>(b, grid, chunk_numel, ga, d_state, s);
+        launch_gated_batch_arith<PS_ARITH_TORCH>(b, grid, chunk_numel, ga, FirstCall{-1, 0, 0}, d_state, s);
     else
-        launch_gated_batch_arith<PS_ARITH_OPERATOR>(b, grid, chunk_numel, ga, d_state, s);
+        launch_gated_batch_arith<PS_ARITH_OPERATOR>(b, grid, chunk_numel, ga, fc, d_state, s);
 }
 
 template <int ARITH, int WD>
@@ -289,14 +331,18 @@ struct HyperParams {
 };
 
 // Host-decided step, operator arithmetic: narrow like the pybind signature of adam_update
-// (float arguments, cpu_adam.cpp:700-712), advance the operator's step scalars, derive the rest.
-StepConsts operator_step_consts(HostAdam& o, size_t step, const HyperParams& hp)
+// (float arguments, cpu_adam.cpp:700-712) and take the operator object through the n_calls
+// adam_update calls of the reference's per-tensor loop, all with this step number: the first call's
+// beta^t, then (from the second call on the object no longer moves) every later call's.
+StepConsts operator_step_consts(HostAdam& o, size_t step, const HyperParams& hp, int64_t n_calls)
 {
     o.advance(step, (float)hp.beta1, (float)hp.beta2);
+    const float first_b1t = o.beta1_t, first_b2t = o.beta2_t;
+    if (n_calls >= 2) o.advance(step, (float)hp.beta1, (float)hp.beta2);
     o.set((float)hp.lr, (float)hp.eps, (float)hp.wd);
     StepConsts c;
     finish_consts(c, o.alpha, o.beta1, o.beta2, o.eps, o.weight_decay, o.adamw, o.beta1_t,
-                  o.beta2_t, hp.bias_correction, (float)hp.loss_scale,
+                  o.beta2_t, first_b1t, first_b2t, hp.bias_correction, (float)hp.loss_scale,
                   clamp_bound(o.grad_clamp, hp.loss_scale));
     return c;
 }
@@ -316,13 +362,15 @@ StepConsts torch_step_consts(const HostAdam& o, size_t step, const HyperParams& 
     return c;
 }
 
-GatedArgs gated_args(const HostAdam& o, double lr, double eps, double wd, int bias_correction)
+GatedArgs gated_args(const HostAdam& o, double lr, double eps, double wd, int bias_correction,
+                     int64_t n_calls)
 {
     GatedArgs ga;
     ga.lr = lr;
     ga.eps = eps;
     ga.wd = wd;
     ga.grad_clamp = o.grad_clamp;
+    ga.n_calls = n_calls;
     ga.adamw = o.adamw ? 1 : 0;
     ga.bias_correction = bias_correction;
     return ga;
@@ -514,7 +562,7 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
     StepConsts c;
     // the reference clamps gradients in Python before it calls the operator: not here
     finish_consts(c, o->alpha, o->beta1, o->beta2, o->eps, o->weight_decay, o->adamw, o->beta1_t,
-                  o->beta2_t, bias_correction != 0, loss_scale, 0.0f);
+                  o->beta2_t, o->beta1_t, o->beta2_t, bias_correction != 0, loss_scale, 0.0f);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const size_t gsz = grads_are_half ? 2 : 4;
     const char* gbytes = static_cast<const char*>(d_grads);
@@ -585,40 +633,44 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
 int ps_adam_step_chunks(int optimizer_id, size_t step, double lr, double beta1, double beta2,
                         double epsilon, double weight_decay, int bias_correction,
                         const ps_chunk* chunks, int n_chunks, size_t chunk_numel,
-                        double loss_scale, ps_stream_t stream)
+                        const ps_call_pattern* calls, double loss_scale, ps_stream_t stream)
 {
     auto o = find_opt(optimizer_id);
     if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
     ChunkList a;
     if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, kTile)) return rc;
+    Calls k;
+    if (int rc = make_calls(k, calls, n_chunks, chunk_numel)) return rc;
     const HyperParams hp{lr, beta1, beta2, epsilon, weight_decay, loss_scale, bias_correction != 0};
     StepConsts c;
     if (o->arith == PS_ARITH_TORCH)
         c = torch_step_consts(*o, step, hp);
     else
-        c = operator_step_consts(*o, step, hp);
+        c = operator_step_consts(*o, step, hp, k.n_calls);
     const int arith = o->arith;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid) {
-        launch_adam_batch(arith, b, grid, chunk_numel, c, s);
+    return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid, int first) {
+        launch_adam_batch(arith, b, grid, chunk_numel, c, k.in_batch(first, (int)grid.y), s);
     });
 }
 
 int ps_adam_step_chunks_gated(int optimizer_id, double lr, double epsilon, double weight_decay,
                               int bias_correction, const ps_chunk* chunks, int n_chunks,
-                              size_t chunk_numel, const ps_step_state* d_state,
-                              ps_stream_t stream)
+                              size_t chunk_numel, const ps_call_pattern* calls,
+                              const ps_step_state* d_state, ps_stream_t stream)
 {
     auto o = find_opt(optimizer_id);
     if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
     if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
     ChunkList a;
     if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, kTile)) return rc;
-    const GatedArgs ga = gated_args(*o, lr, epsilon, weight_decay, bias_correction);
+    Calls k;
+    if (int rc = make_calls(k, calls, n_chunks, chunk_numel)) return rc;
+    const GatedArgs ga = gated_args(*o, lr, epsilon, weight_decay, bias_correction, k.n_calls);
     const int arith = o->arith;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid) {
-        launch_gated_batch(arith, b, grid, chunk_numel, ga, d_state, s);
+    return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid, int first) {
+        launch_gated_batch(arith, b, grid, chunk_numel, ga, k.in_batch(first, (int)grid.y), d_state, s);
     });
 }
 
@@ -639,11 +691,12 @@ int ps_adam_step_tensors(int optimizer_id, size_t step, double lr, double beta1,
             return fail(PS_ERR_BAD_ARG, "tensor %d: numel = %zu is beyond the launch grid", i, numels[i]);
     }
     const int arith = o->arith;
+    // one operator call per tensor, tensors[0] the first of the step
     StepConsts c;
-    GatedArgs ga = gated_args(*o, lr, epsilon, weight_decay, bias_correction);
-    if (d_state == nullptr) {
+    GatedArgs ga = gated_args(*o, lr, epsilon, weight_decay, bias_correction, n_tensors);
+    if (d_state == nullptr && n_tensors > 0) {
         const HyperParams hp{lr, beta1, beta2, epsilon, weight_decay, loss_scale, bias_correction != 0};
-        c = arith == PS_ARITH_TORCH ? torch_step_consts(*o, step, hp) : operator_step_consts(*o, step, hp);
+        c = arith == PS_ARITH_TORCH ? torch_step_consts(*o, step, hp) : operator_step_consts(*o, step, hp, n_tensors);
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
     TensorBatch b;
@@ -666,14 +719,17 @@ int ps_adam_step_tensors(int optimizer_id, size_t step, double lr, double beta1,
         PS_HIP(hipGetLastError());
         in_batch = 0;
         tiles = 0;
+        b.first_call = -1;
         return 0;
     };
     memset(&b, 0, sizeof(b));
+    b.first_call = -1;
     for (int i = 0; i < n_tensors; ++i) {
         if (numels[i] == 0) continue;
         const size_t t_i = (numels[i] + kTile - 1) / kTile;
         if (in_batch == kTensorBatch || tiles + t_i > kMaxGridX)
             if (int rc = flush()) return rc;
+        if (i == 0 && arith == PS_ARITH_OPERATOR) b.first_call = in_batch;
         b.t[in_batch] = tensors[i];
         b.numel[in_batch] = numels[i];
         b.first_tile[in_batch] = (uint32_t)tiles;
@@ -689,7 +745,7 @@ int ps_restore_fp16_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_nu
     ChunkList a;
     if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, kTile)) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid) {
+    return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid, int) {
         hipLaunchKernelGGL(restore_chunks_kernel, grid, dim3(kBlock), 0, s, b, chunk_numel, d_state);
     });
 }
@@ -709,7 +765,8 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, 
                         double epsilon, double weight_decay, int bias_correction,
                         const ps_chunk* chunks, int n_chunks, const ps_chunk* host_chunks,
                         int n_host_chunks, size_t chunk_numel, const ps_chunk* staging, int n_slots,
-                        double loss_scale, const ps_step_state* d_state, ps_stream_t stream)
+                        const ps_call_pattern* calls, double loss_scale, const ps_step_state* d_state,
+                        ps_stream_t stream)
 {
     auto o = find_opt(optimizer_id);
     if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
@@ -725,14 +782,19 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, 
             if (int rc = check_slots(staging, n_slots, true, true)) return rc;
     }
     // Resident chunks take the optimizer's arithmetic, streamed host chunks the operator's (the
-    // reference updates those with the operator).  The operator's step scalars advance once for
-    // the whole list, and only if the operator's arithmetic is used at all.
+    // reference updates those with the operator).  The operator object goes through the calls of
+    // the pattern (over both lists), and only if the operator's arithmetic is used at all.
     const int arith = o->arith;
+    Calls k;
+    if (int rc = make_calls(k, calls, (int64_t)n_chunks + n_host_chunks, chunk_numel)) return rc;
+    if (arith == PS_ARITH_TORCH && k.first_chunk >= 0 && k.first_chunk < n_chunks)
+        return fail(PS_ERR_BAD_ARG, "calls->first_chunk = %lld names a resident chunk, which the torch arithmetic "
+                    "never hands to the operator", (long long)k.first_chunk);
     StepConsts c_resident, c_host;
-    const GatedArgs ga = gated_args(*o, lr, epsilon, weight_decay, bias_correction);
+    const GatedArgs ga = gated_args(*o, lr, epsilon, weight_decay, bias_correction, k.n_calls);
     if (d_state == nullptr) {
         const HyperParams hp{lr, beta1, beta2, epsilon, weight_decay, loss_scale, bias_correction != 0};
-        if (arith == PS_ARITH_OPERATOR || n_host_chunks > 0) c_host = operator_step_consts(*o, step, hp);
+        if (arith == PS_ARITH_OPERATOR || n_host_chunks > 0) c_host = operator_step_consts(*o, step, hp, k.n_calls);
         c_resident = arith == PS_ARITH_TORCH ? torch_step_consts(*o, step, hp) : c_host;
     }
     hipStream_t caller = static_cast<hipStream_t>(stream);
@@ -746,24 +808,25 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, 
         PS_HIP(hipStreamWaitEvent(p->h2d, p->entry, 0));
         PS_HIP(hipStreamWaitEvent(p->compute, p->entry, 0));
     }
-    int rc = for_each_batch(resident, [&](const ChunkBatch& b, dim3 grid) {
+    int rc = for_each_batch(resident, [&](const ChunkBatch& b, dim3 grid, int first) {
+        const FirstCall fc = k.in_batch(first, (int)grid.y);
         if (d_state == nullptr)
-            launch_adam_batch(arith, b, grid, chunk_numel, c_resident, caller);
+            launch_adam_batch(arith, b, grid, chunk_numel, c_resident, fc, caller);
         else
-            launch_gated_batch(arith, b, grid, chunk_numel, ga, d_state, caller);
+            launch_gated_batch(arith, b, grid, chunk_numel, ga, fc, d_state, caller);
     });
     if (rc) return rc;
     if (!stream_host) return 0;
 
     const size_t b32 = chunk_numel * sizeof(float), b16 = chunk_numel * sizeof(uint16_t);
     for (int i = 0; i < kMaxSlots; ++i) p->slot_used[i] = false;
-    auto stream_chunk = [&](int k) -> int {
-        const int s = k % n_slots;
-        const ps_chunk& h = host_chunks[k];
+    auto stream_chunk = [&](int k_host) -> int {
+        const int s = k_host % n_slots;
+        const ps_chunk& h = host_chunks[k_host];
         ps_chunk d = staging[s];
         // a fp16 payload that already lives in HBM is read and written in place: 12 instead of
         // 14 bytes per element cross the link in each direction
-        const bool stage_fp16 = !fp16_in_hbm[k];
+        const bool stage_fp16 = !fp16_in_hbm[k_host];
         if (!stage_fp16) d.param_fp16 = h.param_fp16;
         // the slot is free once its previous occupant has been written back
         if (p->slot_used[s]) PS_HIP(hipStreamWaitEvent(p->h2d, p->d2h_done[s], 0));
@@ -779,10 +842,11 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, 
         memset(&b, 0, sizeof(b));
         b.c[0] = d;
         dim3 grid((unsigned)host.tiles_per_chunk, 1);
+        const FirstCall fc = k.in_batch((int64_t)n_chunks + k_host, 1);
         if (d_state == nullptr)
-            launch_adam_batch(PS_ARITH_OPERATOR, b, grid, chunk_numel, c_host, p->compute);
+            launch_adam_batch(PS_ARITH_OPERATOR, b, grid, chunk_numel, c_host, fc, p->compute);
         else
-            launch_gated_batch(PS_ARITH_OPERATOR, b, grid, chunk_numel, ga, d_state, p->compute);
+            launch_gated_batch(PS_ARITH_OPERATOR, b, grid, chunk_numel, ga, fc, d_state, p->compute);
         PS_HIP(hipGetLastError());
         PS_HIP(hipEventRecord(p->compute_done[s], p->compute));
 
@@ -798,7 +862,7 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, 
         p->slot_used[s] = true;
         return 0;
     };
-    for (int k = 0; k < n_host_chunks && rc == 0; ++k) rc = stream_chunk(k);
+    for (int i = 0; i < n_host_chunks && rc == 0; ++i) rc = stream_chunk(i);
     // later work on the caller's stream sees every chunk written back (also if queuing stopped half way)
     const int joined = p->join(caller);
     return rc ? rc : joined;
@@ -880,8 +944,14 @@ int ps_state_init(ps_step_state* d_state, double init_scale, int init_is_int, do
     s.beta1 = (float)beta1;
     s.beta2 = (float)beta2;
     // Adam_Optimizer starts with beta^t = 1 and step 0; the first update multiplies once.
+    s.operator_step = 0;
+    s.beta1_t_cur = 1.0f;
+    s.beta2_t_cur = 1.0f;
     s.beta1_t_next = 1.0f * s.beta1;
     s.beta2_t_next = 1.0f * s.beta2;
+    // a second call of step 1 finds _step + 1 = 2 != 1 and evaluates pow(beta, 1)
+    s.beta1_t_rest = (float)std::pow((double)s.beta1, 1.0);
+    s.beta2_t_rest = (float)std::pow((double)s.beta2, 1.0);
     s.beta1_f64 = beta1;
     s.beta2_f64 = beta2;
     s.bias_correction1_next = 1.0 - std::pow(beta1, 1.0);
@@ -893,7 +963,7 @@ int ps_state_init(ps_step_state* d_state, double init_scale, int init_is_int, do
 }
 
 int ps_state_seed_step(ps_step_state* d_state, int64_t adam_step, double beta1, double beta2,
-                       ps_stream_t stream)
+                       int fresh_operator, ps_stream_t stream)
 {
     if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
     if (adam_step < 0) return fail(PS_ERR_BAD_ARG, "adam_step is negative");
@@ -901,14 +971,11 @@ int ps_state_seed_step(ps_step_state* d_state, int64_t adam_step, double beta1, 
     a.adam_step = adam_step;
     a.beta1 = (float)beta1;
     a.beta2 = (float)beta2;
-    if (adam_step == 0) {
-        a.b1t_next = 1.0f * a.beta1;
-        a.b2t_next = 1.0f * a.beta2;
-    } else {
-        // a fresh native object that is first asked for step adam_step + 1 takes the pow branch
-        a.b1t_next = (float)std::pow((double)a.beta1, (double)(adam_step + 1));
-        a.b2t_next = (float)std::pow((double)a.beta2, (double)(adam_step + 1));
-    }
+    // what a call for step adam_step + 1 gets when it cannot continue a running product; whether the
+    // first call of that step can is decided on the device, where the operator object's state lives
+    a.b1t_rest = (float)std::pow((double)a.beta1, (double)(adam_step + 1));
+    a.b2t_rest = (float)std::pow((double)a.beta2, (double)(adam_step + 1));
+    a.fresh_operator = fresh_operator != 0;
     a.beta1_f64 = beta1;
     a.beta2_f64 = beta2;
     a.bc1_next = 1.0 - std::pow(beta1, (double)(adam_step + 1));
@@ -964,7 +1031,7 @@ int ps_overflow_scan_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_n
     ChunkList a;
     if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, kScanTile)) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid) {
+    return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid, int) {
         hipLaunchKernelGGL(scan_chunks_kernel, grid, dim3(kAuxBlock), 0, s, b, chunk_numel, d_state);
     });
 }
@@ -1020,14 +1087,16 @@ int ps_grad_to_chunk(const void* d_grad, int grad_is_half, uint16_t* d_slot_fp16
 }
 
 int ps_scaler_update(ps_step_state* d_state, int flag_mode, ps_scale_record* d_log,
-                     int64_t log_capacity, ps_stream_t stream)
+                     int64_t log_capacity, int64_t operator_calls, ps_stream_t stream)
 {
     if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
     if (flag_mode < 0 || flag_mode > 2) return fail(PS_ERR_BAD_ARG, "flag_mode = %d", flag_mode);
     if (d_log != nullptr && log_capacity <= 0)
         return fail(PS_ERR_BAD_ARG, "log_capacity must be positive when d_log is given");
+    if (operator_calls < 0) return fail(PS_ERR_BAD_ARG, "operator_calls = %lld is negative", (long long)operator_calls);
     hipLaunchKernelGGL(scaler_update_kernel, dim3(1), dim3(64), 0,
-                       static_cast<hipStream_t>(stream), d_state, flag_mode, d_log, log_capacity);
+                       static_cast<hipStream_t>(stream), d_state, flag_mode, d_log, log_capacity,
+                       operator_calls);
     PS_HIP(hipGetLastError());
     return 0;
 }

@@ -20,8 +20,15 @@ enum Unscale { UNSCALE_NONE = 0, UNSCALE_DIV = 1, UNSCALE_MUL = 2 };
 constexpr int UNSCALE_RUNTIME = -1;  // template value: look at StepConsts::unscale (uniform branch)
 
 // Per-launch constants (cpu_adam.cpp:39-46 and the SIMD_SET block at :55-77).
+//
+// The reference calls the operator once per tensor with the same step number, and
+// Adam_Optimizer::IncrementStep (cpu_adam.h:143-162) lets only the FIRST call of a step continue the
+// running float product beta^t; every later call of the step evaluates pow.  The two bias-correction
+// scalars therefore exist twice: step_size / bc2inv for every call after the first, first_step_size /
+// first_bc2inv for the elements of the first call's tensor (FirstCall below says which those are).
 struct StepConsts {
     float beta1, beta2, b1m, b2m, bc2inv, eps, step_size, wd_term;
+    float first_step_size, first_bc2inv;
     float scale;  // loss scale (UNSCALE_DIV) or its exact reciprocal (UNSCALE_MUL)
     float clip;   // element-wise clamp bound of the fp16 gradients (an fp16-representable value); 0 = off
     int wd_mode;
@@ -79,25 +86,35 @@ __host__ __device__ inline bool exact_reciprocal(float s, float* inv)
     return true;
 }
 
-__host__ __device__ inline void finish_consts(StepConsts& c, float lr, float beta1, float beta2,
-                                              float eps, float wd, bool adamw, float beta1_t,
-                                              float beta2_t, bool bias_correction,
-                                              float loss_scale, float clip)
+// cpu_adam.h:170-174 and cpu_adam.cpp:44: the two scalars that depend on beta^t.
+__host__ __device__ inline void bias_scalars(float lr, float beta1_t, float beta2_t, bool bias_correction,
+                                             float* step_size, float* bc2inv_out)
 {
-    c.clip = clip;
-    // cpu_adam.h:170-174
     float bc1 = 1.0f, bc2inv = 1.0f;
     if (bias_correction) {
         bc1 = 1.0f - beta1_t;
         bc2inv = 1.0f / sqrtf(1.0f - beta2_t);
     }
+    *step_size = (-1.0f * lr) / bc1;
+    *bc2inv_out = bc2inv;
+}
+
+// beta1_t / beta2_t: beta^t of the calls after the first; first_beta1_t / first_beta2_t: of the first call.
+__host__ __device__ inline void finish_consts(StepConsts& c, float lr, float beta1, float beta2,
+                                              float eps, float wd, bool adamw, float beta1_t,
+                                              float beta2_t, float first_beta1_t, float first_beta2_t,
+                                              bool bias_correction, float loss_scale, float clip)
+{
+    c.clip = clip;
+    float bc2inv;
+    bias_scalars(lr, beta1_t, beta2_t, bias_correction, &c.step_size, &bc2inv);
+    bias_scalars(lr, first_beta1_t, first_beta2_t, bias_correction, &c.first_step_size, &c.first_bc2inv);
     c.beta1 = beta1;
     c.beta2 = beta2;
     c.b1m = 1.0f - beta1;
     c.b2m = 1.0f - beta2;
     c.bc2inv = bc2inv;
     c.eps = eps;
-    c.step_size = (-1.0f * lr) / bc1;
     c.wd_mode = wd > 0.0f ? (adamw ? WD_DECOUPLED : WD_L2) : WD_NONE;
     c.wd_term = adamw ? (-1.0f * lr) * wd : wd;
     c.unscale = UNSCALE_NONE;
@@ -130,6 +147,8 @@ __host__ __device__ inline void torch_consts(StepConsts& c, double lr, double be
     c.bc2inv = (float)(1.0 / sqrt(bc2));  // exp_avg_sq.sqrt() / math.sqrt(bias_correction2)
     c.eps = (float)eps;              // .add_(eps)
     c.step_size = (float)(-(lr / bc1));   // addcdiv_(..., value=-step_size)
+    c.first_step_size = c.step_size;      // Python forms these per tensor from the same step: no first-call form
+    c.first_bc2inv = c.bc2inv;
     c.wd_mode = wd != 0.0 ? (adamw ? WD_DECOUPLED : WD_L2) : WD_NONE;
     c.wd_term = adamw ? (float)(1.0 - lr * wd)  // data.mul_(1 - lr * weight_decay)
                       : (float)wd;              // grad.add(data, alpha=weight_decay)
@@ -141,9 +160,10 @@ __host__ __device__ inline void torch_consts(StepConsts& c, double lr, double be
     }
 }
 
+// step_size / bc2inv are arguments of their own: the caller picks the first call's pair or the later calls'.
 template <int ARITH, int WD, int UNS>
-__device__ __forceinline__ void adam_element(const StepConsts& c, float g, float& p, float& m,
-                                             float& v)
+__device__ __forceinline__ void adam_element(const StepConsts& c, float step_size, float bc2inv, float g,
+                                             float& p, float& m, float& v)
 {
     // element-wise clamp of the fp16 gradient (comparisons, so a NaN stays a NaN like Tensor.clamp_)
     if (c.clip > 0.0f) g = g < -c.clip ? -c.clip : (g > c.clip ? c.clip : g);
@@ -158,10 +178,10 @@ __device__ __forceinline__ void adam_element(const StepConsts& c, float g, float
         float gg = g * g;
         v = __builtin_fmaf(gg, c.b2m, v);
         float d = __builtin_sqrtf(v);
-        d = __builtin_fmaf(d, c.bc2inv, c.eps);
+        d = __builtin_fmaf(d, bc2inv, c.eps);
         float u = m / d;
         if (WD == WD_DECOUPLED) p = __builtin_fmaf(p, c.wd_term, p);
-        p = __builtin_fmaf(u, c.step_size, p);
+        p = __builtin_fmaf(u, step_size, p);
     } else {
         // FP16Adam.torch_adam_update, fp16_cpu_adam.py:259-277, one torch kernel per line
         if (WD == WD_DECOUPLED) p = p * c.wd_term;             // data.mul_(1 - lr * wd)
@@ -172,26 +192,33 @@ __device__ __forceinline__ void adam_element(const StepConsts& c, float g, float
         float gg = g * g;
         v = __builtin_fmaf(c.b2m, gg, v);                      //   .addcmul_(grad, grad, value=1 - beta2)
         float d = __builtin_sqrtf(v);                          // exp_avg_sq.sqrt()
-        d = d * c.bc2inv;                                      //   / math.sqrt(bias_correction2)
+        d = d * bc2inv;                                        //   / math.sqrt(bias_correction2)
         d = d + c.eps;                                         //   .add_(eps)
         float q = m / d;
-        p = __builtin_fmaf(c.step_size, q, p);                 // data.addcdiv_(exp_avg, denom, value=-step_size)
+        p = __builtin_fmaf(step_size, q, p);                   // data.addcdiv_(exp_avg, denom, value=-step_size)
     }
 }
 
 template <int ARITH, int WD, int UNS>
-__device__ __forceinline__ void element_any(const StepConsts& c, float g, float& p, float& m,
-                                            float& v)
+__device__ __forceinline__ void element_any(const StepConsts& c, float step_size, float bc2inv, float g,
+                                            float& p, float& m, float& v)
 {
     if (UNS != UNSCALE_RUNTIME)
-        adam_element<ARITH, WD, UNS>(c, g, p, m, v);
+        adam_element<ARITH, WD, UNS>(c, step_size, bc2inv, g, p, m, v);
     else if (c.unscale == UNSCALE_MUL)
-        adam_element<ARITH, WD, UNSCALE_MUL>(c, g, p, m, v);
+        adam_element<ARITH, WD, UNSCALE_MUL>(c, step_size, bc2inv, g, p, m, v);
     else if (c.unscale == UNSCALE_DIV)
-        adam_element<ARITH, WD, UNSCALE_DIV>(c, g, p, m, v);
+        adam_element<ARITH, WD, UNSCALE_DIV>(c, step_size, bc2inv, g, p, m, v);
     else
-        adam_element<ARITH, WD, UNSCALE_NONE>(c, g, p, m, v);
+        adam_element<ARITH, WD, UNSCALE_NONE>(c, step_size, bc2inv, g, p, m, v);
 }
+
+// Which elements of a launch belong to the step's first operator call: elements [lo, hi) of chunk
+// `chunk` of the launch's batch (-1: none of them).
+struct FirstCall {
+    int chunk;
+    uint64_t lo, hi;
+};
 
 __device__ __forceinline__ float half_bits_to_float(uint32_t h)
 {

@@ -15,21 +15,33 @@ constexpr int kBatch = 64;
 struct ChunkBatch {
     ps_chunk c[kBatch];
 };
-static_assert(sizeof(ps_chunk) == 32 && sizeof(ps_step_state) == 160 && sizeof(ps_scale_record) == 16,
+static_assert(sizeof(ps_chunk) == 32 && sizeof(ps_step_state) == 192 && sizeof(ps_scale_record) == 16 &&
+                  sizeof(ps_call_pattern) == 32,
               "layout of the boundary structs");
 
 // Host-decided step: all scalars arrive as kernel arguments and the
 // arithmetic variant is a compile-time property of the kernel.
+// The span of the step's first operator call, as seen from this workgroup's chunk (empty elsewhere).
+__device__ __forceinline__ void first_call_span(const FirstCall& fc, size_t* lo, size_t* hi)
+{
+    const bool here = fc.chunk == (int)blockIdx.y;
+    *lo = here ? (size_t)fc.lo : 0;
+    *hi = here ? (size_t)fc.hi : 0;
+}
+
 template <int ARITH, int WD, int UNS>
 __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
-    adam_chunks_kernel(ChunkBatch b, size_t chunk_numel, StepConsts c)
+    adam_chunks_kernel(ChunkBatch b, size_t chunk_numel, StepConsts c, FirstCall fc)
 {
-    adam_tile<ARITH, WD, UNS>(c, b.c[blockIdx.y], (size_t)blockIdx.x * kTile, chunk_numel);
+    size_t lo, hi;
+    first_call_span(fc, &lo, &hi);
+    adam_tile<ARITH, WD, UNS>(c, b.c[blockIdx.y], (size_t)blockIdx.x * kTile, chunk_numel, lo, hi);
 }
 
 struct GatedArgs {
     double lr, eps, wd;  // the Python numbers; the operator's arithmetic narrows them to float
     double grad_clamp;
+    int64_t n_calls;  // operator calls the reference makes in this step (its tensors); <= 1: the list is one call
     int adamw;
     int bias_correction;
 };
@@ -46,9 +58,12 @@ __device__ __forceinline__ StepConsts gated_consts(const GatedArgs& ga, const ps
     const float clip = clamp_bound(ga.grad_clamp, st->cur_scale);
     if (ARITH == PS_ARITH_OPERATOR) {
         // The operator takes its scalars and loss_scale as C floats: the Python numbers narrow (RNE).
+        // one operator call in the step: everything is that (first) call
+        const bool one_call = ga.n_calls <= 1;
         finish_consts(c, (float)ga.lr, st->beta1, st->beta2, (float)ga.eps, (float)ga.wd,
-                      ga.adamw != 0, st->beta1_t_next, st->beta2_t_next, ga.bias_correction != 0,
-                      (float)st->cur_scale, clip);
+                      ga.adamw != 0, one_call ? st->beta1_t_next : st->beta1_t_rest,
+                      one_call ? st->beta2_t_next : st->beta2_t_rest, st->beta1_t_next,
+                      st->beta2_t_next, ga.bias_correction != 0, (float)st->cur_scale, clip);
     } else {
         const bool bc = ga.bias_correction != 0;
         torch_consts(c, ga.lr, st->beta1_f64, st->beta2_f64, ga.eps, ga.wd, ga.adamw != 0,
@@ -60,7 +75,7 @@ __device__ __forceinline__ StepConsts gated_consts(const GatedArgs& ga, const ps
 
 template <int ARITH, int WD>
 __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
-    adam_chunks_gated_kernel(ChunkBatch b, size_t chunk_numel, GatedArgs ga,
+    adam_chunks_gated_kernel(ChunkBatch b, size_t chunk_numel, GatedArgs ga, FirstCall fc,
                              const ps_step_state* __restrict__ st)
 {
     const ps_chunk& ch = b.c[blockIdx.y];
@@ -70,7 +85,9 @@ __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
         return;
     }
     const StepConsts c = gated_consts<ARITH>(ga, st);
-    adam_tile<ARITH, WD, UNSCALE_RUNTIME>(c, ch, base, chunk_numel);
+    size_t lo, hi;
+    first_call_span(fc, &lo, &hi);
+    adam_tile<ARITH, WD, UNSCALE_RUNTIME>(c, ch, base, chunk_numel, lo, hi);
 }
 
 // ------------------------------------------------------- tensor-list kernels
@@ -98,7 +115,15 @@ struct TensorBatch {
     ps_chunk t[kTensorBatch];          // fp32 param, exp_avg, exp_avg_sq, fp16 slot of each tensor
     uint64_t numel[kTensorBatch];
     uint32_t first_tile[64];           // of tensor i; 0xFFFFFFFF beyond the last tensor
+    int first_call;                    // which tensor of the batch is the step's first operator call; -1: none
 };
+
+// A tensor is one operator call: its tiles take the first call's scalars as a whole, or none does.
+__device__ __forceinline__ void tensor_call_span(const TensorBatch& b, int k, size_t* lo, size_t* hi)
+{
+    *lo = 0;
+    *hi = k == b.first_call ? (size_t)b.numel[k] : 0;
+}
 
 __device__ __forceinline__ int tensor_of_tile(const TensorBatch& b, uint32_t tile)
 {
@@ -112,7 +137,9 @@ __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
     adam_tensors_kernel(TensorBatch b, StepConsts c)
 {
     const int k = tensor_of_tile(b, blockIdx.x);
-    adam_tile<ARITH, WD, UNS>(c, b.t[k], (size_t)(blockIdx.x - b.first_tile[k]) * kTile, (size_t)b.numel[k]);
+    size_t lo, hi;
+    tensor_call_span(b, k, &lo, &hi);
+    adam_tile<ARITH, WD, UNS>(c, b.t[k], (size_t)(blockIdx.x - b.first_tile[k]) * kTile, (size_t)b.numel[k], lo, hi);
 }
 
 template <int ARITH, int WD>
@@ -126,7 +153,9 @@ __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
         return;
     }
     const StepConsts c = gated_consts<ARITH>(ga, st);
-    adam_tile<ARITH, WD, UNSCALE_RUNTIME>(c, b.t[k], base, (size_t)b.numel[k]);
+    size_t lo, hi;
+    tensor_call_span(b, k, &lo, &hi);
+    adam_tile<ARITH, WD, UNSCALE_RUNTIME>(c, b.t[k], base, (size_t)b.numel[k], lo, hi);
 }
 
 __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
@@ -163,7 +192,7 @@ __global__ void __launch_bounds__(kAuxBlock)
     for (size_t i = (size_t)blockIdx.x * kAuxBlock + threadIdx.x; i < numel; i += stride) {
         float g = GRAD_HALF ? half_bits_to_float(gh[i]) : gf[i];
         float p = p32[i], m = m32[i], v = v32[i];
-        element_any<PS_ARITH_OPERATOR, WD, UNSCALE_RUNTIME>(c, g, p, m, v);
+        element_any<PS_ARITH_OPERATOR, WD, UNSCALE_RUNTIME>(c, c.step_size, c.bc2inv, g, p, m, v);
         p32[i] = p;
         m32[i] = m;
         v32[i] = v;
@@ -183,7 +212,7 @@ __device__ __forceinline__ void flat_tile_math(const StepConsts& c, const float 
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         float pe = p[e], me = m[e], ve = v[e];
-        adam_element<PS_ARITH_OPERATOR, WD, UNS>(c, g[e], pe, me, ve);
+        adam_element<PS_ARITH_OPERATOR, WD, UNS>(c, c.step_size, c.bc2inv, g[e], pe, me, ve);
         p[e] = pe;
         m[e] = me;
         v[e] = ve;
@@ -205,7 +234,7 @@ __global__ void __launch_bounds__(64)
                 float g = GRAD_HALF ? half_bits_to_float(static_cast<const uint16_t*>(grads)[i])
                                     : static_cast<const float*>(grads)[i];
                 float p = p32[i], m = m32[i], v = v32[i];
-                element_any<PS_ARITH_OPERATOR, WD, UNSCALE_RUNTIME>(c, g, p, m, v);
+                element_any<PS_ARITH_OPERATOR, WD, UNSCALE_RUNTIME>(c, c.step_size, c.bc2inv, g, p, m, v);
                 p32[i] = p;
                 m32[i] = m;
                 v32[i] = v;
@@ -438,18 +467,31 @@ __global__ void state_init_kernel(ps_step_state* st, ps_step_state init)
 
 struct SeedArgs {
     int64_t adam_step;
-    float beta1, beta2, b1t_next, b2t_next;
+    float beta1, beta2, b1t_rest, b2t_rest;
     double beta1_f64, beta2_f64, bc1_next, bc2_next;
+    int fresh_operator;
 };
 
 __global__ void state_seed_kernel(ps_step_state* st, SeedArgs a)
 {
     if (threadIdx.x == 0 && blockIdx.x == 0) {
+        // IncrementStep (cpu_adam.h:143-162) for the first call of step adam_step + 1: changed betas restart from
+        // pow; else the running product continues only if the object's own step is adam_step
+        const bool same_betas = st->beta1 == a.beta1 && st->beta2 == a.beta2;
+        if (a.fresh_operator) {
+            // a new native object (cpu_adam.h:68-86): step 0, beta^t = 1
+            st->operator_step = 0;
+            st->beta1_t_cur = 1.0f;
+            st->beta2_t_cur = 1.0f;
+        }
+        const bool follows = (a.fresh_operator || same_betas) && st->operator_step == a.adam_step;
         st->adam_step = a.adam_step;
         st->beta1 = a.beta1;
         st->beta2 = a.beta2;
-        st->beta1_t_next = a.b1t_next;
-        st->beta2_t_next = a.b2t_next;
+        st->beta1_t_next = follows ? st->beta1_t_cur * a.beta1 : a.b1t_rest;
+        st->beta2_t_next = follows ? st->beta2_t_cur * a.beta2 : a.b2t_rest;
+        st->beta1_t_rest = a.b1t_rest;
+        st->beta2_t_rest = a.b2t_rest;
         st->beta1_f64 = a.beta1_f64;
         st->beta2_f64 = a.beta2_f64;
         st->bias_correction1_next = a.bc1_next;
@@ -496,9 +538,12 @@ __global__ void state_set_scaler_kernel(ps_step_state* st, double cur_scale, int
     }
 }
 
-// DynamicLossScaler.update_scale (loss_scaler.py:158-182), one lane.
+// DynamicLossScaler.update_scale (loss_scaler.py:158-182), one lane.  `operator_calls`: how many times the
+// step that was just queued called the native operator in the reference's terms (its tensors; 0 when every
+// chunk took the torch formula): a clean step moves the operator's own step / beta^t state accordingly
+// (Adam_Optimizer::IncrementStep, cpu_adam.h:143-162), a skipped step never reaches the operator.
 __global__ void scaler_update_kernel(ps_step_state* st, int flag_mode, ps_scale_record* log,
-                                     int64_t log_capacity)
+                                     int64_t log_capacity, int64_t operator_calls)
 {
     if (threadIdx.x != 0 || blockIdx.x != 0) return;
     ps_step_state s = *st;
@@ -527,10 +572,23 @@ __global__ void scaler_update_kernel(ps_step_state* st, int flag_mode, ps_scale_
             s.cur_scale = s.cur_scale * s.scale_factor;
             s.scale_is_int = s.scale_is_int && s.factor_is_int;
         }
-        // the step ran: state["step"] += 1 and the float running products advance
-        s.adam_step += 1;
-        s.beta1_t_next = s.beta1_t_next * s.beta1;
-        s.beta2_t_next = s.beta2_t_next * s.beta2;
+        // the step ran: state["step"] += 1
+        const int64_t t = s.adam_step + 1;
+        s.adam_step = t;
+        if (operator_calls >= 1) {
+            // what the operator object holds after its last call of step t: the first call's beta^t if it
+            // was the only one, else pow(beta, t) from the second call on
+            s.beta1_t_cur = operator_calls == 1 ? s.beta1_t_next : s.beta1_t_rest;
+            s.beta2_t_cur = operator_calls == 1 ? s.beta2_t_next : s.beta2_t_rest;
+            s.operator_step = t;
+        }
+        // step t + 1: every call after the first evaluates (float)pow((double)beta, t + 1); the first call
+        // multiplies the held value by beta if the object's step is t, else it evaluates pow as well
+        s.beta1_t_rest = (float)pow_int((double)s.beta1, t + 1);
+        s.beta2_t_rest = (float)pow_int((double)s.beta2, t + 1);
+        const bool follows = s.operator_step == t;
+        s.beta1_t_next = follows ? s.beta1_t_cur * s.beta1 : s.beta1_t_rest;
+        s.beta2_t_next = follows ? s.beta2_t_cur * s.beta2 : s.beta2_t_rest;
         // fp16_cpu_adam.py:412-413 for the next step
         s.bias_correction1_next = 1.0 - pow_int(s.beta1_f64, s.adam_step + 1);
         s.bias_correction2_next = 1.0 - pow_int(s.beta2_f64, s.adam_step + 1);

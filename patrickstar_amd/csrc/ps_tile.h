@@ -118,7 +118,7 @@ struct LaneTile {
 };
 
 template <int ARITH, int WD, int UNS>
-__device__ __forceinline__ void lane_math(const StepConsts& c, LaneTile& r)
+__device__ __forceinline__ void lane_math(const StepConsts& c, float step_size, float bc2inv, LaneTile& r)
 {
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
@@ -132,8 +132,8 @@ __device__ __forceinline__ void lane_math(const StepConsts& c, LaneTile& r)
                   v0 = r.v[u][e0 >> 2][e0 & 3];
             float p1 = r.p[u][e1 >> 2][e1 & 3], m1 = r.m[u][e1 >> 2][e1 & 3],
                   v1 = r.v[u][e1 >> 2][e1 & 3];
-            adam_element<ARITH, WD, UNS>(c, g0, p0, m0, v0);
-            adam_element<ARITH, WD, UNS>(c, g1, p1, m1, v1);
+            adam_element<ARITH, WD, UNS>(c, step_size, bc2inv, g0, p0, m0, v0);
+            adam_element<ARITH, WD, UNS>(c, step_size, bc2inv, g1, p1, m1, v1);
             r.p[u][e0 >> 2][e0 & 3] = p0;
             r.m[u][e0 >> 2][e0 & 3] = m0;
             r.v[u][e0 >> 2][e0 & 3] = v0;
@@ -145,14 +145,16 @@ __device__ __forceinline__ void lane_math(const StepConsts& c, LaneTile& r)
     }
 }
 
-// One tile of one chunk, fast path: the whole tile is in range and all four
-// bases are 16-byte aligned.  All loads of the tile are issued before the
-// first use.  Loads and stores are written once, outside any branch on the
-// arithmetic variant.
+// One tile of one chunk, fast path: the whole tile is in range, all four
+// bases are 16-byte aligned and the whole tile belongs to one operator call
+// (step_size / bc2inv are that call's).  All loads of the tile are issued
+// before the first use.  Loads and stores are written once, outside any
+// branch on the arithmetic variant.
 template <int ARITH, int WD, int UNS>
-__device__ __forceinline__ void adam_tile_vec(const StepConsts& c, float* __restrict__ p32,
-                                              float* __restrict__ m32, float* __restrict__ v32,
-                                              uint16_t* __restrict__ h16, size_t base)
+__device__ __forceinline__ void adam_tile_vec(const StepConsts& c, float step_size, float bc2inv,
+                                              float* __restrict__ p32, float* __restrict__ m32,
+                                              float* __restrict__ v32, uint16_t* __restrict__ h16,
+                                              size_t base)
 {
     LaneTile r;
 #pragma unroll
@@ -167,13 +169,13 @@ __device__ __forceinline__ void adam_tile_vec(const StepConsts& c, float* __rest
         for (int q = 0; q < kQuads; ++q) r.v[u][q] = ld_f4(v32 + i + 4 * q);
     }
     if (UNS != UNSCALE_RUNTIME) {
-        lane_math<ARITH, WD, UNS>(c, r);
+        lane_math<ARITH, WD, UNS>(c, step_size, bc2inv, r);
     } else if (c.unscale == UNSCALE_MUL) {
-        lane_math<ARITH, WD, UNSCALE_MUL>(c, r);
+        lane_math<ARITH, WD, UNSCALE_MUL>(c, step_size, bc2inv, r);
     } else if (ARITH == PS_ARITH_OPERATOR && c.unscale == UNSCALE_DIV) {
-        lane_math<ARITH, WD, UNSCALE_DIV>(c, r);
+        lane_math<ARITH, WD, UNSCALE_DIV>(c, step_size, bc2inv, r);
     } else {
-        lane_math<ARITH, WD, UNSCALE_NONE>(c, r);
+        lane_math<ARITH, WD, UNSCALE_NONE>(c, step_size, bc2inv, r);
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
@@ -188,15 +190,19 @@ __device__ __forceinline__ void adam_tile_vec(const StepConsts& c, float* __rest
     }
 }
 
-// Same elements, one at a time: ragged tile ends and unaligned bases.
+// Same elements, one at a time: ragged tile ends, unaligned bases and tiles that an operator call's
+// boundary runs through (elements [first_lo, first_hi) take the first call's scalars).
 template <int ARITH, int WD, int UNS>
 __device__ __forceinline__ void adam_tile_scalar(const StepConsts& c, float* p32, float* m32,
-                                                 float* v32, uint16_t* h16, size_t base, size_t end)
+                                                 float* v32, uint16_t* h16, size_t base, size_t end,
+                                                 size_t first_lo, size_t first_hi)
 {
     for (size_t i = base + threadIdx.x; i < end; i += kBlock) {
         float g = half_bits_to_float(h16[i]);
         float p = p32[i], m = m32[i], v = v32[i];
-        element_any<ARITH, WD, UNS>(c, g, p, m, v);
+        const bool first = i >= first_lo && i < first_hi;
+        element_any<ARITH, WD, UNS>(c, first ? c.first_step_size : c.step_size,
+                                    first ? c.first_bc2inv : c.bc2inv, g, p, m, v);
         p32[i] = p;
         m32[i] = m;
         v32[i] = v;
@@ -210,18 +216,24 @@ __device__ __forceinline__ bool aligned16(const void* a, const void* b, const vo
     return (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)d) & 15u) == 0;
 }
 
+// first_lo .. first_hi: the elements of THIS chunk that the step's first operator call covers
+// (first_hi <= first_lo: none).  Whole tiles inside or outside that span are uniform and keep the vector
+// path; the at most two tiles that its ends run through go element by element.
 template <int ARITH, int WD, int UNS>
 __device__ __forceinline__ void adam_tile(const StepConsts& c, const ps_chunk& ch, size_t base,
-                                          size_t chunk_numel)
+                                          size_t chunk_numel, size_t first_lo, size_t first_hi)
 {
     size_t end = base + kTile;
-    if (end <= chunk_numel && aligned16(ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16)) {
-        adam_tile_vec<ARITH, WD, UNS>(c, ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16,
-                                      base);
+    const size_t last = end < chunk_numel ? end : chunk_numel;  // one past the tile's last element
+    const bool inside = base >= first_lo && last <= first_hi;
+    const bool cut = !inside && base < first_hi && last > first_lo;
+    if (!cut && end <= chunk_numel && aligned16(ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16)) {
+        adam_tile_vec<ARITH, WD, UNS>(c, inside ? c.first_step_size : c.step_size,
+                                      inside ? c.first_bc2inv : c.bc2inv, ch.param_fp32, ch.exp_avg,
+                                      ch.exp_avg_sq, ch.param_fp16, base);
     } else {
-        if (end > chunk_numel) end = chunk_numel;
         adam_tile_scalar<ARITH, WD, UNS>(c, ch.param_fp32, ch.exp_avg, ch.exp_avg_sq,
-                                         ch.param_fp16, base, end);
+                                         ch.param_fp16, base, last, first_lo, first_hi);
     }
 }
 

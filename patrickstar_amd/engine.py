@@ -134,6 +134,9 @@ class PatrickStarEngine(torch.nn.Module):
         for p in self.client.chunk_based_param_fp16:
             if p in self._copied:
                 continue
+            if not p.requires_grad:
+                # a frozen parameter: the optimizer skips it (fp16_cpu_adam.py:566-569), its slot keeps the parameter
+                continue
             if p.grad is not None:
                 self._gradient_to_chunk(p)
             else:

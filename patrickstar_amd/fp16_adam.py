@@ -25,6 +25,7 @@ to 5e-5 on the second moment (the operator forms ``1 - beta2`` in float).
 kernels, on chunks resident in HBM and keeps the operator's for host-resident
 chunks -- bit for bit what the reference computes under the same placement.
 """
+import ctypes
 import weakref
 from copy import deepcopy
 
@@ -152,6 +153,9 @@ class FP16Adam(torch.optim.Optimizer):
         if arithmetic == "torch":
             _lib.check(self._lib.ps_adam_set_arithmetic(self.opt_id, _lib.PS_ARITH_TORCH), "ps_adam_set_arithmetic")
         self._tables = None
+        self._tensor_table = None  # (ps_chunk rows, numels, count) when the step has to go tensor by tensor
+        self._calls = None  # ps_call_pattern of one step (None: no operator call at all)
+        self._operator_calls = 0
         if self._dynamic and torch.cuda.is_available():
             self.loss_scaler.materialize(self.client.device, betas=betas)
 
@@ -170,16 +174,36 @@ class FP16Adam(torch.optim.Optimizer):
             group.setdefault("amsgrad", False)
 
     # -- chunk descriptor tables -------------------------------------------------
+    def _trainable(self):
+        """The parameters ``step()`` updates, in the order the reference visits them (``fp16_cpu_adam.py:566-605``)."""
+        return [p for group in self.param_groups for p in group["params"] if p.requires_grad and p.ps_attr.is_local()]
+
     def _build_tables(self):
-        """Array of ps_chunk descriptors for HBM-resident positions; list of host-resident ones."""
-        dev_rows, host_positions = [], []
+        """Descriptors of what one step covers, and how the reference would have cut it into operator calls.
+
+        Whole-chunk form (the normal case): an array of ps_chunk descriptors for HBM-resident positions and a list of
+        host-resident ones.  If some tensor of a chunk is NOT updated (``requires_grad=False``, or not handed to the
+        optimizer) the whole-chunk pass does not apply; the step then goes tensor by tensor through
+        ``ps_adam_step_tensors`` over the trainable tensors only, as the reference's loop skips the others.
+        """
         cl = self.client.chunk_list
+        index = self.client.chunk_tensor_index
+        trainable = self._trainable()
+        live_ids = {p.ps_attr.data_id() for p in trainable}
+        chunk_of = {p: index.get_tensor_info(p.ps_attr.data_id()).chunk_id for p in trainable}
+        live_chunks = set(chunk_of.values())
+        partly_frozen = any(
+            info.tensor_id not in live_ids for cid in live_chunks for info in index.generate_tensor_info_in_order(cid)
+        )
+        dev_rows, host_positions, where = [], [], {}
         for pos in self.client.positions():
-            if pos.exp_avg is None or pos.exp_avg_sq is None:
+            if pos.fp16 not in live_chunks or pos.exp_avg is None or pos.exp_avg_sq is None:
                 continue  # a chunk position without trainable parameters
             if pos.on_host:
+                where[pos.fp16] = ("host", len(host_positions))
                 host_positions.append(pos)
             else:
+                where[pos.fp16] = ("hbm", len(dev_rows))
                 dev_rows.append(
                     [
                         cl[pos.fp32].payload.data_ptr(),
@@ -188,6 +212,38 @@ class FP16Adam(torch.optim.Optimizer):
                         cl[pos.fp16].payload.data_ptr(),
                     ]
                 )
+        self._tensor_table = None
+        if partly_frozen:
+            if host_positions:
+                raise NotImplementedError(
+                    "chunks that mix trainable and frozen parameters cannot be combined with host-resident positions"
+                )
+            rows, numels = [], []
+            for p in trainable:
+                st = self.state[p]
+                views = [
+                    self.client.access_data(q)
+                    for q in (self.client.param_fp16_to_param_fp32_map[p], dict.__getitem__(st, "exp_avg"),
+                              dict.__getitem__(st, "exp_avg_sq"), p)
+                ]
+                rows.append([v.data_ptr() for v in views])
+                numels.append(p.ps_attr.numel)
+            self._tensor_table = (_lib.chunk_array(rows), (ctypes.c_size_t * len(numels))(*numels), len(numels))
+        # The operator calls of one step: with the operator's arithmetic every trainable tensor is one, with the torch
+        # arithmetic only those whose optimizer state lives in host memory (fp16_cpu_adam.py:415-443).
+        if self.arithmetic == "torch":
+            called = [p for p in trainable if where[chunk_of[p]][0] == "host"]
+        else:
+            called = trainable
+        self._operator_calls = len(called)
+        self._calls = None
+        if called:
+            first = called[0]
+            info = index.get_tensor_info(first.ps_attr.data_id())
+            kind, k = where[info.chunk_id]
+            self._calls = _lib.call_pattern(
+                len(called), k if kind == "hbm" else len(dev_rows) + k, info.start_offset, info.numel
+            )
         table = _lib.chunk_array(dev_rows) if dev_rows else None
         self._tables = (table, len(dev_rows), host_positions)
         if host_positions:
@@ -285,17 +341,29 @@ class FP16Adam(torch.optim.Optimizer):
                 scaler = self.loss_scaler
                 if self.scan_in_step:
                     self.check_overflow_chunks()
-                if host_positions:
-                    self._streamer.step(self.opt_id, 0, lr, beta1, beta2, eps, weight_decay, -1.0, table, n_dev, scaler)
+                if self._tensor_table is not None:
+                    rows, numels, n_tensors = self._tensor_table
+                    _lib.check(
+                        self._lib.ps_adam_step_tensors(
+                            self.opt_id, 0, lr, beta1, beta2, eps, weight_decay, 1, rows, numels, n_tensors, -1.0,
+                            scaler.state_ptr, stream,
+                        ),
+                        "ps_adam_step_tensors",
+                    )
+                elif host_positions:
+                    self._streamer.step(self.opt_id, 0, lr, beta1, beta2, eps, weight_decay, -1.0, table, n_dev,
+                                        self._calls, scaler)
                 elif n_dev:
                     _lib.check(
                         self._lib.ps_adam_step_chunks_gated(
-                            self.opt_id, lr, eps, weight_decay, 1, table, n_dev, chunk_numel,
+                            self.opt_id, lr, eps, weight_decay, 1, table, n_dev, chunk_numel, self._calls,
                             scaler.state_ptr, stream,
                         ),
                         "ps_adam_step_chunks_gated",
                     )
-                scaler.update_scale(None)  # consume the device flag; advances state["step"] on a clean step
+                # consume the device flag; a clean step advances state["step"] and takes the operator object
+                # through this step's calls
+                scaler.update_scale(None, operator_calls=self._operator_calls)
                 self._steps_dirty = True
                 return loss
 
@@ -308,13 +376,23 @@ class FP16Adam(torch.optim.Optimizer):
             self._steps_dirty = True
             step_no = self._host_step
             loss_scale = self.loss_scaler.loss_scale if self.loss_scaler is not None else -1
-            if host_positions:
-                self._streamer.step(self.opt_id, step_no, lr, beta1, beta2, eps, weight_decay, loss_scale, table, n_dev)
+            if self._tensor_table is not None:
+                rows, numels, n_tensors = self._tensor_table
+                _lib.check(
+                    self._lib.ps_adam_step_tensors(
+                        self.opt_id, step_no, lr, beta1, beta2, eps, weight_decay, 1, rows, numels, n_tensors,
+                        float(loss_scale), None, stream,
+                    ),
+                    "ps_adam_step_tensors",
+                )
+            elif host_positions:
+                self._streamer.step(self.opt_id, step_no, lr, beta1, beta2, eps, weight_decay, loss_scale, table, n_dev,
+                                    self._calls)
             elif n_dev:
                 _lib.check(
                     self._lib.ps_adam_step_chunks(
                         self.opt_id, step_no, lr, beta1, beta2, eps, weight_decay, 1, table, n_dev,
-                        chunk_numel, float(loss_scale), stream,
+                        chunk_numel, self._calls, float(loss_scale), stream,
                     ),
                     "ps_adam_step_chunks",
                 )
@@ -366,6 +444,8 @@ class FP16Adam(torch.optim.Optimizer):
         if self._dynamic:
             self.loss_scaler.materialize(self.client.device)
             if step_seen is not None:
-                self.loss_scaler._seed_step(step_seen)
+                # the operator object behind this optimizer stays the one it was (fp16_cpu_adam.py:660-694 does not
+                # touch it); a new optimizer got a new one when it was constructed
+                self.loss_scaler._seed_step(step_seen, fresh_operator=False)
             if "loss_scaler" in state_dict:
                 self.loss_scaler.load_state_dict(state_dict["loss_scaler"])

@@ -54,13 +54,15 @@ class HostChunkStreamer:
         )
         self._lib = _lib.load()
 
-    def step(self, opt_id, step_no, lr, beta1, beta2, eps, weight_decay, loss_scale, resident, n_resident, scaler=None):
+    def step(self, opt_id, step_no, lr, beta1, beta2, eps, weight_decay, loss_scale, resident, n_resident, calls=None,
+             scaler=None):
         """One optimizer step over the resident chunk array AND the host-resident chunks.
+        ``calls``: the step's ps_call_pattern over both lists (resident positions counted first).
         ``scaler`` (a device-resident DynamicLossScaler) selects the device-gated form."""
         _lib.check(
             self._lib.ps_adam_step_hybrid(
                 opt_id, step_no, lr, beta1, beta2, eps, weight_decay, 1, resident, n_resident, self.host_table,
-                self.n_host, self.chunk_numel, self.staging, self.n_slots, float(loss_scale),
+                self.n_host, self.chunk_numel, self.staging, self.n_slots, calls, float(loss_scale),
                 scaler.state_ptr if scaler is not None else None, _lib.current_stream_handle(),
             ),
             "ps_adam_step_hybrid",

@@ -3,7 +3,7 @@
 ``LossScaler`` (static) and ``DynamicLossScaler`` keep the constructor
 arguments, methods and semantics of ``patrickstar/fp16/loss_scaler.py:46-190``.
 The dynamic scaler's state (current scale, iteration, last overflow iteration,
-hysteresis credit) lives in a 160-byte device struct (``ps_step_state``) that the
+hysteresis credit) lives in a 192-byte device struct (``ps_step_state``) that the
 HIP kernels read and update, so the optimizer step never has to ask the host
 whether gradients overflowed.  Reading a field from Python
 (``loss_scale``, ``cur_iter``, ...) copies the struct back, which is the only
@@ -119,10 +119,13 @@ class DynamicLossScaler:
             )
         return self
 
-    def _seed_step(self, adam_step):
+    def _seed_step(self, adam_step, fresh_operator=True):
+        """Set the Adam step counter.  ``fresh_operator``: a newly created operator object stands behind it (a new
+        optimizer); False keeps the running one, as the reference's ``load_state_dict`` does."""
         _lib.check(
             _lib.load().ps_state_seed_step(
-                self._state.data_ptr(), int(adam_step), self._betas[0], self._betas[1], _lib.current_stream_handle()
+                self._state.data_ptr(), int(adam_step), self._betas[0], self._betas[1], int(bool(fresh_operator)),
+                _lib.current_stream_handle(),
             ),
             "ps_state_seed_step",
         )
@@ -232,15 +235,18 @@ class DynamicLossScaler:
         return probe.overflow_flag
 
     # -- state machine ----------------------------------------------------------------
-    def update_scale(self, overflow):
-        """``overflow`` is a bool, or None to consume the sticky device flag; asynchronous."""
+    def update_scale(self, overflow, operator_calls=1):
+        """``overflow`` is a bool, or None to consume the sticky device flag; asynchronous.
+        ``operator_calls``: how many tensors the optimizer step behind this call handed to the native operator in the
+        reference's terms; a clean step takes the operator's step / beta^t state through that many calls."""
         self.materialize()
         mode = _lib.PS_FLAG_FROM_DEVICE if overflow is None else (_lib.PS_FLAG_TRUE if overflow else _lib.PS_FLAG_FALSE)
         log_ptr = self._log.data_ptr() if self._log is not None else None
         with torch.cuda.device(self._state.device):
             _lib.check(
                 _lib.load().ps_scaler_update(
-                    self._state.data_ptr(), mode, log_ptr, self._log_capacity, _lib.current_stream_handle()
+                    self._state.data_ptr(), mode, log_ptr, self._log_capacity, int(operator_calls),
+                    _lib.current_stream_handle()
                 ),
                 "ps_scaler_update",
             )

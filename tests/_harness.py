@@ -21,6 +21,20 @@ def assert_bits_equal(got, want, what):
         )
 
 
+def tensor_spans(client, optimizer):
+    """(chunk position, element offset, numel) of every trainable parameter, in the optimizer's own order: the
+    operator calls the reference makes in one step, as the oracle wants them."""
+    index = client.chunk_tensor_index
+    position_of = {q.fp16: i for i, q in enumerate(client.positions())}
+    out = []
+    for group in optimizer.param_groups:
+        for p in group["params"]:
+            if p.requires_grad:
+                info = index.get_tensor_info(p.ps_attr.data_id())
+                out.append((position_of[info.chunk_id], info.start_offset, info.numel))
+    return out
+
+
 class ChunkHarness:
     """n_chunks x chunk_size synthetic chunk list on cuda:0 with an FP16Adam on top."""
 

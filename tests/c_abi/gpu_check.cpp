@@ -145,18 +145,23 @@ int main()
     oracle_adam_init(&native, lr, b1, b2, eps, wd, 1);
     PS_OK(ps_adam_create(31, lr, b1, b2, eps, wd, 1, 0));
 
-    // ---- host-decided steps with a static scale: t = 100 (cold), then 101 and 102 (running products)
+    // Every chunk holds one tensor: the reference makes one operator call per chunk and step, the first of them
+    // for the whole of chunk 0.
+    const ps_call_pattern calls = {C, 0, 0, n};
+
+    // ---- host-decided steps with a static scale: t = 100 (cold), then 101 and 102 (the first call of each
+    //      multiplies the running product, the later calls evaluate pow)
     const double scale = 4096.0;
     for (uint64_t step = 100; step < 103; ++step) {
         for (int c = 0; c < C; ++c) {
             new_gradients(rng, host[c], scale);
             if (upload(host[c], dev[c], n)) return 2;
         }
-        PS_OK(ps_adam_step_chunks(31, step, lr, b1, b2, eps, wd, 1, table, C, n, scale, stream));
+        PS_OK(ps_adam_step_chunks(31, step, lr, b1, b2, eps, wd, 1, table, C, n, &calls, scale, stream));
         HIP_OK(hipStreamSynchronize(stream));
-        oracle_adam_advance(&native, step, b1, b2);
-        oracle_adam_set(&native, lr, eps, wd, 1);
         for (int c = 0; c < C; ++c) {
+            oracle_adam_advance(&native, step, b1, b2);  // one adam_update per tensor, same step number
+            oracle_adam_set(&native, lr, eps, wd, 1);
             if (oracle_adam_span(&native, host[c].p.data(), host[c].h.data(), 1, host[c].m.data(), host[c].v.data(),
                                  n, (float)scale, 0) <= 0)
                 return 5;
@@ -181,8 +186,8 @@ int main()
             if (upload(host[c], dev[c], n)) return 2;
         }
         PS_OK(ps_overflow_scan_chunks(table, C, n, d_state, stream));
-        PS_OK(ps_adam_step_chunks_gated(32, lr, eps, wd, 1, table, C, n, d_state, stream));
-        PS_OK(ps_scaler_update(d_state, PS_FLAG_FROM_DEVICE, NULL, 0, stream));
+        PS_OK(ps_adam_step_chunks_gated(32, lr, eps, wd, 1, table, C, n, &calls, d_state, stream));
+        PS_OK(ps_scaler_update(d_state, PS_FLAG_FROM_DEVICE, NULL, 0, calls.n_calls, stream));
         HIP_OK(hipStreamSynchronize(stream));
         if (poison) {
             for (int c = 0; c < C; ++c) oracle_cast_f32_to_f16(host[c].p.data(), host[c].h.data(), n);
@@ -190,9 +195,9 @@ int main()
             last_overflow = cur_iter;
         } else {
             adam_step += 1;
-            oracle_adam_advance(&native, (uint64_t)adam_step, b1, b2);
-            oracle_adam_set(&native, lr, eps, wd, 1);
             for (int c = 0; c < C; ++c) {
+                oracle_adam_advance(&native, (uint64_t)adam_step, b1, b2);
+                oracle_adam_set(&native, lr, eps, wd, 1);
                 if (oracle_adam_span(&native, host[c].p.data(), host[c].h.data(), 1, host[c].m.data(),
                                      host[c].v.data(), n, (float)cur_scale, 0) <= 0)
                     return 5;
@@ -257,12 +262,12 @@ int main()
                     HIP_OK(hipMemcpy(dev[c].h, host[c].h.data(), n * 2, hipMemcpyHostToDevice));
             }
         }
-        PS_OK(ps_adam_step_hybrid(33, step, lr, b1, b2, eps, wd, 1, table, 1, host_table, 2, n, staging, 2, scale, NULL,
-                                  stream));
+        PS_OK(ps_adam_step_hybrid(33, step, lr, b1, b2, eps, wd, 1, table, 1, host_table, 2, n, staging, 2, &calls, scale,
+                                  NULL, stream));
         HIP_OK(hipStreamSynchronize(stream));
-        oracle_adam_advance(&native, step, b1, b2);
-        oracle_adam_set(&native, lr, eps, wd, 1);
         for (int c = 0; c < C; ++c) {
+            oracle_adam_advance(&native, step, b1, b2);
+            oracle_adam_set(&native, lr, eps, wd, 1);
             if (oracle_adam_span(&native, host[c].p.data(), host[c].h.data(), 1, host[c].m.data(), host[c].v.data(),
                                  n, (float)scale, 0) <= 0)
                 return 5;

@@ -65,7 +65,7 @@ def test_bert_base_at_the_reference_chunk_size_matches_the_oracle():
     import numpy as np
 
     import oracle
-    from _harness import assert_bits_equal
+    from _harness import assert_bits_equal, tensor_spans
 
     cfg = transformers.BertConfig(vocab_size=10, hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0, num_labels=2)
     torch.manual_seed(0)
@@ -89,7 +89,11 @@ def test_bert_base_at_the_reference_chunk_size_matches_the_oracle():
     mirror = [{"p32": snap(cl[q.fp32].payload), "m": snap(cl[q.exp_avg].payload), "v": snap(cl[q.exp_avg_sq].payload),
                "p16": snap(cl[q.fp16].payload)} for q in pos]
     oscaler = oracle.scaler_from_config(config["fp16"])
-    oopt = oracle.OptimizerStepOracle(mirror, oscaler, lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
+    # one operator call per parameter tensor, in parameters() order, as the reference's loop makes them
+    spans = tensor_spans(client, optimizer)
+    assert len(spans) == len(list(engine.module.parameters())) > 190
+    oopt = oracle.OptimizerStepOracle(mirror, oscaler, lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True,
+                                      tensors=spans)
     ids = torch.randint(0, 10, (4, 64), device="cuda")
     labels = torch.randint(0, 2, (4,), device="cuda")
     for it in range(3):

@@ -7,7 +7,7 @@ import torch
 
 import oracle
 import patrickstar_amd as ps
-from _harness import HybridHarness, assert_bits_equal
+from _harness import HybridHarness, assert_bits_equal, tensor_spans
 
 pytestmark = pytest.mark.gpu
 
@@ -112,7 +112,12 @@ def test_engine_end_to_end_against_oracle(loss_scale, host_positions):
     mirror = [{"p32": _snap(cl[q.fp32].payload), "m": _snap(cl[q.exp_avg].payload),
                "v": _snap(cl[q.exp_avg_sq].payload), "p16": _snap(cl[q.fp16].payload)} for q in pos]
     oscaler = oracle.scaler_from_config(config["fp16"])
-    oopt = oracle.OptimizerStepOracle(mirror, oscaler, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
+    # The reference calls the operator once per parameter in parameters() order: `gain` (the module's own parameter,
+    # which sits in the SECOND chunk) comes first and is the one call of a step that may continue the running beta^t.
+    spans = tensor_spans(client, optimizer)
+    assert spans[0] == (1, 328, 8) and len(spans) == 5
+    oopt = oracle.OptimizerStepOracle(mirror, oscaler, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True,
+                                      tensors=spans)
     x = torch.randn(16, 24, device="cuda").half()
     losses = []
     for it in range(6):
@@ -313,3 +318,71 @@ def test_config5_full_shape_180_chunks_60_on_the_host():
         s = pd.view(torch.int32).sum(dtype=torch.int64).item()
         assert s != before[i % 3], f"chunk {i} was not updated"
         assert ref.setdefault(i % 3, s) == s, f"chunk {i} differs from its twins"
+
+
+class _PartlyFrozen(torch.nn.Module):
+    """fc1 is frozen before the engine sees the model; fc2 and `gain` train.  With 1100-element chunks fc1 has the
+    first chunk to itself (a position that drops out of the step) and the trainable tensors share the second; with
+    2000-element chunks all five tensors share ONE chunk, frozen and trainable side by side."""
+
+    def __init__(self):
+        super().__init__()
+        self.fc1 = torch.nn.Linear(24, 40)
+        self.fc2 = torch.nn.Linear(40, 8)
+        self.gain = torch.nn.Parameter(torch.ones(8))
+        for p in self.fc1.parameters():
+            p.requires_grad_(False)
+
+    def forward(self, x):
+        return (self.fc2(torch.tanh(self.fc1(x))) * self.gain).float().pow(2).mean()
+
+
+@pytest.mark.parametrize("chunk_size", [1100, 2000])
+@pytest.mark.parametrize("optim_type,loss_scale", [("AdamW", 0), ("Adam", 128)])
+def test_frozen_parameters_are_skipped_like_the_reference_skips_them(optim_type, loss_scale, chunk_size):
+    """requires_grad=False parameters are not updated, not decayed and not counted (fp16_cpu_adam.py:566-569), even with
+    weight decay and when they share a chunk with trainable ones; the trainable ones match the oracle bit for bit."""
+    torch.manual_seed(0)
+    config = {
+        "optimizer": {"type": optim_type, "params": {"lr": 1e-2, "betas": (0.9, 0.999), "eps": 1e-8, "weight_decay": 0.1}},
+        "fp16": {"enabled": True, "loss_scale": loss_scale, "initial_scale_power": 7, "loss_scale_window": 3, "hysteresis": 2, "min_loss_scale": 1},
+        "default_chunk_size": chunk_size,
+    }
+    engine, optimizer = ps.initialize_engine(model_func=_PartlyFrozen, local_rank=0, config=config)
+    client = engine.client
+    cl = client.chunk_list
+    pos = client.positions()
+    assert len(pos) == (2 if chunk_size == 1100 else 1)
+    frozen = list(engine.module.fc1.parameters())
+    masters = [client.access_data(client.param_fp16_to_param_fp32_map[p]) for p in frozen]
+    frozen_before = [(p.detach().clone(), m.clone()) for p, m in zip(frozen, masters)]
+    spans = tensor_spans(client, optimizer)
+    assert len(spans) == 3  # gain, fc2.weight, fc2.bias
+    mirror = [{"p32": _snap(cl[q.fp32].payload), "m": _snap(cl[q.exp_avg].payload),
+               "v": _snap(cl[q.exp_avg_sq].payload), "p16": _snap(cl[q.fp16].payload)} for q in pos]
+    oscaler = oracle.scaler_from_config(config["fp16"])
+    oopt = oracle.OptimizerStepOracle(mirror, oscaler, lr=1e-2, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.1,
+                                      use_adamw=(optim_type == "AdamW"), tensors=spans)
+    x = torch.randn(16, 24, device="cuda").half()
+    for it in range(6):
+        loss = engine(x * (1.0 if it != 2 or loss_scale else 3e4))  # dynamic scaler: iteration 2 overflows
+        engine.backward(loss)
+        for q, c in zip(pos, mirror):
+            c["p16"][...] = _snap(cl[q.fp16].payload)
+        # the slots of frozen parameters still hold the parameters, not zeros
+        for p, (p0, _) in zip(frozen, frozen_before):
+            assert torch.equal(client.access_data(p), p0)
+        optimizer.step()
+        torch.cuda.synchronize()
+        oopt.check_overflow()
+        skipped = oopt.step()
+        if loss_scale == 0:
+            assert skipped == (it == 2)
+        for p, m, (p0, m0) in zip(frozen, masters, frozen_before):
+            assert torch.equal(p.detach(), p0) and torch.equal(m, m0), "a frozen parameter moved"
+        for q, c in zip(pos, mirror):
+            for key, cid in (("p32", q.fp32), ("m", q.exp_avg), ("v", q.exp_avg_sq), ("p16", q.fp16)):
+                assert_bits_equal(_snap(cl[cid].payload), c[key], f"iteration {it} {key}")
+    live = [p for p in engine.module.parameters() if p.requires_grad]
+    assert optimizer.state[live[0]]["step"] == (5 if loss_scale == 0 else 6)
+    assert optimizer.state[frozen[0]]["step"] == 0

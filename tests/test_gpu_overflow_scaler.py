@@ -237,38 +237,76 @@ def test_config3_full_size_flags_and_scale_trajectory():
 
 def test_state_dict_round_trip_continues_bit_exact():
     """Semantics of the reference's checkpoint test (unitest/test_checkpoint.py:44-180): save, keep training,
-    reload, replay the same gradients -> identical results, incl. step and (an addition) the scaler state."""
+    reload, replay the same gradients, incl. step and (an addition) the scaler state.
+
+    What "identical" can mean is set by the operator object (cpu_adam.h:143-162), which a checkpoint does not carry:
+    reloading into the SAME optimizer right at the saved step leaves it in step with the counter, and training
+    continues exactly as if nothing had happened; a NEW optimizer starts with a new operator object, whose first call
+    (the first tensor of the first step after the reload) evaluates pow(beta, t) where the uninterrupted run
+    multiplied pow(beta, t-1) by beta.  Every other tensor is the same bit for bit in all three runs."""
     kw = dict(init_scale=2**10, scale_factor=2, scale_window=4, min_scale=1)
-    h = ChunkHarness(2, 2048 + 99, ps.DynamicLossScaler(**kw), seed=21, lr=1e-3, weight_decay=0.01, use_adamw=True)
-    h.fill_state()
-    grads = [[(torch.randn(h.chunk_size, device="cuda") * 1e-3 * 512).half() for _ in range(2)] for _ in range(8)]
+    akw = dict(lr=1e-3, weight_decay=0.01, use_adamw=True)
+    n = 2048 + 99
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(5)
+    grads = [[(torch.randn(n, device="cuda", generator=gen) * 1e-3 * 512).half() for _ in range(2)] for _ in range(8)]
     grads[5][1][7] = float("inf")
 
-    def run(lo, hi):
+    def run(h, lo, hi, oopt=None):
         for s in range(lo, hi):
             for i in range(2):
                 h.payloads(i)[3].copy_(grads[s][i])
+                if oopt is not None:
+                    oopt.chunks[i]["p16"][...] = grads[s][i].cpu().numpy()
             h.opt.step()
+            if oopt is not None:
+                oopt.check_overflow()
+                oopt.step()
 
-    run(0, 3)
-    sd = h.opt.state_dict()
-    master = [h.payloads(i)[0].clone() for i in range(2)]
+    def bits(t):
+        return t.view(torch.int16 if t.dtype == torch.half else torch.int32)
+
+    # run A: uninterrupted
+    a = ChunkHarness(2, n, ps.DynamicLossScaler(**kw), seed=21, **akw)
+    a.fill_state()
+    run(a, 0, 3)
+    sd = a.opt.state_dict()
+    master = [a.payloads(i)[0].clone() for i in range(2)]
     assert sd["state"][0]["step"] == 3 and sd["state"][0]["exp_avg"].device.type == "cpu"
-    run(3, 8)
-    final = [tuple(t.clone() for t in h.payloads(i)) for i in range(2)]
-    final_scale, final_step = h.opt.loss_scaler.loss_scale, h.opt.state[h.params[0]]["step"]
+    # run B: the same optimizer reloads its own checkpoint at once, then continues
+    b = ChunkHarness(2, n, ps.DynamicLossScaler(**kw), seed=21, **akw)
+    b.fill_state()
+    run(b, 0, 3)
+    b.opt.load_state_dict(b.opt.state_dict())
+    run(a, 3, 8)
+    run(b, 3, 8)
+    final = [tuple(t.clone() for t in a.payloads(i)) for i in range(2)]
+    final_scale, final_step = a.opt.loss_scaler.loss_scale, a.opt.state[a.params[0]]["step"]
+    for i in range(2):
+        for x, y in zip(b.payloads(i), final[i]):
+            assert torch.equal(bits(x), bits(y)), "an immediate reload into the same optimizer changed the run"
 
-    h2 = ChunkHarness(2, 2048 + 99, ps.DynamicLossScaler(**kw), seed=99, lr=1e-3, weight_decay=0.01, use_adamw=True)
+    # run C: a new optimizer (new operator object) loads the checkpoint and replays steps 3..7
+    c = ChunkHarness(2, n, ps.DynamicLossScaler(**kw), seed=99, **akw)
     for i in range(2):
-        h2.payloads(i)[0].copy_(master[i])  # the model checkpoint restores the fp32 master params
-    h2.opt.load_state_dict(sd)
-    assert h2.opt.state[h2.params[0]]["step"] == 3
-    h, h_old = h2, h
-    run(3, 8)
-    for i in range(2):
-        for a, b in zip(h.payloads(i), final[i]):
-            assert torch.equal(a.view(torch.int16 if a.dtype == torch.half else torch.int32), b.view(torch.int16 if b.dtype == torch.half else torch.int32))
-    assert h.opt.loss_scaler.loss_scale == final_scale and h.opt.state[h.params[0]]["step"] == final_step == 7
+        c.payloads(i)[0].copy_(master[i])  # the model checkpoint restores the fp32 master params
+    c.opt.load_state_dict(sd)
+    assert c.opt.state[c.params[0]]["step"] == 3
+    oc = c.oracle_chunks()
+    oscaler = oracle.ScalerOracle(**kw)
+    for f in (False, False, False):
+        oscaler.update_scale(f)
+    oopt = oracle.OptimizerStepOracle(oc, oscaler, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
+    oopt.step_count = 3  # with a fresh native object behind it, like the new optimizer
+    run(c, 3, 8, oopt)
+    c.compare(oc, what="reloaded into a new optimizer")
+    for x, y in zip(c.payloads(1), final[1]):
+        assert torch.equal(bits(x), bits(y)), "chunk 1 is never the first operator call: must not notice the reload"
+    p_c, p_a = c.payloads(0)[0], final[0][0]
+    # chunk 0 took one step with pow(beta, 4) in place of pow(beta, 3) * beta: 1 / sqrt(1 - beta2^t) moves by up to 1e-5
+    # relative at such small t, i.e. the parameter by about lr * 1e-5
+    assert not torch.equal(bits(p_c), bits(p_a)) and torch.allclose(p_c, p_a, rtol=0, atol=1e-3 * 5e-5)
+    assert c.opt.loss_scaler.loss_scale == final_scale and c.opt.state[c.params[0]]["step"] == final_step == 7
 
 
 def test_fused_gradient_clamp_follows_the_device_resident_scale():

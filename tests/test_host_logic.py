@@ -185,14 +185,14 @@ def test_library_loads_and_exports_every_declared_symbol():
     lib = _lib.load()
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.ps_abi_version() == 2
+    assert lib.ps_abi_version() == 3
     # host-only entry points: registry and argument checks work without a GPU
     assert lib.ps_adam_create(77, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, 0) == 0
     assert lib.ps_adam_destroy(77) == 0
-    assert lib.ps_scaler_update(None, 0, None, 0, None) == _lib.PS_ERR_BAD_ARG
+    assert lib.ps_scaler_update(None, 0, None, 0, 1, None) == _lib.PS_ERR_BAD_ARG
     assert b"d_state" in lib.ps_last_error()
     assert lib.ps_state_init(None, 1.0, 1, 2.0, 1, 10, 1.0, 1, 1, 0, 0.9, 0.999, None) == _lib.PS_ERR_BAD_ARG
-    assert ctypes.sizeof(_lib.ps_step_state) == 160 and ctypes.sizeof(_lib.ps_chunk) == 32
+    assert ctypes.sizeof(_lib.ps_step_state) == 192 and ctypes.sizeof(_lib.ps_chunk) == 32
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
@@ -268,15 +268,15 @@ def test_argument_checks_happen_before_any_gpu_work():
     fake = _lib.chunk_array([[16, 32, 48, 64]])  # never dereferenced: every call below fails validation first
     bad_slot = _lib.chunk_array([[16, 0, 48, 64]])
     E = _lib.PS_ERR_BAD_ARG
-    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, None, 2, 1.0, None, None) == E
+    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, None, 2, None, 1.0, None, None) == E
     assert b"staging" in lib.ps_last_error()
-    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, fake, 0, 1.0, None, None) == E
-    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, fake, 9, 1.0, None, None) == E
-    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, bad_slot, 1, 1.0, None, None) == E
-    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, bad_slot, 1, 1024, fake, 1, 1.0, None, None) == E
+    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, fake, 0, None, 1.0, None, None) == E
+    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, fake, 9, None, 1.0, None, None) == E
+    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, bad_slot, 1, None, 1.0, None, None) == E
+    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, bad_slot, 1, 1024, fake, 1, None, 1.0, None, None) == E
     assert b"host chunk 0" in lib.ps_last_error()
-    assert lib.ps_adam_step_hybrid(4711, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, fake, 1, 1.0, None, None) == _lib.PS_ERR_UNKNOWN_ID
-    assert lib.ps_adam_step_chunks_gated(88, 1e-3, 1e-8, 0.0, 1, fake, 1, 1024, None, None) == E
+    assert lib.ps_adam_step_hybrid(4711, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, fake, 1, None, 1.0, None, None) == _lib.PS_ERR_UNKNOWN_ID
+    assert lib.ps_adam_step_chunks_gated(88, 1e-3, 1e-8, 0.0, 1, fake, 1, 1024, None, None, None) == E
     assert lib.ps_overflow_scan_host_chunks(fake, 1, 1024, fake, 1, None, None) == E
     assert lib.ps_overflow_scan(None, 10, None, None) == E
     assert lib.ps_adam_set_grad_clamp(4711, 1.0) == _lib.PS_ERR_UNKNOWN_ID
@@ -286,12 +286,13 @@ def test_argument_checks_happen_before_any_gpu_work():
     assert lib.ps_adam_set_arithmetic(88, _lib.PS_ARITH_OPERATOR) == 0
     assert lib.ps_adam_set_arithmetic(4711, _lib.PS_ARITH_TORCH) == _lib.PS_ERR_UNKNOWN_ID
     # descriptors are validated before the operator's step scalars advance or anything is enqueued
-    assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, bad_slot, 1, 1024, 1.0, None) == E
+    assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, bad_slot, 1, 1024, None, 1.0, None) == E
     assert b"chunk 0 has a NULL payload" in lib.ps_last_error()
     assert lib.ps_state_init(ctypes.c_void_p(16), 1.0, 1, 2.0, 1, 0, 1.0, 1, 1, 0, 0.9, 0.999, None) == E  # window 0
     assert b"scale_window" in lib.ps_last_error()
-    assert lib.ps_scaler_update(ctypes.c_void_p(16), 3, None, 0, None) == E
-    assert lib.ps_state_seed_step(ctypes.c_void_p(16), -1, 0.9, 0.999, None) == E
+    assert lib.ps_scaler_update(ctypes.c_void_p(16), 3, None, 0, 1, None) == E
+    assert lib.ps_scaler_update(ctypes.c_void_p(16), 0, None, 0, -1, None) == E
+    assert lib.ps_state_seed_step(ctypes.c_void_p(16), -1, 0.9, 0.999, 1, None) == E
     lib.ps_adam_destroy(88)
 
 
@@ -365,3 +366,46 @@ def test_client_append_and_access_known_answer():
     for param, ref in zip(params, refs):
         assert torch.max(client.access_data(param, torch.device("cpu:0")) - ref) == 0
         client.release_data(param)
+
+
+@pytest.mark.skipif(not os.path.exists(_lib.LIB_PATH), reason="HIP library not built")
+def test_step_tables_follow_the_reference_call_order_and_skip_frozen_parameters():
+    """What FP16Adam hands to the library for one step (no GPU needed to build it).  The reference visits
+    parameters in param_groups order and skips those with requires_grad=False (fp16_cpu_adam.py:566-605): the first
+    operator call of a step is the first TRAINABLE parameter, wherever its chunk is; a chunk that also holds a frozen
+    parameter cannot be updated as a whole."""
+    def build(freeze=(), arithmetic="operator"):
+        client = ps.PatrickStarClient(0, 32, device="cpu")
+        model = _Tiny()
+        for name in freeze:
+            dict(model.named_parameters())[name].requires_grad_(False)
+        client.register_model(model)
+        opt = ps.FP16Adam(client, model.parameters(), lr=1e-3, weight_decay=0.1, arithmetic=arithmetic)
+        opt._build_tables()
+        return client, model, opt
+
+    # parameters() order: scale (the parent's own, chunk 1 offset 14), a.weight, a.bias, b.weight, b.bias
+    client, model, opt = build()
+    assert opt._tensor_table is None and opt._tables[1] == 2 and opt._operator_calls == 5
+    pat = opt._calls._obj
+    assert (pat.n_calls, pat.first_chunk, pat.first_offset, pat.first_numel) == (5, 1, 14, 3)
+
+    # the torch formula never calls the operator for HBM-resident state
+    _, _, opt = build(arithmetic="torch")
+    assert opt._calls is None and opt._operator_calls == 0
+
+    # scale frozen: the first call moves to a.weight; chunk 1 now mixes frozen and trainable -> tensor by tensor
+    client, model, opt = build(freeze=("scale",))
+    rows, numels, n = opt._tensor_table
+    assert n == 4 and list(numels) == [24, 6, 12, 2] and opt._operator_calls == 4
+    want = [client.access_data(p).data_ptr() for p in (model.a.weight, model.a.bias, model.b.weight, model.b.bias)]
+    assert [rows[i].param_fp16 for i in range(4)] == want
+    for i, p in enumerate((model.a.weight, model.a.bias, model.b.weight, model.b.bias)):
+        assert rows[i].param_fp32 == client.access_data(client.param_fp16_to_param_fp32_map[p]).data_ptr()
+        assert rows[i].exp_avg == client.access_data(dict.__getitem__(opt.state[p], "exp_avg")).data_ptr()
+
+    # a whole chunk frozen (a.weight and a.bias are all of chunk 0): that position simply drops out
+    client, model, opt = build(freeze=("a.weight", "a.bias"))
+    assert opt._tensor_table is None and opt._tables[1] == 1 and opt._operator_calls == 3
+    pat = opt._calls._obj
+    assert (pat.n_calls, pat.first_chunk, pat.first_offset, pat.first_numel) == (3, 0, 14, 3)
