@@ -323,6 +323,22 @@ int ps_overflow_scan_f32(const float* d_grads_fp32, size_t numel, ps_step_state*
 int ps_overflow_scan_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_numel,
                             ps_step_state* d_state, ps_stream_t stream);
 
+/* ps_overflow_scan_chunks for callers that cannot allocate device memory.  It has no counterpart in the
+ * reference: it exists for code running under HIP graph capture, tight serving loops and harnesses that
+ * forbid hipMalloc, which have no ps_step_state to hand over.  The flag is an ordinary word of the
+ * caller's (device-accessible, 4-byte aligned), set to 1 if any fp16 payload holds an inf / nan and
+ * left alone otherwise (sticky, like ps_step_state::overflow).  The probe runs without atomics: every
+ * workgroup leaves its partial result in a word of a file-scope device array inside the library
+ * (4 MiB per GPU, resolved with hipGetSymbolAddress at the first call on a device), and a second kernel
+ * reduces those words.  The call allocates and frees nothing.
+ *   limit   n_chunks * ceil(chunk_numel / 8192) <= 1,048,576 scratch words, i.e. at most 8 Gi elements
+ *           per call; more is rejected with PS_ERR_BAD_ARG before anything is queued
+ *   sharing every call on one GPU uses that GPU's one scratch array: calls that overlap in time on
+ *           one GPU (different streams or host threads) race.  Nothing in it needs clearing: each call
+ *           overwrites every word it later reads. */
+int ps_overflow_scan_chunks_noalloc(const ps_chunk* chunks, int n_chunks, size_t chunk_numel,
+                                    uint32_t* d_flag, ps_stream_t stream);
+
 /* Backward-side producer (patrickstar/core/hook.py:200-230): copy one parameter's
  * gradient (fp16, or fp32 rounded RNE) into its slot of the fp16 chunk and, in
  * the same pass, OR "holds inf/nan" into d_state->overflow (skipped when

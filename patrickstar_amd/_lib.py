@@ -112,6 +112,7 @@ SIGNATURES = {
     "ps_overflow_scan": (_i, [_vp, _sz, _vp, _vp]),
     "ps_overflow_scan_f32": (_i, [_vp, _sz, _vp, _vp]),
     "ps_overflow_scan_chunks": (_i, [_vp, _i, _sz, _vp, _vp]),
+    "ps_overflow_scan_chunks_noalloc": (_i, [_vp, _i, _sz, _vp, _vp]),
     "ps_grad_to_chunk": (_i, [_vp, _i, _vp, _sz, _vp, _vp]),
     "ps_scaler_update": (_i, [_vp, _i, _vp, _i64, _i64, _vp]),
     "ps_state_read": (_i, [_vp, ctypes.POINTER(ps_step_state), _vp]),

@@ -491,6 +491,40 @@ int fp16_payloads_in_hbm(const ps_chunk* host_chunks, int n, bool* in_hbm, bool*
 
 }  // namespace
 
+// ------------------------------------------- library-owned device scratch
+//
+// Partial results of ps_overflow_scan_chunks_noalloc: one word per workgroup of its first kernel.  A
+// file-scope device array, so the entry point needs no allocation; every GPU the library runs on
+// holds its own copy (4 MiB) at its own address until the process ends.  In host code the array's
+// name is only a handle: the device address comes from hipGetSymbolAddress, once per device.
+constexpr size_t kScratchWords = (size_t)1 << 20;
+static __device__ __align__(256) uint32_t g_scan_scratch[kScratchWords];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+uint32_t* g_scratch_ptr[kMaxDevices] = {};
+
+// The current device's copy of g_scan_scratch.
+int scratch_address(uint32_t** out)
+{
+    int dev = 0;
+    PS_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(PS_ERR_BAD_ARG, "device ordinal %d is beyond %d", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        PS_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(g_scan_scratch)));
+        if (p == nullptr) return fail(PS_ERR_NO_DEVICE, "hipGetSymbolAddress gave no address for the scratch array");
+        g_scratch_ptr[dev] = static_cast<uint32_t*>(p);
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+
+}  // namespace
+
 // ====================================================================== ABI
 
 extern "C" {
@@ -1034,6 +1068,35 @@ int ps_overflow_scan_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_n
     return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid, int) {
         hipLaunchKernelGGL(scan_chunks_kernel, grid, dim3(kAuxBlock), 0, s, b, chunk_numel, d_state);
     });
+}
+
+int ps_overflow_scan_chunks_noalloc(const ps_chunk* chunks, int n_chunks, size_t chunk_numel,
+                                    uint32_t* d_flag, ps_stream_t stream)
+{
+    if (!d_flag) return fail(PS_ERR_BAD_ARG, "d_flag is NULL");
+    ChunkList a;
+    if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, kScanTile)) return rc;
+    if (n_chunks == 0 || a.tiles_per_chunk == 0) return 0;
+    // one scratch word per workgroup of the first kernel
+    const size_t max_chunks = kScratchWords / a.tiles_per_chunk;  // 0 when one chunk alone is too long
+    if ((size_t)n_chunks > max_chunks)
+        return fail(PS_ERR_BAD_ARG,
+                    "%d chunks of %zu elements need %zu scratch words; this entry point holds %zu (at most %zu "
+                    "elements per call): split the list or use ps_overflow_scan_chunks",
+                    n_chunks, chunk_numel, (size_t)n_chunks * a.tiles_per_chunk, kScratchWords,
+                    kScratchWords * (size_t)kScanTile);
+    uint32_t* scratch = nullptr;
+    if (int rc = scratch_address(&scratch)) return rc;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    int rc = for_each_batch(a, [&](const ChunkBatch& b, dim3 grid, int first) {
+        hipLaunchKernelGGL(scan_chunks_partial_kernel, grid, dim3(kAuxBlock), 0, s, b, chunk_numel,
+                           scratch + (size_t)first * a.tiles_per_chunk);
+    });
+    if (rc) return rc;
+    hipLaunchKernelGGL(scan_reduce_kernel, dim3(1), dim3(kReduceBlock), 0, s, scratch,
+                       (size_t)n_chunks * a.tiles_per_chunk, d_flag);
+    PS_HIP(hipGetLastError());
+    return 0;
 }
 
 int ps_grad_to_chunk(const void* d_grad, int grad_is_half, uint16_t* d_slot_fp16, size_t numel,

@@ -360,6 +360,46 @@ __global__ void __launch_bounds__(kAuxBlock)
     block_flag_commit(hit, &st->overflow);
 }
 
+// The same probe without atomics and without a caller-side state: every workgroup leaves the OR over its tile in
+// its own word of a partial-result array; a second, single-workgroup kernel ORs those words into the caller's flag.
+__global__ void __launch_bounds__(kAuxBlock)
+    scan_chunks_partial_kernel(ChunkBatch b, size_t chunk_numel, uint32_t* __restrict__ partial)
+{
+    __shared__ uint32_t wave_hit[kAuxBlock / 64];
+    uint32_t hit = scan_tile_f16(b.c[blockIdx.y].param_fp16, chunk_numel, blockIdx.x);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) hit |= (uint32_t)__shfl_xor((int)hit, off, 64);
+    if ((threadIdx.x & 63) == 0) wave_hit[threadIdx.x >> 6] = hit;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t any = 0;
+#pragma unroll
+        for (int w = 0; w < kAuxBlock / 64; ++w) any |= wave_hit[w];
+        // written unconditionally: the array keeps whatever an earlier call left in it
+        partial[(size_t)blockIdx.y * gridDim.x + blockIdx.x] = any ? 1u : 0u;
+    }
+}
+
+constexpr int kReduceBlock = 1024;
+__global__ void __launch_bounds__(kReduceBlock)
+    scan_reduce_kernel(const uint32_t* __restrict__ partial, size_t n_words, uint32_t* flag)
+{
+    __shared__ uint32_t wave_hit[kReduceBlock / 64];
+    uint32_t hit = 0;
+#pragma unroll 8
+    for (size_t i = threadIdx.x; i < n_words; i += kReduceBlock) hit |= partial[i];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) hit |= (uint32_t)__shfl_xor((int)hit, off, 64);
+    if ((threadIdx.x & 63) == 0) wave_hit[threadIdx.x >> 6] = hit;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t any = 0;
+#pragma unroll
+        for (int w = 0; w < kReduceBlock / 64; ++w) any |= wave_hit[w];
+        if (any) *flag = 1u;  // sticky, like ps_step_state::overflow: only ever set here
+    }
+}
+
 // Backward-side producer: copy one gradient into its slot of the fp16 chunk
 // (patrickstar/core/hook.py:212-216) and probe it for inf/nan in the same pass
 // (loss_scaler.py:133-155), instead of a separate cast + sum + host sync per
