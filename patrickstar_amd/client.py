@@ -80,11 +80,19 @@ class PatrickStarClient:
         self.host_chunk_policy: Optional[Callable[[int], bool]] = None
         default_opts = {"with_mem_saving_comm": False, "with_mem_cache": False, "with_async_move": False}
         self.opt_config = dict(default_opts)
+        # Placement when no policy is given: decided once, from the HBM that is free when the model is registered.
+        self.use_hybrid_adam = True  # the optimizer's switch (fp16_cpu_adam.py:523-528); initialize_engine sets it
+        self.hbm_budget_bytes = None  # None: ask the device (torch.cuda.mem_get_info)
+        self.margin_use_ratio = 0.8  # the reference's default share of the margin (memtracer.py:190-214)
+        self.staging_slots = 2
+        self.placement = None  # what plan_placement decided, for inspection
         if config is not None:
             self.opt_config.update(config.get("opts", {}))
             if "host_chunk_policy" in config:
                 self.host_chunk_policy = config["host_chunk_policy"]
             self.host_keeps_fp16 = bool(config.get("host_keeps_fp16", True))
+            self.hbm_budget_bytes = config.get("hbm_budget_bytes", None)
+            self.margin_use_ratio = config.get("margin_use_ratio", 0.8)
 
     # -- building the lists -----------------------------------------------
     def append_chunk(self, data_type, chunk_type):
@@ -144,6 +152,47 @@ class PatrickStarClient:
             self.append_tensor(fp16_list, torch.half, AccessType.DATA, ChunkType.PARAM_FP16)
             self.append_tensor(fp32_list, torch.float, AccessType.DATA, ChunkType.PARAM_FP32)
 
+    def plan_placement(self, free_bytes=None):
+        """Decide which chunk positions keep their optimizer state (fp32 param, m, v) in pinned host memory.
+
+        The reference measures a memory margin during its warm-up iteration, turns it into a number of chunks,
+        ``margin / (chunk_size * 12) * margin_use_ratio`` (``patrickstar/core/memtracer/memtracer.py:190-214``), hands the
+        FIRST that many chunks to the GPU and updates the rest on the CPU (``patrickstar/ops/chunk_io_buff.py:234-239``),
+        all of it only when ``use_hybrid_adam`` is set (``patrickstar/ops/fp16_cpu_adam.py:523-528``).  Here the margin is
+        the HBM that is free when the model is registered (or ``config["client"]["hbm_budget_bytes"]``); the fp16 payloads
+        of all positions stay in HBM (2 B/element), a resident position costs 12 B/element more and the streaming path
+        needs ``staging_slots`` positions' worth of staging.  Everything fits -> every position is resident (the normal
+        case with 288 GB).  It does not fit -> the LAST positions go to the host if ``use_hybrid_adam``, else an error.
+        An explicit ``host_chunk_policy`` is left alone.  Called by ``register_model`` before any payload exists.
+        """
+        if self.host_chunk_policy is not None:
+            self.placement = {"source": "host_chunk_policy"}
+            return
+        n_positions = self.chunk_tensor_index.chunk_num(ChunkType.PARAM_FP16)
+        if free_bytes is None:
+            free_bytes = self.hbm_budget_bytes
+        if free_bytes is None:
+            if self.device.type != "cuda" or not torch.cuda.is_available():
+                self.placement = {"source": "no device to ask", "host_positions": []}
+                return
+            free_bytes = torch.cuda.mem_get_info(self.device)[0]
+        planned = plan_host_positions(
+            n_positions, self.default_chunk_size, free_bytes, staging_slots=self.staging_slots,
+            margin_use_ratio=self.margin_use_ratio, host_keeps_fp16=False,
+        )
+        self.placement = {"source": "free HBM", "free_bytes": free_bytes, "positions": n_positions,
+                          "host_positions": sorted(planned)}
+        if not planned:
+            return
+        if not self.use_hybrid_adam:
+            need = 14 * self.default_chunk_size * n_positions
+            raise RuntimeError(
+                f"{n_positions} chunk positions of {self.default_chunk_size} elements need {need} bytes of HBM for fp16 + "
+                f"fp32 + momentum + variance; {free_bytes} are free (x {self.margin_use_ratio}) and use_hybrid_adam is "
+                "False, so no optimizer state may live in host memory"
+            )
+        self.host_chunk_policy = planned.__contains__
+
     def register_model(self, model):
         """Register every module's own parameters in module CONSTRUCTION order (children finish
         constructing before their parent does), copy the initial values into the fp16 and fp32
@@ -159,6 +208,7 @@ class PatrickStarClient:
             self.register_module_params(m)
 
         visit(model)
+        self.plan_placement()
         self.allocate_payloads()
         for p16 in self.chunk_based_param_fp16:
             init = p16.data

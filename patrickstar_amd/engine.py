@@ -210,6 +210,9 @@ def initialize_engine(model_func, local_rank, config=None, client=None):
         cfg = config if config is not None else {}
         default_chunk_size = cfg.get("default_chunk_size", DEFAULT_CHUNK_SIZE)
         client = PatrickStarClient(rank=local_rank, default_chunk_size=default_chunk_size, config=cfg.get("client", None))
+        # hybrid Adam (optimizer state of some chunk positions in host memory) is the optimizer's switch; the client
+        # needs it when it places the payloads
+        client.use_hybrid_adam = bool(parse_config(config)[1].get("use_hybrid_adam", True))
         model = model_func()
         client.register_model(model)
     engine = PatrickStarEngine(model=model, client=client, config=config)

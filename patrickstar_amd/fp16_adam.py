@@ -141,6 +141,11 @@ class FP16Adam(torch.optim.Optimizer):
                     # the layout of momentum and variance chunks follows the fp16 parameter chunks
                     self.client.append_tensor_as_ref(sp, torch.float, AccessType.DATA, ctype, p)
         self.client.allocate_payloads()
+        if not use_hybrid_adam and self.client.host_fp16_chunk_ids:
+            raise ValueError(
+                "use_hybrid_adam=False keeps every optimizer state in HBM, but the client placed chunk positions "
+                f"{sorted(self.client.host_fp16_chunk_ids)} in host memory"
+            )
 
         self.opt_id = FP16Adam.optimizer_id
         FP16Adam.optimizer_id = FP16Adam.optimizer_id + 1

@@ -251,8 +251,23 @@ class DynamicLossScaler:
                 "ps_scaler_update",
             )
 
+    @property
+    def scale_tensor(self):
+        """The current loss scale as a 0-dim float64 tensor that ALIASES the device-resident state: it always holds
+        what the latest queued ``update_scale`` leaves there, and reading it on the device needs no host round trip."""
+        self.materialize()
+        off = _lib.ps_step_state.cur_scale.offset
+        return self._state[off : off + 8].view(torch.float64).reshape(())
+
     def backward(self, loss, retain_graph=False):
-        scaled_loss = loss * self.loss_scale
+        """``(loss * loss_scale).backward()`` (``patrickstar/fp16/loss_scaler.py:188-190``) with the scale taken from
+        the device: the host does not wait for the previous optimizer step to learn it.  The product is formed as
+        torch forms ``tensor * python_number``: in float for half and float losses, the scale narrowed to float."""
+        scale = self.scale_tensor
+        if loss.dtype == torch.float64:
+            scaled_loss = loss * scale
+        else:
+            scaled_loss = (loss.float() * scale.float()).to(loss.dtype)
         scaled_loss.backward(retain_graph=retain_graph)
 
     # -- checkpointing (the reference does not save its scaler; this is an addition) ----

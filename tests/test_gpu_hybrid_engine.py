@@ -386,3 +386,124 @@ def test_frozen_parameters_are_skipped_like_the_reference_skips_them(optim_type,
     live = [p for p in engine.module.parameters() if p.requires_grad]
     assert optimizer.state[live[0]]["step"] == (5 if loss_scale == 0 else 6)
     assert optimizer.state[frozen[0]]["step"] == 0
+
+
+def test_training_loop_never_reads_the_step_state_back(monkeypatch):
+    """engine.backward multiplies the loss by the device-resident scale; optimizer.step only queues work.  Over eight
+    iterations, one of them poisoned, nothing may call ps_state_read (the one synchronising entry point), and the
+    result must still be the oracle's bit for bit, scale sequence included."""
+    torch.manual_seed(0)
+    config = {
+        "optimizer": {"type": "AdamW", "params": {"lr": 1e-3, "betas": (0.9, 0.999), "eps": 1e-8, "weight_decay": 0.01}},
+        "fp16": {"enabled": True, "loss_scale": 0, "initial_scale_power": 7, "loss_scale_window": 3, "hysteresis": 2, "min_loss_scale": 1},
+        "default_chunk_size": 1100,
+    }
+    engine, optimizer = ps.initialize_engine(model_func=_MLP, local_rank=0, config=config)
+    client = engine.client
+    cl = client.chunk_list
+    pos = client.positions()
+    scaler = optimizer.loss_scaler
+    scaler.enable_log(16)
+    mirror = [{"p32": _snap(cl[q.fp32].payload), "m": _snap(cl[q.exp_avg].payload),
+               "v": _snap(cl[q.exp_avg_sq].payload), "p16": _snap(cl[q.fp16].payload)} for q in pos]
+    oscaler = oracle.scaler_from_config(config["fp16"])
+    oopt = oracle.OptimizerStepOracle(mirror, oscaler, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01,
+                                      use_adamw=True, tensors=tensor_spans(client, optimizer))
+    reads = []
+    real_read = ps.DynamicLossScaler._read
+    monkeypatch.setattr(ps.DynamicLossScaler, "_read", lambda self: reads.append(1) or real_read(self))
+    x = torch.randn(16, 24, device="cuda").half()
+    grads_per_iteration, expected_scales = [], []
+    for it in range(8):
+        loss = engine(x * (1.0 if it != 4 else 3e4))
+        engine.backward(loss)
+        grads_per_iteration.append([cl[q.fp16].payload.clone() for q in pos])  # device-side copies: no host sync
+        optimizer.step()
+    assert reads == [], "the training loop read the device-resident step state back"
+    monkeypatch.undo()
+    torch.cuda.synchronize()
+    for it, grads in enumerate(grads_per_iteration):
+        for c, g in zip(mirror, grads):
+            c["p16"][...] = g.cpu().numpy()
+        oopt.check_overflow()
+        assert oopt.step() == (it == 4)
+        expected_scales.append((it == 4, oscaler.loss_scale))
+    for i, (q, c) in enumerate(zip(pos, mirror)):
+        for key, cid in (("p32", q.fp32), ("m", q.exp_avg), ("v", q.exp_avg_sq), ("p16", q.fp16)):
+            assert_bits_equal(_snap(cl[cid].payload), c[key], f"position {i} {key}")
+    log = scaler.read_log()
+    assert [(f, s) for f, s in log] == expected_scales and [type(s) for _, s in log] == [type(s) for _, s in expected_scales]
+    assert optimizer.state[next(engine.module.parameters())]["step"] == 7
+    # the aliasing scale tensor tracks the state
+    assert float(scaler.scale_tensor) == scaler.loss_scale == oscaler.loss_scale
+
+
+class _Deep(torch.nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.layers = torch.nn.ModuleList([torch.nn.Linear(16, 16) for _ in range(6)])
+
+    def forward(self, x):
+        for layer in self.layers:
+            x = torch.tanh(layer(x))
+        return x.float().pow(2).mean()
+
+
+@pytest.mark.parametrize("arithmetic", ["operator", "torch"])
+def test_engine_places_optimizer_state_by_the_hbm_budget(arithmetic):
+    """No policy given, an artificially small HBM budget: initialize_engine keeps the first two positions' optimizer
+    state in HBM and puts the other four in pinned host memory (use_hybrid_adam), and training is bit for bit what the
+    reference computes under that placement: the operator everywhere, or (arithmetic="torch") the torch formula on the
+    resident positions and the operator on the host ones."""
+    torch.manual_seed(0)
+    config = {
+        "optimizer": {"type": "AdamW", "params": {"lr": 1e-3, "betas": (0.9, 0.999), "eps": 1e-8, "weight_decay": 0.01,
+                                                  "use_hybrid_adam": True, "arithmetic": arithmetic}},
+        "fp16": {"enabled": True, "loss_scale": 0, "initial_scale_power": 7, "loss_scale_window": 3, "hysteresis": 2, "min_loss_scale": 1},
+        "default_chunk_size": 300,
+        "client": {"hbm_budget_bytes": 25000},
+    }
+    engine, optimizer = ps.initialize_engine(model_func=_Deep, local_rank=0, config=config)
+    client = engine.client
+    assert client.placement["host_positions"] == [2, 3, 4, 5]
+    cl = client.chunk_list
+    pos = client.positions()
+    assert [q.on_host for q in pos] == [False, False, True, True, True, True]
+    for q in pos:
+        assert cl[q.fp16].payload.is_cuda
+        for cid in (q.fp32, q.exp_avg, q.exp_avg_sq):
+            assert cl[cid].payload.is_pinned() == q.on_host and cl[cid].payload.is_cuda != q.on_host
+    mirror = [{"p32": _snap(cl[q.fp32].payload), "m": _snap(cl[q.exp_avg].payload),
+               "v": _snap(cl[q.exp_avg_sq].payload), "p16": _snap(cl[q.fp16].payload)} for q in pos]
+    oscaler = oracle.scaler_from_config(config["fp16"])
+    oopt = oracle.OptimizerStepOracle(mirror, oscaler, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01,
+                                      use_adamw=True, tensors=tensor_spans(client, optimizer), arithmetic=arithmetic,
+                                      operator_chunks=(2, 3, 4, 5))
+    x = torch.randn(8, 16, device="cuda").half()
+    for it in range(6):
+        loss = engine(x * (1.0 if it != 2 else 6e4))
+        engine.backward(loss)
+        for q, c in zip(pos, mirror):
+            c["p16"][...] = _snap(cl[q.fp16].payload)
+        optimizer.step()
+        torch.cuda.synchronize()
+        oopt.check_overflow()
+        assert oopt.step() == (it == 2)
+        for i, (q, c) in enumerate(zip(pos, mirror)):
+            for key, cid in (("p32", q.fp32), ("m", q.exp_avg), ("v", q.exp_avg_sq), ("p16", q.fp16)):
+                assert_bits_equal(_snap(cl[cid].payload), c[key], f"{arithmetic} iteration {it} position {i} {key}")
+        assert optimizer.loss_scaler.loss_scale == oscaler.loss_scale
+
+
+def test_engine_refuses_host_placement_without_hybrid_adam():
+    config = {
+        "optimizer": {"type": "Adam", "params": {"lr": 1e-3, "use_hybrid_adam": False}},
+        "default_chunk_size": 300,
+        "client": {"hbm_budget_bytes": 25000},
+    }
+    with pytest.raises(RuntimeError, match="use_hybrid_adam is False"):
+        ps.initialize_engine(model_func=_Deep, local_rank=0, config=config)
+    # with room for everything the switch changes nothing
+    config["client"] = {"hbm_budget_bytes": 10**9}
+    engine, optimizer = ps.initialize_engine(model_func=_Deep, local_rank=0, config=config)
+    assert not any(q.on_host for q in engine.client.positions())

@@ -409,3 +409,36 @@ def test_step_tables_follow_the_reference_call_order_and_skip_frozen_parameters(
     assert opt._tensor_table is None and opt._tables[1] == 1 and opt._operator_calls == 3
     pat = opt._calls._obj
     assert (pat.n_calls, pat.first_chunk, pat.first_offset, pat.first_numel) == (3, 0, 14, 3)
+
+
+def test_placement_is_decided_from_the_free_hbm_when_the_model_is_registered():
+    """use_hybrid_adam + a memory margin decide where optimizer state lives (fp16_cpu_adam.py:523-528,
+    memtracer.py:190-214, chunk_io_buff.py:234-239): everything resident when it fits, the FIRST positions resident
+    when it does not, an error when it does not and hybrid Adam is off; an explicit policy is left alone."""
+    def client_with(n_layers=6, **cfg):
+        client = ps.PatrickStarClient(0, 300, device="cpu", config=cfg or None)
+        for _ in range(n_layers):
+            client.register_module_params(torch.nn.Linear(16, 16))  # 272 elements: one position each
+        return client
+
+    per = 14 * 300
+    c = client_with()
+    c.plan_placement(free_bytes=6 * per / 0.8)
+    assert c.host_chunk_policy is None and c.placement["host_positions"] == []
+    # 20,000 usable bytes: 6 fp16 payloads (3,600) + 2 staging slots (7,200) leave room for 2 resident states (3,600 each)
+    c = client_with(hbm_budget_bytes=25000)
+    c.plan_placement()
+    assert c.placement["host_positions"] == [2, 3, 4, 5] and c.placement["free_bytes"] == 25000
+    assert [c.host_chunk_policy(i) for i in range(6)] == [False, False, True, True, True, True]
+    c = client_with(hbm_budget_bytes=25000)
+    c.use_hybrid_adam = False
+    with pytest.raises(RuntimeError, match="use_hybrid_adam is False"):
+        c.plan_placement()
+    keep = lambda pos: pos == 0
+    c = client_with(hbm_budget_bytes=1, host_chunk_policy=keep)
+    c.plan_placement()
+    assert c.host_chunk_policy is keep and c.placement == {"source": "host_chunk_policy"}
+    # no budget and no GPU to ask: nothing is moved
+    c = client_with()
+    c.plan_placement()
+    assert c.host_chunk_policy is None
