@@ -228,7 +228,8 @@ int ps_adam_step_chunks_gated(int optimizer_id, double lr, double epsilon, doubl
  * Same arithmetic, clamp and 28 B/element as the chunk-list form.  Every tensor is one operator call of the
  * reference's loop, tensors[0] the first of the step (zero-length tensors included: the reference calls the
  * operator for them too); follow a device-gated call with ps_scaler_update(..., n_tensors).
- * Up to 48 tensors go into one launch. */
+ * Tensors of (nearly) equal length share a launch, up to 64 of them; the order of the list decides nothing
+ * but which tensor is the first call. */
 int ps_adam_step_tensors(int optimizer_id, size_t step, double lr, double beta1, double beta2,
                          double epsilon, double weight_decay, int bias_correction,
                          const ps_chunk* tensors, const size_t* numels, int n_tensors,

@@ -37,6 +37,7 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -44,6 +45,7 @@
 #include <memory>
 #include <mutex>
 #include <unordered_map>
+#include <vector>
 
 #include "ps_adam.h"
 
@@ -287,40 +289,40 @@ void launch_gated_batch(int arith, const ChunkBatch& b, dim3 grid, size_t chunk_
 }
 
 template <int ARITH, int WD>
-void launch_tensors_wd(const TensorBatch& b, unsigned n_tiles, const StepConsts& c, hipStream_t s)
+void launch_tensors_wd(const TensorBatch& b, dim3 grid, const StepConsts& c, hipStream_t s)
 {
-    dim3 grid(n_tiles), block(kBlock);
+    dim3 block(kBlock);
     if (c.unscale == UNSCALE_MUL)
-        hipLaunchKernelGGL((adam_tensors_kernel<ARITH, WD, UNSCALE_MUL>), grid, block, kTensorLdsBytes, s, b, c);
+        hipLaunchKernelGGL((adam_tensors_kernel<ARITH, WD, UNSCALE_MUL>), grid, block, kLdsBytes, s, b, c);
     else if (ARITH == PS_ARITH_OPERATOR && c.unscale == UNSCALE_DIV)
-        hipLaunchKernelGGL((adam_tensors_kernel<ARITH, WD, UNSCALE_DIV>), grid, block, kTensorLdsBytes, s, b, c);
+        hipLaunchKernelGGL((adam_tensors_kernel<ARITH, WD, UNSCALE_DIV>), grid, block, kLdsBytes, s, b, c);
     else
-        hipLaunchKernelGGL((adam_tensors_kernel<ARITH, WD, UNSCALE_NONE>), grid, block, kTensorLdsBytes, s, b, c);
+        hipLaunchKernelGGL((adam_tensors_kernel<ARITH, WD, UNSCALE_NONE>), grid, block, kLdsBytes, s, b, c);
 }
 
 template <int ARITH>
-void launch_tensors_arith(const TensorBatch& b, unsigned n_tiles, const StepConsts& c, hipStream_t s)
+void launch_tensors_arith(const TensorBatch& b, dim3 grid, const StepConsts& c, hipStream_t s)
 {
     if (c.wd_mode == WD_DECOUPLED)
-        launch_tensors_wd<ARITH, WD_DECOUPLED>(b, n_tiles, c, s);
+        launch_tensors_wd<ARITH, WD_DECOUPLED>(b, grid, c, s);
     else if (c.wd_mode == WD_L2)
-        launch_tensors_wd<ARITH, WD_L2>(b, n_tiles, c, s);
+        launch_tensors_wd<ARITH, WD_L2>(b, grid, c, s);
     else
-        launch_tensors_wd<ARITH, WD_NONE>(b, n_tiles, c, s);
+        launch_tensors_wd<ARITH, WD_NONE>(b, grid, c, s);
 }
 
 template <int ARITH>
-void launch_tensors_gated_arith(const TensorBatch& b, unsigned n_tiles, const GatedArgs& ga,
+void launch_tensors_gated_arith(const TensorBatch& b, dim3 grid, const GatedArgs& ga,
                                 const ps_step_state* d_state, hipStream_t s)
 {
-    dim3 grid(n_tiles), block(kBlock);
+    dim3 block(kBlock);
     const bool decay = ARITH == PS_ARITH_OPERATOR ? (float)ga.wd > 0.0f : ga.wd != 0.0;
     if (decay && ga.adamw)
-        hipLaunchKernelGGL((adam_tensors_gated_kernel<ARITH, WD_DECOUPLED>), grid, block, kTensorLdsBytes, s, b, ga, d_state);
+        hipLaunchKernelGGL((adam_tensors_gated_kernel<ARITH, WD_DECOUPLED>), grid, block, kLdsBytes, s, b, ga, d_state);
     else if (decay)
-        hipLaunchKernelGGL((adam_tensors_gated_kernel<ARITH, WD_L2>), grid, block, kTensorLdsBytes, s, b, ga, d_state);
+        hipLaunchKernelGGL((adam_tensors_gated_kernel<ARITH, WD_L2>), grid, block, kLdsBytes, s, b, ga, d_state);
     else
-        hipLaunchKernelGGL((adam_tensors_gated_kernel<ARITH, WD_NONE>), grid, block, kTensorLdsBytes, s, b, ga, d_state);
+        hipLaunchKernelGGL((adam_tensors_gated_kernel<ARITH, WD_NONE>), grid, block, kLdsBytes, s, b, ga, d_state);
 }
 
 // The Python numbers of one step as they cross the boundary.
@@ -342,8 +344,8 @@ StepConsts operator_step_consts(HostAdam& o, size_t step, const HyperParams& hp,
     o.set((float)hp.lr, (float)hp.eps, (float)hp.wd);
     StepConsts c;
     finish_consts(c, o.alpha, o.beta1, o.beta2, o.eps, o.weight_decay, o.adamw, o.beta1_t,
-                  o.beta2_t, first_b1t, first_b2t, hp.bias_correction, (float)hp.loss_scale,
-                  clamp_bound(o.grad_clamp, hp.loss_scale));
+                  o.beta2_t, hp.bias_correction, (float)hp.loss_scale, clamp_bound(o.grad_clamp, hp.loss_scale));
+    bias_scalars(o.alpha, first_b1t, first_b2t, hp.bias_correction, &c.first_step_size, &c.first_bc2inv);
     return c;
 }
 
@@ -596,7 +598,7 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
     StepConsts c;
     // the reference clamps gradients in Python before it calls the operator: not here
     finish_consts(c, o->alpha, o->beta1, o->beta2, o->eps, o->weight_decay, o->adamw, o->beta1_t,
-                  o->beta2_t, o->beta1_t, o->beta2_t, bias_correction != 0, loss_scale, 0.0f);
+                  o->beta2_t, bias_correction != 0, loss_scale, 0.0f);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const size_t gsz = grads_are_half ? 2 : 4;
     const char* gbytes = static_cast<const char*>(d_grads);
@@ -721,7 +723,7 @@ int ps_adam_step_tensors(int optimizer_id, size_t step, double lr, double beta1,
         const ps_chunk& t = tensors[i];
         if (numels[i] > 0 && (!t.param_fp32 || !t.exp_avg || !t.exp_avg_sq || !t.param_fp16))
             return fail(PS_ERR_BAD_ARG, "tensor %d has a NULL address", i);
-        if ((numels[i] + kTile - 1) / kTile > kMaxGridX)
+        if ((numels[i] + kTile - 1) / kTile >= kMaxGridX || numels[i] > kNumelMask)
             return fail(PS_ERR_BAD_ARG, "tensor %d: numel = %zu is beyond the launch grid", i, numels[i]);
     }
     const int arith = o->arith;
@@ -733,44 +735,68 @@ int ps_adam_step_tensors(int optimizer_id, size_t step, double lr, double beta1,
         c = arith == PS_ARITH_TORCH ? torch_step_consts(*o, step, hp) : operator_step_consts(*o, step, hp, n_tensors);
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    TensorBatch b;
-    int in_batch = 0;
-    size_t tiles = 0;
-    auto flush = [&]() -> int {
-        if (in_batch == 0) return 0;
-        for (int i = in_batch; i < 64; ++i) b.first_tile[i] = 0xFFFFFFFFu;
-        if (d_state == nullptr) {
-            if (arith == PS_ARITH_TORCH)
-                launch_tensors_arith<PS_ARITH_TORCH>(b, (unsigned)tiles, c, s);
-            else
-                launch_tensors_arith<PS_ARITH_OPERATOR>(b, (unsigned)tiles, c, s);
-        } else {
-            if (arith == PS_ARITH_TORCH)
-                launch_tensors_gated_arith<PS_ARITH_TORCH>(b, (unsigned)tiles, ga, d_state, s);
-            else
-                launch_tensors_gated_arith<PS_ARITH_OPERATOR>(b, (unsigned)tiles, ga, d_state, s);
-        }
-        PS_HIP(hipGetLastError());
-        in_batch = 0;
-        tiles = 0;
-        b.first_call = -1;
-        return 0;
+    // Where each tensor's tile grid starts (the fp32 parameter's first 1 KiB boundary; what lies in front of it is a
+    // tile of its own) and how many tiles it has.  Addresses that are not even element-aligned keep the plain
+    // numbering.
+    struct Item {
+        int index;
+        uint32_t head;
+        size_t body, tiles;
     };
-    memset(&b, 0, sizeof(b));
-    b.first_call = -1;
+    std::vector<Item> items;
+    try {
+        items.reserve((size_t)n_tensors);
+    } catch (const std::exception&) {  // nothing may throw across the boundary
+        return fail(PS_ERR_BAD_ARG, "no host memory for a list of %d tensors", n_tensors);
+    }
     for (int i = 0; i < n_tensors; ++i) {
         if (numels[i] == 0) continue;
-        const size_t t_i = (numels[i] + kTile - 1) / kTile;
-        if (in_batch == kTensorBatch || tiles + t_i > kMaxGridX)
-            if (int rc = flush()) return rc;
-        if (i == 0 && arith == PS_ARITH_OPERATOR) b.first_call = in_batch;
-        b.t[in_batch] = tensors[i];
-        b.numel[in_batch] = numels[i];
-        b.first_tile[in_batch] = (uint32_t)tiles;
-        tiles += t_i;
-        in_batch += 1;
+        const uintptr_t p_addr = reinterpret_cast<uintptr_t>(tensors[i].param_fp32);
+        size_t head = p_addr % sizeof(float) ? 0 : (kTile - (p_addr / sizeof(float)) % kTile) % kTile;
+        if (head > numels[i]) head = numels[i];
+        const size_t body = numels[i] - head;
+        items.push_back(Item{i, (uint32_t)head, body, (head ? 1 : 0) + (body + kTile - 1) / kTile});
     }
-    return flush();
+    // Longest first; one launch takes tensors of nearly the same length (its grid is as wide as the longest of
+    // them: at most a tenth of a launch's workgroups find nothing to do), short tensors all together.
+    std::stable_sort(items.begin(), items.end(), [](const Item& a, const Item& b) { return a.tiles > b.tiles; });
+    constexpr size_t kShortTensorTiles = 256;
+    TensorBatch b;
+    size_t next = 0;
+    while (next < items.size()) {
+        memset(&b, 0, sizeof(b));
+        b.first_call = -1;
+        const size_t widest = items[next].tiles;
+        int in_batch = 0;
+        while (next < items.size() && in_batch < kTensorBatch &&
+               (items[next].tiles * 10 >= widest * 9 || widest <= kShortTensorTiles)) {
+            const Item& it = items[next];
+            ps_chunk t = tensors[it.index];
+            t.param_fp32 += it.head;
+            t.exp_avg += it.head;
+            t.exp_avg_sq += it.head;
+            t.param_fp16 += it.head;
+            b.t[in_batch] = t;
+            b.numel_head[in_batch] = (uint64_t)it.body | ((uint64_t)it.head << 56);
+            if (it.index == 0 && arith == PS_ARITH_OPERATOR) b.first_call = in_batch;
+            in_batch += 1;
+            next += 1;
+        }
+        const dim3 grid((unsigned)widest, (unsigned)in_batch);
+        if (d_state == nullptr) {
+            if (arith == PS_ARITH_TORCH)
+                launch_tensors_arith<PS_ARITH_TORCH>(b, grid, c, s);
+            else
+                launch_tensors_arith<PS_ARITH_OPERATOR>(b, grid, c, s);
+        } else {
+            if (arith == PS_ARITH_TORCH)
+                launch_tensors_gated_arith<PS_ARITH_TORCH>(b, grid, ga, d_state, s);
+            else
+                launch_tensors_gated_arith<PS_ARITH_OPERATOR>(b, grid, ga, d_state, s);
+        }
+        PS_HIP(hipGetLastError());
+    }
+    return 0;
 }
 
 int ps_restore_fp16_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_numel,

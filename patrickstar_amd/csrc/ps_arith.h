@@ -99,16 +99,17 @@ __host__ __device__ inline void bias_scalars(float lr, float beta1_t, float beta
     *bc2inv_out = bc2inv;
 }
 
-// beta1_t / beta2_t: beta^t of the calls after the first; first_beta1_t / first_beta2_t: of the first call.
+// beta1_t / beta2_t: beta^t of the call(s) the constants are for.  The first call's pair is set to the same
+// values; a caller whose step has a first call with another beta^t overwrites it (bias_scalars).
 __host__ __device__ inline void finish_consts(StepConsts& c, float lr, float beta1, float beta2,
                                               float eps, float wd, bool adamw, float beta1_t,
-                                              float beta2_t, float first_beta1_t, float first_beta2_t,
-                                              bool bias_correction, float loss_scale, float clip)
+                                              float beta2_t, bool bias_correction, float loss_scale, float clip)
 {
     c.clip = clip;
     float bc2inv;
     bias_scalars(lr, beta1_t, beta2_t, bias_correction, &c.step_size, &bc2inv);
-    bias_scalars(lr, first_beta1_t, first_beta2_t, bias_correction, &c.first_step_size, &c.first_bc2inv);
+    c.first_step_size = c.step_size;
+    c.first_bc2inv = bc2inv;
     c.beta1 = beta1;
     c.beta2 = beta2;
     c.b1m = 1.0f - beta1;

@@ -51,8 +51,11 @@ struct GatedArgs {
 // The weight-decay form is known to the host; the unscale form depends on
 // the device-resident scale and is a uniform branch around the arithmetic.
 // Step constants of a device-decided step, formed by every wave from the device-resident state.
+// `with_first_call`: this workgroup's chunk (tensor) holds elements of the step's first operator call; every
+// other workgroup is spared the second pair of bias scalars (a divide and a square root per wave).
 template <int ARITH>
-__device__ __forceinline__ StepConsts gated_consts(const GatedArgs& ga, const ps_step_state* __restrict__ st)
+__device__ __forceinline__ StepConsts gated_consts(const GatedArgs& ga, const ps_step_state* __restrict__ st,
+                                                   bool with_first_call)
 {
     StepConsts c;
     const float clip = clamp_bound(ga.grad_clamp, st->cur_scale);
@@ -60,10 +63,13 @@ __device__ __forceinline__ StepConsts gated_consts(const GatedArgs& ga, const ps
         // The operator takes its scalars and loss_scale as C floats: the Python numbers narrow (RNE).
         // one operator call in the step: everything is that (first) call
         const bool one_call = ga.n_calls <= 1;
-        finish_consts(c, (float)ga.lr, st->beta1, st->beta2, (float)ga.eps, (float)ga.wd,
-                      ga.adamw != 0, one_call ? st->beta1_t_next : st->beta1_t_rest,
-                      one_call ? st->beta2_t_next : st->beta2_t_rest, st->beta1_t_next,
-                      st->beta2_t_next, ga.bias_correction != 0, (float)st->cur_scale, clip);
+        const float b1t = one_call ? st->beta1_t_next : st->beta1_t_rest;
+        const float b2t = one_call ? st->beta2_t_next : st->beta2_t_rest;
+        finish_consts(c, (float)ga.lr, st->beta1, st->beta2, (float)ga.eps, (float)ga.wd, ga.adamw != 0, b1t, b2t,
+                      ga.bias_correction != 0, (float)st->cur_scale, clip);
+        if (with_first_call && !one_call)
+            bias_scalars((float)ga.lr, st->beta1_t_next, st->beta2_t_next, ga.bias_correction != 0, &c.first_step_size,
+                         &c.first_bc2inv);
     } else {
         const bool bc = ga.bias_correction != 0;
         torch_consts(c, ga.lr, st->beta1_f64, st->beta2_f64, ga.eps, ga.wd, ga.adamw != 0,
@@ -84,7 +90,7 @@ __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
         restore_tile(ch.param_fp32, ch.param_fp16, base, chunk_numel);
         return;
     }
-    const StepConsts c = gated_consts<ARITH>(ga, st);
+    const StepConsts c = gated_consts<ARITH>(ga, st, fc.chunk == (int)blockIdx.y);
     size_t lo, hi;
     first_call_span(fc, &lo, &hi);
     adam_tile<ARITH, WD, UNSCALE_RUNTIME>(c, ch, base, chunk_numel, lo, hi);
@@ -96,66 +102,93 @@ __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
 // parameter's momentum and variance do not sit at the parameter's own offset (the reference packs
 // optimizer-state tensors first-fit in parameters() order, patrickstar/core/client.py:282-309, so the
 // whole-chunk pass does not apply and the reference loops over tensors, fp16_cpu_adam.py:336-468).
-// Grid: x = tile of the batch; tiles are numbered tensor by tensor.  A wave finds its tensor with one
-// 64-lane load of the batch's first-tile table, a ballot and a population count.
+//
+// Grid: x = tile inside a tensor, y = tensor inside the batch, exactly like the chunk-list kernels, so that a
+// wave reaches its first data load after ONE scalar load of its descriptor.  The host sorts the tensors by length
+// and puts tensors of (nearly) the same length into one launch; x runs up to the longest tensor of the batch and
+// the few workgroups beyond a shorter tensor's end leave at once.  (A one-dimensional grid over all tiles with a
+// tile -> tensor table costs a second dependent scalar load per wave: 4 to 10 % at this kernel's operating point.)
+//
+// Tensors start at arbitrary element offsets of their chunks.  The tile grid of a tensor is laid over the ADDRESSES
+// of its fp32 parameter, not over its element numbers: the up to 255 elements in front of the parameter's first
+// 1 KiB boundary form a tile of their own (done element by element), and every later tile is one whole aligned KiB
+// of the fp32 parameter (and of every other list that shares the parameter's phase: the fp16 list does in the
+// reference's layout).  Wave accesses at a 256-, 512- or 768-byte phase of a KiB measured 6 to 8 % slower than
+// aligned ones (all four lists shifted), 2 % with only the fp16 list at a 256-byte phase.
 
-// A wave of the tensor-list kernels starts with one more dependent load (the lookup) than a wave of the
-// chunk-list kernels; 13 resident workgroups per CU (12 KiB each) instead of 9 make up for it
-// (GPT-2 XL's 580 tensors, 1.56 G elements: 7.42 ms with 12 KiB, 7.97 ms with 17 KiB, 7.05 ms as one chunk).
-#ifndef PS_TENSOR_LDS_KB
-#define PS_TENSOR_LDS_KB 12
-#endif
-constexpr unsigned kTensorLdsBytes = PS_TENSOR_LDS_KB * 1024u;
-#ifndef PS_TENSOR_BATCH
-#define PS_TENSOR_BATCH 48
-#endif
-constexpr int kTensorBatch = PS_TENSOR_BATCH;
-static_assert(kTensorBatch <= 64, "the first-tile table is read by one wave");
+constexpr int kTensorBatch = 64;
 struct TensorBatch {
-    ps_chunk t[kTensorBatch];          // fp32 param, exp_avg, exp_avg_sq, fp16 slot of each tensor
-    uint64_t numel[kTensorBatch];
-    uint32_t first_tile[64];           // of tensor i; 0xFFFFFFFF beyond the last tensor
+    ps_chunk t[kTensorBatch];          // fp32 param, exp_avg, exp_avg_sq, fp16 slot: addresses of the tile grid's origin
+    uint64_t numel_head[kTensorBatch]; // low 56 bits: elements from the origin on; high 8 bits: elements in front of it
+                                       // (0..255; they are tile 0 of the tensor if there are any)
     int first_call;                    // which tensor of the batch is the step's first operator call; -1: none
 };
+constexpr uint64_t kNumelMask = (1ull << 56) - 1;
 
-// A tensor is one operator call: its tiles take the first call's scalars as a whole, or none does.
-__device__ __forceinline__ void tensor_call_span(const TensorBatch& b, int k, size_t* lo, size_t* hi)
+// The elements in front of a tensor's tile grid: indices -head .. -1 relative to the descriptor's addresses.
+template <int ARITH, int WD, int UNS>
+__device__ __forceinline__ void adam_head(const StepConsts& c, const ps_chunk& t, int head, bool first_call)
 {
-    *lo = 0;
-    *hi = k == b.first_call ? (size_t)b.numel[k] : 0;
-}
-
-__device__ __forceinline__ int tensor_of_tile(const TensorBatch& b, uint32_t tile)
-{
-    const uint32_t first = b.first_tile[threadIdx.x & 63];
-    // the same in every lane: say so, and descriptor and length come through scalar loads
-    return __builtin_amdgcn_readfirstlane(__popcll(__ballot(tile >= first)) - 1);
+    const float step_size = first_call ? c.first_step_size : c.step_size;
+    const float bc2inv = first_call ? c.first_bc2inv : c.bc2inv;
+    for (int j = threadIdx.x; j < head; j += kBlock) {
+        const ptrdiff_t i = (ptrdiff_t)j - head;
+        float g = half_bits_to_float(t.param_fp16[i]);
+        float p = t.param_fp32[i], m = t.exp_avg[i], v = t.exp_avg_sq[i];
+        element_any<ARITH, WD, UNS>(c, step_size, bc2inv, g, p, m, v);
+        t.param_fp32[i] = p;
+        t.exp_avg[i] = m;
+        t.exp_avg_sq[i] = v;
+        t.param_fp16[i] = (uint16_t)float_to_half_bits(p);
+    }
 }
 
 template <int ARITH, int WD, int UNS>
 __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
     adam_tensors_kernel(TensorBatch b, StepConsts c)
 {
-    const int k = tensor_of_tile(b, blockIdx.x);
-    size_t lo, hi;
-    tensor_call_span(b, k, &lo, &hi);
-    adam_tile<ARITH, WD, UNS>(c, b.t[k], (size_t)(blockIdx.x - b.first_tile[k]) * kTile, (size_t)b.numel[k], lo, hi);
+    const int k = blockIdx.y;
+    const uint64_t nh = b.numel_head[k];
+    const size_t numel = (size_t)(nh & kNumelMask);
+    const int head = (int)(nh >> 56);
+    const bool first = k == b.first_call;  // a tensor is one operator call: all of its tiles, or none
+    const ptrdiff_t tile = (ptrdiff_t)blockIdx.x - (head ? 1 : 0);
+    if (tile < 0) {
+        adam_head<ARITH, WD, UNS>(c, b.t[k], head, first);
+        return;
+    }
+    const size_t base = (size_t)tile * kTile;
+    if (base >= numel) return;  // the grid is as wide as the longest tensor of the batch
+    adam_tile<ARITH, WD, UNS>(c, b.t[k], base, numel, 0, first ? numel : 0);
 }
 
 template <int ARITH, int WD>
 __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
     adam_tensors_gated_kernel(TensorBatch b, GatedArgs ga, const ps_step_state* __restrict__ st)
 {
-    const int k = tensor_of_tile(b, blockIdx.x);
-    const size_t base = (size_t)(blockIdx.x - b.first_tile[k]) * kTile;
+    const int k = blockIdx.y;
+    const uint64_t nh = b.numel_head[k];
+    const size_t numel = (size_t)(nh & kNumelMask);
+    const int head = (int)(nh >> 56);
+    const bool first = k == b.first_call;
+    const ptrdiff_t tile = (ptrdiff_t)blockIdx.x - (head ? 1 : 0);
+    const size_t base = tile < 0 ? 0 : (size_t)tile * kTile;
+    if (tile >= 0 && base >= numel) return;
     if (st->overflow) {
-        restore_tile(b.t[k].param_fp32, b.t[k].param_fp16, base, (size_t)b.numel[k]);
+        if (tile < 0) {
+            for (int j = threadIdx.x; j < head; j += kBlock)
+                b.t[k].param_fp16[(ptrdiff_t)j - head] = (uint16_t)float_to_half_bits(b.t[k].param_fp32[(ptrdiff_t)j - head]);
+        } else {
+            restore_tile(b.t[k].param_fp32, b.t[k].param_fp16, base, numel);
+        }
         return;
     }
-    const StepConsts c = gated_consts<ARITH>(ga, st);
-    size_t lo, hi;
-    tensor_call_span(b, k, &lo, &hi);
-    adam_tile<ARITH, WD, UNSCALE_RUNTIME>(c, b.t[k], base, (size_t)b.numel[k], lo, hi);
+    const StepConsts c = gated_consts<ARITH>(ga, st, first);
+    if (tile < 0) {
+        adam_head<ARITH, WD, UNSCALE_RUNTIME>(c, b.t[k], head, first);
+        return;
+    }
+    adam_tile<ARITH, WD, UNSCALE_RUNTIME>(c, b.t[k], base, numel, 0, first ? numel : 0);
 }
 
 __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
