@@ -53,28 +53,51 @@ struct GatedArgs {
 // Step constants of a device-decided step, formed by every wave from the device-resident state.
 // `with_first_call`: this workgroup's chunk (tensor) holds elements of the step's first operator call; every
 // other workgroup is spared the second pair of bias scalars (a divide and a square root per wave).
+// What a device-decided step reads from the device-resident state, fetched in one go (a handful of wide scalar
+// loads issued together) instead of field by field as the arithmetic gets to them.
+struct StateView {
+    double cur_scale, beta1_f64, beta2_f64, bc1_next, bc2_next;
+    float beta1, beta2, b1t_next, b2t_next, b1t_rest, b2t_rest;
+    uint32_t overflow;
+};
+__device__ __forceinline__ StateView view_state(const ps_step_state* __restrict__ st)
+{
+    StateView s;
+    s.overflow = st->overflow;
+    s.cur_scale = st->cur_scale;
+    s.beta1 = st->beta1;
+    s.beta2 = st->beta2;
+    s.b1t_next = st->beta1_t_next;
+    s.b2t_next = st->beta2_t_next;
+    s.b1t_rest = st->beta1_t_rest;
+    s.b2t_rest = st->beta2_t_rest;
+    s.beta1_f64 = st->beta1_f64;
+    s.beta2_f64 = st->beta2_f64;
+    s.bc1_next = st->bias_correction1_next;
+    s.bc2_next = st->bias_correction2_next;
+    return s;
+}
+
 template <int ARITH>
-__device__ __forceinline__ StepConsts gated_consts(const GatedArgs& ga, const ps_step_state* __restrict__ st,
-                                                   bool with_first_call)
+__device__ __forceinline__ StepConsts gated_consts(const GatedArgs& ga, const StateView& st, bool with_first_call)
 {
     StepConsts c;
-    const float clip = clamp_bound(ga.grad_clamp, st->cur_scale);
+    const float clip = clamp_bound(ga.grad_clamp, st.cur_scale);
     if (ARITH == PS_ARITH_OPERATOR) {
         // The operator takes its scalars and loss_scale as C floats: the Python numbers narrow (RNE).
         // one operator call in the step: everything is that (first) call
         const bool one_call = ga.n_calls <= 1;
-        const float b1t = one_call ? st->beta1_t_next : st->beta1_t_rest;
-        const float b2t = one_call ? st->beta2_t_next : st->beta2_t_rest;
-        finish_consts(c, (float)ga.lr, st->beta1, st->beta2, (float)ga.eps, (float)ga.wd, ga.adamw != 0, b1t, b2t,
-                      ga.bias_correction != 0, (float)st->cur_scale, clip);
+        const float b1t = one_call ? st.b1t_next : st.b1t_rest;
+        const float b2t = one_call ? st.b2t_next : st.b2t_rest;
+        finish_consts(c, (float)ga.lr, st.beta1, st.beta2, (float)ga.eps, (float)ga.wd, ga.adamw != 0, b1t, b2t,
+                      ga.bias_correction != 0, (float)st.cur_scale, clip);
         if (with_first_call && !one_call)
-            bias_scalars((float)ga.lr, st->beta1_t_next, st->beta2_t_next, ga.bias_correction != 0, &c.first_step_size,
+            bias_scalars((float)ga.lr, st.b1t_next, st.b2t_next, ga.bias_correction != 0, &c.first_step_size,
                          &c.first_bc2inv);
     } else {
         const bool bc = ga.bias_correction != 0;
-        torch_consts(c, ga.lr, st->beta1_f64, st->beta2_f64, ga.eps, ga.wd, ga.adamw != 0,
-                     bc ? st->bias_correction1_next : 1.0, bc ? st->bias_correction2_next : 1.0,
-                     st->cur_scale, clip);
+        torch_consts(c, ga.lr, st.beta1_f64, st.beta2_f64, ga.eps, ga.wd, ga.adamw != 0, bc ? st.bc1_next : 1.0,
+                     bc ? st.bc2_next : 1.0, st.cur_scale, clip);
     }
     return c;
 }
@@ -86,14 +109,16 @@ __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
 {
     const ps_chunk& ch = b.c[blockIdx.y];
     const size_t base = (size_t)blockIdx.x * kTile;
-    if (st->overflow) {
+    const StateView sv = view_state(st);
+    if (sv.overflow) {
         restore_tile(ch.param_fp32, ch.param_fp16, base, chunk_numel);
         return;
     }
-    const StepConsts c = gated_consts<ARITH>(ga, st, fc.chunk == (int)blockIdx.y);
+    const bool here = fc.chunk == (int)blockIdx.y;
     size_t lo, hi;
     first_call_span(fc, &lo, &hi);
-    adam_tile<ARITH, WD, UNSCALE_RUNTIME>(c, ch, base, chunk_numel, lo, hi);
+    adam_tile_late_consts<ARITH, WD, UNSCALE_RUNTIME>([&]() { return gated_consts<ARITH>(ga, sv, here); }, ch, base,
+                                                      chunk_numel, lo, hi);
 }
 
 // ------------------------------------------------------- tensor-list kernels
@@ -174,7 +199,8 @@ __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
     const ptrdiff_t tile = (ptrdiff_t)blockIdx.x - (head ? 1 : 0);
     const size_t base = tile < 0 ? 0 : (size_t)tile * kTile;
     if (tile >= 0 && base >= numel) return;
-    if (st->overflow) {
+    const StateView sv = view_state(st);
+    if (sv.overflow) {
         if (tile < 0) {
             for (int j = threadIdx.x; j < head; j += kBlock)
                 b.t[k].param_fp16[(ptrdiff_t)j - head] = (uint16_t)float_to_half_bits(b.t[k].param_fp32[(ptrdiff_t)j - head]);
@@ -183,12 +209,12 @@ __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
         }
         return;
     }
-    const StepConsts c = gated_consts<ARITH>(ga, st, first);
     if (tile < 0) {
-        adam_head<ARITH, WD, UNSCALE_RUNTIME>(c, b.t[k], head, first);
+        adam_head<ARITH, WD, UNSCALE_RUNTIME>(gated_consts<ARITH>(ga, sv, first), b.t[k], head, first);
         return;
     }
-    adam_tile<ARITH, WD, UNSCALE_RUNTIME>(c, b.t[k], base, numel, 0, first ? numel : 0);
+    adam_tile_late_consts<ARITH, WD, UNSCALE_RUNTIME>([&]() { return gated_consts<ARITH>(ga, sv, first); }, b.t[k], base,
+                                                      numel, 0, first ? numel : 0);
 }
 
 __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY

@@ -150,13 +150,10 @@ __device__ __forceinline__ void lane_math(const StepConsts& c, float step_size, 
 // (step_size / bc2inv are that call's).  All loads of the tile are issued
 // before the first use.  Loads and stores are written once, outside any
 // branch on the arithmetic variant.
-template <int ARITH, int WD, int UNS>
-__device__ __forceinline__ void adam_tile_vec(const StepConsts& c, float step_size, float bc2inv,
-                                              float* __restrict__ p32, float* __restrict__ m32,
-                                              float* __restrict__ v32, uint16_t* __restrict__ h16,
-                                              size_t base)
+// The loads of one whole, aligned tile: all of them issued back to back, nothing waited for.
+__device__ __forceinline__ void tile_load(LaneTile& r, const float* __restrict__ p32, const float* __restrict__ m32,
+                                          const float* __restrict__ v32, const uint16_t* __restrict__ h16, size_t base)
 {
-    LaneTile r;
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
         size_t i = base + ((size_t)u * kBlock + threadIdx.x) * kLaneElems;
@@ -168,6 +165,14 @@ __device__ __forceinline__ void adam_tile_vec(const StepConsts& c, float step_si
 #pragma unroll
         for (int q = 0; q < kQuads; ++q) r.v[u][q] = ld_f4(v32 + i + 4 * q);
     }
+}
+
+// Arithmetic and stores of a tile whose loads are under way.
+template <int ARITH, int WD, int UNS>
+__device__ __forceinline__ void tile_finish(const StepConsts& c, float step_size, float bc2inv, LaneTile& r,
+                                            float* __restrict__ p32, float* __restrict__ m32,
+                                            float* __restrict__ v32, uint16_t* __restrict__ h16, size_t base)
+{
     if (UNS != UNSCALE_RUNTIME) {
         lane_math<ARITH, WD, UNS>(c, step_size, bc2inv, r);
     } else if (c.unscale == UNSCALE_MUL) {
@@ -188,6 +193,17 @@ __device__ __forceinline__ void adam_tile_vec(const StepConsts& c, float step_si
         for (int q = 0; q < kQuads; ++q) st_f4(v32 + i + 4 * q, r.v[u][q]);
         st_halves(h16 + i, r.h[u]);
     }
+}
+
+template <int ARITH, int WD, int UNS>
+__device__ __forceinline__ void adam_tile_vec(const StepConsts& c, float step_size, float bc2inv,
+                                              float* __restrict__ p32, float* __restrict__ m32,
+                                              float* __restrict__ v32, uint16_t* __restrict__ h16,
+                                              size_t base)
+{
+    LaneTile r;
+    tile_load(r, p32, m32, v32, h16, base);
+    tile_finish<ARITH, WD, UNS>(c, step_size, bc2inv, r, p32, m32, v32, h16, base);
 }
 
 // Same elements, one at a time: ragged tile ends, unaligned bases and tiles that an operator call's
@@ -219,6 +235,30 @@ __device__ __forceinline__ bool aligned16(const void* a, const void* b, const vo
 // first_lo .. first_hi: the elements of THIS chunk that the step's first operator call covers
 // (first_hi <= first_lo: none).  Whole tiles inside or outside that span are uniform and keep the vector
 // path; the at most two tiles that its ends run through go element by element.
+// The same with the step constants still to be formed (a device-decided step builds them from the device-resident
+// state): `make_consts()` is called AFTER the tile's loads have been issued, so that the scalar loads and the
+// divisions and square roots behind the constants run in the shadow of the data loads instead of in front of them.
+template <int ARITH, int WD, int UNS, typename MakeConsts>
+__device__ __forceinline__ void adam_tile_late_consts(MakeConsts make_consts, const ps_chunk& ch, size_t base,
+                                                      size_t chunk_numel, size_t first_lo, size_t first_hi)
+{
+    size_t end = base + kTile;
+    const size_t last = end < chunk_numel ? end : chunk_numel;
+    const bool inside = base >= first_lo && last <= first_hi;
+    const bool cut = !inside && base < first_hi && last > first_lo;
+    if (!cut && end <= chunk_numel && aligned16(ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16)) {
+        LaneTile r;
+        tile_load(r, ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16, base);
+        const StepConsts c = make_consts();
+        tile_finish<ARITH, WD, UNS>(c, inside ? c.first_step_size : c.step_size, inside ? c.first_bc2inv : c.bc2inv, r,
+                                    ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16, base);
+    } else {
+        const StepConsts c = make_consts();
+        adam_tile_scalar<ARITH, WD, UNS>(c, ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16, base, last,
+                                         first_lo, first_hi);
+    }
+}
+
 template <int ARITH, int WD, int UNS>
 __device__ __forceinline__ void adam_tile(const StepConsts& c, const ps_chunk& ch, size_t base,
                                           size_t chunk_numel, size_t first_lo, size_t first_hi)
