@@ -226,11 +226,17 @@ class DynamicLossScaler:
         The sticky flag of the optimizer is left as it was."""
         return DynamicLossScaler._has_inf_or_nan(param.grad)
 
+    _probes = {}  # device -> a scaler kept only for its flag word (one small device state per GPU, made once)
+
     @staticmethod
     def _has_inf_or_nan(x):
         if not x.is_cuda:
             raise RuntimeError("the overflow probe runs on the GPU; got a tensor on " + str(x.device))
-        probe = DynamicLossScaler(init_scale=1)
+        probe = DynamicLossScaler._probes.get(x.device)
+        if probe is None:
+            probe = DynamicLossScaler._probes[x.device] = DynamicLossScaler(init_scale=1).materialize(x.device)
+        off = _lib.ps_step_state.overflow.offset
+        probe._state[off : off + 4].zero_()
         probe.scan(x)
         return probe.overflow_flag
 

@@ -79,7 +79,7 @@ def test_two_calls_in_a_row_match_the_allocating_entry_point():
 def test_limits_and_argument_checks():
     lib = _lib.load()
     flag = torch.zeros(1, dtype=torch.int32, device="cuda")
-    slab, table = _chunks(2, 100, seed=3)
+    slab, table = _chunks(3, 100, seed=3)  # three descriptors: no call below names more chunks than the array holds
     s = _lib.current_stream_handle()
     E = _lib.PS_ERR_BAD_ARG
     assert lib.ps_overflow_scan_chunks_noalloc(table, 2, 100, None, s) == E
