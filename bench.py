@@ -302,6 +302,32 @@ def run_hybrid(args, with_cpu_baseline=True):
     h2d()  # leave finite data in the slot for the kernel leg
     t_kernel = timed(kernels)
     lib.ps_adam_destroy(991)
+
+    # What the link gives when both directions are busy: plain copies of the pipeline's piece sizes, downward on one
+    # stream and upward on another, nothing else running.  A perfectly overlapped pipeline cannot beat link bytes / this.
+    duplex_rate = None
+    if len(host_pos) >= 2:
+        slot_up = [torch.empty_like(t) for t in slot]
+        side = [torch.cuda.Stream(), torch.cuda.Stream()]
+        reps = 6
+        a, b = host_pos[0], host_pos[-1]
+
+        def duplex():
+            for st in side:
+                st.wait_stream(torch.cuda.current_stream())
+            for _ in range(reps):
+                with torch.cuda.stream(side[0]):
+                    for dst, cid in list(zip(slot, (a.fp32, a.exp_avg, a.exp_avg_sq, a.fp16)))[:n_streamed]:
+                        dst.copy_(cl[cid].payload, non_blocking=True)
+                with torch.cuda.stream(side[1]):
+                    for src_, cid in list(zip(slot_up, (b.fp32, b.exp_avg, b.exp_avg_sq, b.fp16)))[:n_streamed]:
+                        cl[cid].payload.copy_(src_, non_blocking=True)
+            for st in side:
+                torch.cuda.current_stream().wait_stream(st)
+
+        duplex()
+        duplex_rate = reps * link_per_element * N / timed(duplex)
+        del slot_up
     del opt, client, params, slot
     torch.cuda.empty_cache()
     bound = max(t_h2d, t_d2h, t_kernel)
@@ -320,6 +346,9 @@ def run_hybrid(args, with_cpu_baseline=True):
         "h2d_GBps": link_bytes / t_h2d / 1e9 if H else None,
         "d2h_GBps": link_bytes / t_d2h / 1e9 if H else None,
         "link_GBps_each_way_during_step": link_bytes / wall / 1e9 if H else None,
+        "link_duplex_GBps_each_way": duplex_rate / 1e9 if duplex_rate else None,
+        "link_duplex_floor_s": link_bytes / duplex_rate if duplex_rate else None,
+        "wall_over_link_duplex_floor": wall * duplex_rate / link_bytes if duplex_rate else None,
         "setup_s": t_setup,
     }
     if with_cpu_baseline and H:
