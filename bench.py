@@ -638,6 +638,31 @@ def ceiling(args):
         if name == "update4":
             results["probe_update4_step_shape"] = entry(measure(lambda: fn(1, 17)), nbytes, reads, writes, tiles_per_workgroup=1, lds_kb=17,
                                                         resident_workgroups_per_cu=9)
+    # Is the limit the DRAM or the path to it?  (1) The pure-read kernel over a window small enough to stay in the
+    # memory-side cache (256 MiB on this GPU), launched again and again: data that never leaves the chip.  (2) A window
+    # read once (so that it sits in that cache) and then copied, window after window over the whole list, against plain
+    # copies of the same windows: would keeping a step's DRAM reads and DRAM writes apart in time pay?
+    windows = {}
+    ru, rl = results["probe_read"]["tiles_per_workgroup"], results["probe_read"]["lds_kb"]
+    for mib in (64, 128, 256, 1024):
+        k = mib * (1 << 18)
+        if k > n or k % (256 * 8):
+            continue
+        e = {"reread_GBps": 4 * k / (measure(lambda: probe.ps_probe_read(p.data_ptr(), k, sink.data_ptr(), ru, rl, s())) * 1e-3) / 1e9}
+        n_win = min(n // k, (1 << 30) // k) or 1  # over 4 GiB of the list
+
+        def plain_copies():
+            for i in range(n_win):
+                probe.ps_probe_copy(p.data_ptr() + 4 * i * k, m.data_ptr() + 4 * i * k, k, 1, 0, s())
+
+        def read_then_copy():
+            for i in range(n_win):
+                probe.ps_probe_read(p.data_ptr() + 4 * i * k, k, sink.data_ptr(), ru, rl, s())
+                probe.ps_probe_copy(p.data_ptr() + 4 * i * k, m.data_ptr() + 4 * i * k, k, 1, 0, s())
+
+        e["plain_copy_GBps"] = 8 * k * n_win / (measure(plain_copies) * 1e-3) / 1e9
+        e["read_then_copy_GBps"] = 8 * k * n_win / (measure(read_then_copy) * 1e-3) / 1e9
+        windows[f"{mib}MiB"] = {key: round(val, 1) for key, val in e.items()}
     # the probe kernels have rewritten the lists: refill what the optimizer kernels need to stay finite
     m.normal_(0, 1e-4)
     v.normal_(0, 1e-6).abs_()
@@ -661,9 +686,12 @@ def ceiling(args):
         "kernels": results,
         "time_sliced_bound_GBps": 28.0 / (14.0 / r + 14.0 / w),
         "sweeps_GBps": sweeps,
+        "windows": windows,
         "note": "probe_*: best launch shape of the sweep (sweeps_GBps holds every shape); time_sliced_bound: 14 B/element read at the "
         "pure-read rate plus 14 B/element written at the pure-write rate, as if reads and writes never met on the memory bus; "
-        "probe_update4 is the step's access pattern without its arithmetic",
+        "probe_update4 is the step's access pattern without its arithmetic; windows: reread = the pure-read kernel launched repeatedly "
+        "over one window of that size (a window of up to 256 MiB stays in the memory-side cache), plain_copy / read_then_copy = 4 GiB "
+        "copied window by window, without and with a pure-read pass over each window just before its copy (GB/s of the copy's bytes)",
     }
     print(json.dumps(out))
 
