@@ -267,7 +267,11 @@ int ps_restore_fp16_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_nu
  *                ps_adam_step_chunks_gated (step, betas and loss_scale ignored)
  * Work queued on `stream` before the call is waited for; work queued on it
  * afterwards waits for the last write-back.  The call itself never blocks.
- * Calls that overlap in time on one device share the side streams and race. */
+ * Calls on one device (from several host threads, on several streams) take turns: a per-device
+ * lock is held while a call queues its work, and the streamed part of a later call is ordered
+ * behind everything an earlier call left on the side streams, so concurrent callers get correct
+ * results but their copies do not overlap one another's.  The same holds between this entry
+ * point and ps_overflow_scan_host_chunks. */
 int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, double beta2,
                         double epsilon, double weight_decay, int bias_correction,
                         const ps_chunk* chunks, int n_chunks, const ps_chunk* host_chunks,

@@ -42,8 +42,10 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <exception>
 #include <memory>
 #include <mutex>
+#include <new>
 #include <unordered_map>
 #include <vector>
 
@@ -391,6 +393,7 @@ constexpr int kMaxSlots = 8;
 
 struct Pipeline {
     bool ready = false;
+    std::mutex in_use;  // held by a call while it queues work on the side streams: calls on one device take turns
     hipStream_t h2d = nullptr, compute = nullptr, d2h = nullptr;
     hipEvent_t entry = nullptr;
     hipEvent_t joined[3] = {};  // one per side stream: "everything queued there so far"
@@ -426,6 +429,24 @@ struct Pipeline {
         for (int i = 0; i < kMaxSlots; ++i) drop(h2d_done[i]), drop(compute_done[i]), drop(d2h_done[i]);
     }
 
+    // A call begins: the copies and kernels it is about to queue on the side streams come after everything `caller`
+    // has queued so far (gradients written, the device flag set) and after whatever an EARLIER call, possibly of
+    // another host thread on another stream, left on any side stream (its staging slots may be the same memory).  For
+    // one caller the second part is implied by the first (every call ends with join()).
+    int begin(hipStream_t caller)
+    {
+        hipStream_t side[3] = {h2d, compute, d2h};
+        for (int i = 0; i < 3; ++i) PS_HIP(hipEventRecord(joined[i], side[i]));
+        PS_HIP(hipEventRecord(entry, caller));
+        for (hipStream_t st : {h2d, compute}) {
+            PS_HIP(hipStreamWaitEvent(st, entry, 0));
+            for (int i = 0; i < 3; ++i)
+                if (side[i] != st) PS_HIP(hipStreamWaitEvent(st, joined[i], 0));
+        }
+        for (int i = 0; i < kMaxSlots; ++i) slot_used[i] = false;
+        return 0;
+    }
+
     // Later work on `caller` comes after everything queued on the side streams so far.  Also used on
     // an error path, so that a half-queued step cannot race with whatever the caller does next.
     int join(hipStream_t caller)
@@ -447,15 +468,20 @@ int get_pipeline(Pipeline** out)
     int dev = 0;
     PS_HIP(hipGetDevice(&dev));
     std::lock_guard<std::mutex> lock(g_pipeline_mutex);
-    Pipeline& p = g_pipelines[dev];
-    if (!p.ready) {
-        if (int rc = p.create()) {
-            p.destroy();
+    Pipeline* p = nullptr;
+    try {
+        p = &g_pipelines[dev];
+    } catch (const std::exception&) {  // nothing may throw across the boundary
+        return fail(PS_ERR_BAD_ARG, "no host memory for the streaming state of device %d", dev);
+    }
+    if (!p->ready) {
+        if (int rc = p->create()) {
+            p->destroy();
             return rc;
         }
-        p.ready = true;
+        p->ready = true;
     }
-    *out = &p;
+    *out = p;
     return 0;
 }
 
@@ -538,16 +564,18 @@ const char* ps_last_error(void) { return g_err; }
 int ps_adam_create(int optimizer_id, float alpha, float beta1, float beta2, float eps,
                    float weight_decay, int adamw_mode, int should_log)
 {
-    auto o = std::make_shared<HostAdam>();
-    o->alpha = alpha;
-    o->beta1 = beta1;
-    o->beta2 = beta2;
-    o->eps = eps;
-    o->weight_decay = weight_decay;
-    o->adamw = adamw_mode != 0;
-    {
+    try {
+        auto o = std::make_shared<HostAdam>();
+        o->alpha = alpha;
+        o->beta1 = beta1;
+        o->beta2 = beta2;
+        o->eps = eps;
+        o->weight_decay = weight_decay;
+        o->adamw = adamw_mode != 0;
         std::lock_guard<std::mutex> lock(g_registry_mutex);
         g_registry[optimizer_id] = o;
+    } catch (const std::exception&) {  // nothing may throw across the boundary
+        return fail(PS_ERR_BAD_ARG, "no host memory for optimizer %d", optimizer_id);
     }
     if (should_log) {
         printf("Adam Optimizer #%d is created with gfx950 HIP arithmetic capability.\n",
@@ -833,7 +861,8 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, 
     ChunkList resident, host;
     if (int rc = make_chunk_list(resident, chunks, n_chunks, chunk_numel, kTile)) return rc;
     if (int rc = make_chunk_list(host, host_chunks, n_host_chunks, chunk_numel, kTile, false, "host chunk")) return rc;
-    std::unique_ptr<bool[]> fp16_in_hbm(new bool[n_host_chunks > 0 ? n_host_chunks : 1]);
+    std::unique_ptr<bool[]> fp16_in_hbm(new (std::nothrow) bool[n_host_chunks > 0 ? n_host_chunks : 1]);
+    if (!fp16_in_hbm) return fail(PS_ERR_BAD_ARG, "no host memory for a list of %d host chunks", n_host_chunks);
     if (n_host_chunks > 0) {
         if (int rc = check_slots(staging, n_slots, true, false)) return rc;
         bool any_on_host = false;
@@ -860,13 +889,12 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, 
     hipStream_t caller = static_cast<hipStream_t>(stream);
     const bool stream_host = n_host_chunks > 0 && chunk_numel > 0;
     Pipeline* p = nullptr;
+    std::unique_lock<std::mutex> turn;
     if (stream_host) {
         if (int rc = get_pipeline(&p)) return rc;
-        // Everything the caller queued so far (gradients written, the device flag set) comes
-        // first; the resident chunks' kernels, queued next, do NOT hold the copies back.
-        PS_HIP(hipEventRecord(p->entry, caller));
-        PS_HIP(hipStreamWaitEvent(p->h2d, p->entry, 0));
-        PS_HIP(hipStreamWaitEvent(p->compute, p->entry, 0));
+        turn = std::unique_lock<std::mutex>(p->in_use);
+        // the resident chunks' kernels, queued next on the caller's stream, do NOT hold the copies back
+        if (int rc = p->begin(caller)) return rc;
     }
     int rc = for_each_batch(resident, [&](const ChunkBatch& b, dim3 grid, int first) {
         const FirstCall fc = k.in_batch(first, (int)grid.y);
@@ -879,7 +907,6 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, 
     if (!stream_host) return 0;
 
     const size_t b32 = chunk_numel * sizeof(float), b16 = chunk_numel * sizeof(uint16_t);
-    for (int i = 0; i < kMaxSlots; ++i) p->slot_used[i] = false;
     auto stream_chunk = [&](int k_host) -> int {
         const int s = k_host % n_slots;
         const ps_chunk& h = host_chunks[k_host];
@@ -936,7 +963,8 @@ int ps_overflow_scan_host_chunks(const ps_chunk* host_chunks, int n_chunks, size
     ChunkList a;
     if (int rc = make_chunk_list(a, host_chunks, n_chunks, chunk_numel, kScanTile, true, "host chunk")) return rc;
     if (n_chunks == 0 || chunk_numel == 0) return 0;
-    std::unique_ptr<bool[]> fp16_in_hbm(new bool[n_chunks]);
+    std::unique_ptr<bool[]> fp16_in_hbm(new (std::nothrow) bool[n_chunks]);
+    if (!fp16_in_hbm) return fail(PS_ERR_BAD_ARG, "no host memory for a list of %d host chunks", n_chunks);
     bool any_on_host = false;
     if (int rc = fp16_payloads_in_hbm(host_chunks, n_chunks, fp16_in_hbm.get(), &any_on_host)) return rc;
     hipStream_t caller = static_cast<hipStream_t>(stream);
@@ -953,10 +981,8 @@ int ps_overflow_scan_host_chunks(const ps_chunk* host_chunks, int n_chunks, size
     if (int rc = check_slots(staging, n_slots, false, true)) return rc;
     Pipeline* p = nullptr;
     if (int rc = get_pipeline(&p)) return rc;
-    PS_HIP(hipEventRecord(p->entry, caller));
-    PS_HIP(hipStreamWaitEvent(p->h2d, p->entry, 0));
-    PS_HIP(hipStreamWaitEvent(p->compute, p->entry, 0));
-    for (int i = 0; i < kMaxSlots; ++i) p->slot_used[i] = false;
+    std::lock_guard<std::mutex> turn(p->in_use);
+    if (int rc = p->begin(caller)) return rc;
     int streamed = 0;
     auto stream_chunk = [&](int k) -> int {
         const int s = streamed++ % n_slots;

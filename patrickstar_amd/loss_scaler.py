@@ -50,8 +50,11 @@ class DynamicLossScaler:
 
     Number semantics follow Python's, as in the reference: ``loss_scale`` is an
     ``int`` until the first halving (a true division) and the ``min_scale``
-    object's own type when the clamp bites.  Scales beyond 2**53 are not
-    representable exactly (the device keeps a binary64).
+    object's own type when the clamp bites.  The device keeps the scale as a
+    binary64: an ``int`` argument that a binary64 cannot hold exactly (beyond
+    2**53 only powers of two times a 53-bit integer can) is refused here
+    instead of being rounded silently; an ``int`` scale that GROWS past 2**53
+    by a factor that is not a power of two is rounded like a float from there on.
     """
 
     def __init__(
@@ -71,6 +74,14 @@ class DynamicLossScaler:
             delayed_shift=delayed_shift,
             consecutive_hysteresis=consecutive_hysteresis,
         )
+        for name, x in (("init_scale", init_scale), ("scale_factor", scale_factor), ("min_scale", min_scale)):
+            if _is_int(x):
+                try:
+                    exact = int(float(x)) == x
+                except OverflowError:
+                    exact = False
+                if not exact:
+                    raise ValueError(f"{name} = {x} is an int that a binary64 cannot hold exactly; pass a representable value")
         self.scale_factor = scale_factor
         self.scale_window = scale_window
         self.min_scale = min_scale

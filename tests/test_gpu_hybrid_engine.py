@@ -507,3 +507,63 @@ def test_engine_refuses_host_placement_without_hybrid_adam():
     config["client"] = {"hbm_budget_bytes": 10**9}
     engine, optimizer = ps.initialize_engine(model_func=_Deep, local_rank=0, config=config)
     assert not any(q.on_host for q in engine.client.positions())
+
+
+def test_two_host_threads_stream_host_chunks_on_one_gpu_at_the_same_time():
+    """Two optimizers with host-resident positions, stepped by two host threads on two streams of the same GPU at the
+    same moment (a barrier in front of every step; ctypes drops the GIL inside the call).  Both use the library's
+    one set of side streams for that GPU: the calls take turns there, and both must match the oracle bit for bit."""
+    import threading
+
+    n, steps = 256 * 1024 + 77, 4
+    cases = [
+        dict(host=[1, 2, 4], keeps=True, scaler=lambda: ps.LossScaler(2**10), oscaler=lambda: oracle.StaticScalerOracle(2**10),
+             kw=dict(lr=1e-3, weight_decay=0.01, use_adamw=True)),
+        dict(host=[0, 3], keeps=False, scaler=lambda: ps.DynamicLossScaler(init_scale=2**8, scale_factor=2, scale_window=2),
+             oscaler=lambda: oracle.ScalerOracle(init_scale=2**8, scale_factor=2, scale_window=2), kw=dict(lr=1e-4, weight_decay=0.0)),
+    ]
+    hs = [HybridHarness(5, n, c["host"], c["scaler"](), seed=31 + i, host_keeps_fp16=c["keeps"], **c["kw"]) for i, c in enumerate(cases)]
+    for h in hs:
+        h.opt.staging_slots = 2
+        h.fill_state()
+    start = [h.oracle_chunks() for h in hs]
+    grads = [[] for _ in hs]  # per harness, per step: the fp16 payloads as the step found them
+    barrier = threading.Barrier(2)
+    errors = []
+
+    def worker(t):
+        try:
+            h, stream = hs[t], torch.cuda.Stream()
+            scale = 2.0**10 if t == 0 else 2.0**8
+            for step in range(steps):
+                with torch.cuda.stream(stream):
+                    h.fill_grads(1e-3, scale)
+                    if t == 1 and step == 1:
+                        h.payloads(3)[3][n - 1] = float("inf")  # last element of a host position's fp16 payload
+                    grads[t].append([h.download(i)[3] for i in range(5)])
+                    barrier.wait(timeout=60)
+                    h.opt.step()
+            stream.synchronize()
+        except Exception as e:  # surfaced by the main thread
+            errors.append((t, repr(e)))
+            barrier.abort()
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(2)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
+    torch.cuda.synchronize()
+    for t, (h, c) in enumerate(zip(hs, cases)):
+        oc = start[t]
+        oscaler = c["oscaler"]()
+        oopt = oracle.OptimizerStepOracle(oc, oscaler, **c["kw"])
+        for step in range(steps):
+            for i, ch in enumerate(oc):
+                ch["p16"][...] = grads[t][step][i]
+            oopt.check_overflow()
+            assert oopt.step() == (t == 1 and step == 1)
+        h.compare(oc, what=f"thread {t}")
+        if t == 1:
+            assert h.opt.loss_scaler.loss_scale == oscaler.loss_scale and h.opt.loss_scaler.cur_iter == steps

@@ -71,6 +71,10 @@ CASES = [
     dict(init_scale=16, scale_factor=2.0, scale_window=5, delayed_shift=3, consecutive_hysteresis=True),
     dict(init_scale=1000.0, scale_factor=3, scale_window=2),
     dict(init_scale=2**32, scale_factor=2.0, scale_window=7, min_scale=0.5),
+    # beyond 2**53: powers of two stay exact in the device's binary64, as ints (2**60 -> 2**120) and as floats
+    dict(init_scale=2**60, scale_factor=2, scale_window=2, min_scale=2**55),
+    dict(init_scale=2**100, scale_factor=2.0, scale_window=3),
+    dict(init_scale=3 * 2**70, scale_factor=4, scale_window=2, min_scale=3 * 2**60),
 ]
 
 

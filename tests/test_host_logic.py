@@ -213,6 +213,16 @@ def test_dynamic_scaler_needs_a_gpu_for_anything_but_its_configuration():
             s.update_scale(True)
 
 
+def test_dynamic_scaler_refuses_int_scales_a_binary64_cannot_hold():
+    # the device keeps the scale as a binary64; Python ints are exact at any size, so an int that would be rounded on
+    # its way to the device is refused rather than changed silently
+    for bad in (dict(init_scale=2**53 + 1), dict(min_scale=2**60 + 2**5), dict(scale_factor=2**53 + 1), dict(init_scale=2**2000)):
+        with pytest.raises(ValueError, match="binary64"):
+            ps.DynamicLossScaler(**bad)
+    for good in (dict(init_scale=2**53), dict(init_scale=2**200), dict(init_scale=3 * 2**70, min_scale=5 * 2**60), dict(init_scale=2.0**60 + 1.0)):
+        assert ps.DynamicLossScaler(**good).loss_scale == good["init_scale"]
+
+
 def test_bench_refuses_more_than_one_gpu():
     import subprocess
     import sys
