@@ -334,8 +334,9 @@ int ps_overflow_scan_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_n
  * caller's (device-accessible, 4-byte aligned), set to 1 if any fp16 payload holds an inf / nan and
  * left alone otherwise (sticky, like ps_step_state::overflow).  The probe runs without atomics: every
  * workgroup leaves its partial result in a word of a file-scope device array inside the library
- * (4 MiB per GPU, resolved with hipGetSymbolAddress at the first call on a device), and a second kernel
- * reduces those words.  The call allocates and frees nothing.
+ * (4 MiB per GPU, resolved with hipGetSymbolAddress at the first call on a device: make that call
+ * outside a stream capture), and a second kernel reduces those words.  The call allocates and frees
+ * nothing and records kernel launches only (no memset), so it can be captured into a HIP graph.
  *   limit   n_chunks * ceil(chunk_numel / 8192) <= 1,048,576 scratch words, i.e. at most 8 Gi elements
  *           per call; more is rejected with PS_ERR_BAD_ARG before anything is queued
  *   sharing every call on one GPU uses that GPU's one scratch array: calls that overlap in time on

@@ -108,3 +108,29 @@ def test_full_size_probe_matches_the_atomic_form():
     slab[17 * n + 12345] = float("nan")
     _noalloc(table, c, n, flag)
     assert int(flag.item()) == _existing(table, c, n) == 1
+
+
+def test_probe_replays_from_a_hip_graph():
+    """What the entry point is for: a caller under stream capture.  The two launches are captured once (after one
+    eager call, which resolves the scratch array's address on this GPU) and replayed over changing data, with eager
+    work and synchronisation between the replays; every replay must give the allocating entry point's answer."""
+    n, c = 8192 * 3 + 5, 66  # two launches of the first kernel
+    slab, table = _chunks(c, n, seed=5)
+    flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+    _noalloc(table, c, n, flag)  # eager
+    assert int(flag.item()) == 0
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _noalloc(table, c, n, flag)
+    clean = slab.clone()
+    for it, (chunk, pos, val) in enumerate([(None, 0, 0.0), (65, n - 1, float("inf")), (None, 0, 0.0), (0, 0, float("nan")),
+                                            (33, 8192, float("-inf")), (None, 0, 0.0)]):
+        slab.copy_(clean)
+        if chunk is not None:
+            slab[chunk * (n + 8) + pos] = val
+        flag.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = _existing(table, c, n)
+        assert want == (chunk is not None)
+        assert int(flag.item()) == want, (it, chunk, pos, val)
