@@ -554,7 +554,7 @@ def tensor_list_leg(cfg, steps, warmup):
     def step():
         t[0] += 1
         _lib.check(lib.ps_adam_step_tensors(993, t[0], HYPER["lr"], 0.9, 0.999, HYPER["eps"], HYPER["weight_decay"], 1, table, numels,
-                                            len(sizes), 4096.0, None, _lib.current_stream_handle()), "ps_adam_step_tensors")
+                                            len(sizes), None, 4096.0, None, _lib.current_stream_handle()), "ps_adam_step_tensors")
 
     ms, kernel_ms = time_steps(torch, step, steps, warmup)
     lib.ps_adam_destroy(993)

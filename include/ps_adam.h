@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define PS_ABI_VERSION 3
+#define PS_ABI_VERSION 4
 
 #define PS_ERR_BAD_ARG (-10001)     /* null pointer, negative count, unknown mode */
 #define PS_ERR_UNKNOWN_ID (-10002)  /* optimizer id was never created (the reference dereferences null here) */
@@ -115,6 +115,11 @@ typedef struct ps_step_state {
  * (float)pow(beta, t).  The two differ in the last bits (1 / sqrt(1 - beta2^t) by up to 1e-5
  * relative at small t), so a fused pass over whole chunks has to know which elements the first call
  * covered.  Only the operator's arithmetic looks at this; the torch formula has no such state.
+ *
+ * One step may be spread over several calls of the step entry points (say ps_adam_step_tensors for
+ * chunks that hold frozen parameters and ps_adam_step_hybrid for the rest): every call is given the
+ * n_calls of the WHOLE step; the call whose list holds the first operator call's tensor is made first and
+ * names it; every other call passes first_numel = 0.  ps_scaler_update follows the last of them, once.
  */
 typedef struct ps_call_pattern {
     int64_t n_calls;       /* operator calls of the step over this list = its trainable tensors (>= 1) */
@@ -225,15 +230,21 @@ int ps_adam_step_chunks_gated(int optimizer_id, double lr, double epsilon, doubl
  *               (gradient in, fp16 parameter out), numels[i] elements each; both are host arrays
  *   d_state     NULL: host-decided step with loss_scale; else device-gated like ps_adam_step_chunks_gated
  *               (step, betas and loss_scale ignored; a flagged step restores the fp16 slots from fp32)
+ *   calls       NULL: the list is the whole step, n_tensors operator calls, tensors[0] the first.  Else
+ *               n_calls = the operator calls of the whole step (some of them may be made through other
+ *               entry points, see ps_call_pattern) and first_chunk = the index in tensors[] of the
+ *               step's first call, with first_offset = 0 and first_numel = numels[first_chunk]
+ *               (a tensor is one call); first_numel = 0: the first call is not in this list
  * Same arithmetic, clamp and 28 B/element as the chunk-list form.  Every tensor is one operator call of the
- * reference's loop, tensors[0] the first of the step (zero-length tensors included: the reference calls the
- * operator for them too); follow a device-gated call with ps_scaler_update(..., n_tensors).
+ * reference's loop (zero-length tensors included: the reference calls the operator for them too); follow a
+ * device-gated call with ps_scaler_update(..., the step's number of calls).
  * Tensors of (nearly) equal length share a launch, up to 64 of them; the order of the list decides nothing
- * but which tensor is the first call. */
+ * but, without a pattern, which tensor is the first call. */
 int ps_adam_step_tensors(int optimizer_id, size_t step, double lr, double beta1, double beta2,
                          double epsilon, double weight_decay, int bias_correction,
                          const ps_chunk* tensors, const size_t* numels, int n_tensors,
-                         double loss_scale, const ps_step_state* d_state, ps_stream_t stream);
+                         const ps_call_pattern* calls, double loss_scale, const ps_step_state* d_state,
+                         ps_stream_t stream);
 
 /* Unconditional restore p16 = RNE(p32) of a chunk list (FP16ChunkWriteBuffer,
  * chunk_io_buff.py:85-151), or only when d_state->overflow is set if d_state != NULL. */

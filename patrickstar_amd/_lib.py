@@ -11,7 +11,7 @@ LIB_PATH = os.path.join(PKG_DIR, "libps_adam.so")
 PS_FLAG_FALSE, PS_FLAG_TRUE, PS_FLAG_FROM_DEVICE = 0, 1, 2
 PS_ERR_BAD_ARG, PS_ERR_UNKNOWN_ID, PS_ERR_NO_DEVICE = -10001, -10002, -10003
 PS_ARITH_OPERATOR, PS_ARITH_TORCH = 0, 1
-PS_ABI_VERSION = 3
+PS_ABI_VERSION = 4
 
 
 class ps_chunk(ctypes.Structure):
@@ -101,7 +101,7 @@ SIGNATURES = {
     "ps_adam_update": (_i, [_i, _sz, _f, _f, _f, _f, _f, _i, _vp, _vp, _i, _vp, _vp, _sz, _f, _vp, _vp]),
     "ps_adam_step_chunks": (_i, [_i, _sz, _d, _d, _d, _d, _d, _i, _vp, _i, _sz, _vp, _d, _vp]),
     "ps_adam_step_chunks_gated": (_i, [_i, _d, _d, _d, _i, _vp, _i, _sz, _vp, _vp, _vp]),
-    "ps_adam_step_tensors": (_i, [_i, _sz, _d, _d, _d, _d, _d, _i, _vp, _vp, _i, _d, _vp, _vp]),
+    "ps_adam_step_tensors": (_i, [_i, _sz, _d, _d, _d, _d, _d, _i, _vp, _vp, _i, _vp, _d, _vp, _vp]),
     "ps_adam_step_hybrid": (_i, [_i, _sz, _d, _d, _d, _d, _d, _i, _vp, _i, _vp, _i, _sz, _vp, _i, _vp, _d, _vp, _vp]),
     "ps_overflow_scan_host_chunks": (_i, [_vp, _i, _sz, _vp, _i, _vp, _vp]),
     "ps_restore_fp16_chunks": (_i, [_vp, _i, _sz, _vp, _vp]),

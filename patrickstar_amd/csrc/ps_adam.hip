@@ -741,7 +741,8 @@ int ps_adam_step_chunks_gated(int optimizer_id, double lr, double epsilon, doubl
 int ps_adam_step_tensors(int optimizer_id, size_t step, double lr, double beta1, double beta2,
                          double epsilon, double weight_decay, int bias_correction,
                          const ps_chunk* tensors, const size_t* numels, int n_tensors,
-                         double loss_scale, const ps_step_state* d_state, ps_stream_t stream)
+                         const ps_call_pattern* calls, double loss_scale, const ps_step_state* d_state,
+                         ps_stream_t stream)
 {
     auto o = find_opt(optimizer_id);
     if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
@@ -755,12 +756,30 @@ int ps_adam_step_tensors(int optimizer_id, size_t step, double lr, double beta1,
             return fail(PS_ERR_BAD_ARG, "tensor %d: numel = %zu is beyond the launch grid", i, numels[i]);
     }
     const int arith = o->arith;
-    // one operator call per tensor, tensors[0] the first of the step
+    // One operator call per tensor.  Without a pattern the list is the whole step and tensors[0] its first call;
+    // a pattern says how many calls the step has in all and which tensor of THIS list, if any, is the first.
+    int64_t n_calls = n_tensors;
+    int first_tensor = 0;
+    if (calls != nullptr) {
+        if (calls->n_calls < 1)
+            return fail(PS_ERR_BAD_ARG, "calls->n_calls = %lld must be at least 1", (long long)calls->n_calls);
+        n_calls = calls->n_calls;
+        first_tensor = -1;
+        if (calls->first_numel != 0) {
+            if (calls->first_chunk < 0 || calls->first_chunk >= n_tensors)
+                return fail(PS_ERR_BAD_ARG, "calls->first_chunk = %lld is outside the list of %d tensors",
+                            (long long)calls->first_chunk, n_tensors);
+            if (calls->first_offset != 0 || calls->first_numel != numels[calls->first_chunk])
+                return fail(PS_ERR_BAD_ARG, "the first call is a whole tensor: calls->first_offset must be 0 and "
+                            "calls->first_numel the length of tensor %lld", (long long)calls->first_chunk);
+            first_tensor = (int)calls->first_chunk;
+        }
+    }
     StepConsts c;
-    GatedArgs ga = gated_args(*o, lr, epsilon, weight_decay, bias_correction, n_tensors);
+    GatedArgs ga = gated_args(*o, lr, epsilon, weight_decay, bias_correction, n_calls);
     if (d_state == nullptr && n_tensors > 0) {
         const HyperParams hp{lr, beta1, beta2, epsilon, weight_decay, loss_scale, bias_correction != 0};
-        c = arith == PS_ARITH_TORCH ? torch_step_consts(*o, step, hp) : operator_step_consts(*o, step, hp, n_tensors);
+        c = arith == PS_ARITH_TORCH ? torch_step_consts(*o, step, hp) : operator_step_consts(*o, step, hp, n_calls);
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
     // Where each tensor's tile grid starts (the fp32 parameter's first 1 KiB boundary; what lies in front of it is a
@@ -806,7 +825,7 @@ int ps_adam_step_tensors(int optimizer_id, size_t step, double lr, double beta1,
             t.param_fp16 += it.head;
             b.t[in_batch] = t;
             b.numel_head[in_batch] = (uint64_t)it.body | ((uint64_t)it.head << 56);
-            if (it.index == 0 && arith == PS_ARITH_OPERATOR) b.first_call = in_batch;
+            if (it.index == first_tensor && arith == PS_ARITH_OPERATOR) b.first_call = in_batch;
             in_batch += 1;
             next += 1;
         }

@@ -160,6 +160,7 @@ class FP16Adam(torch.optim.Optimizer):
         self._tables = None
         self._tensor_table = None  # (ps_chunk rows, numels, count) when the step has to go tensor by tensor
         self._calls = None  # ps_call_pattern of one step (None: no operator call at all)
+        self._stages = None  # the entry-point calls of a step that cannot be made as one (see _plan_stages)
         self._operator_calls = 0
         if self._dynamic and torch.cuda.is_available():
             self.loss_scaler.materialize(self.client.device, betas=betas)
@@ -218,22 +219,8 @@ class FP16Adam(torch.optim.Optimizer):
                     ]
                 )
         self._tensor_table = None
-        if partly_frozen:
-            if host_positions:
-                raise NotImplementedError(
-                    "chunks that mix trainable and frozen parameters cannot be combined with host-resident positions"
-                )
-            rows, numels = [], []
-            for p in trainable:
-                st = self.state[p]
-                views = [
-                    self.client.access_data(q)
-                    for q in (self.client.param_fp16_to_param_fp32_map[p], dict.__getitem__(st, "exp_avg"),
-                              dict.__getitem__(st, "exp_avg_sq"), p)
-                ]
-                rows.append([v.data_ptr() for v in views])
-                numels.append(p.ps_attr.numel)
-            self._tensor_table = (_lib.chunk_array(rows), (ctypes.c_size_t * len(numels))(*numels), len(numels))
+        if partly_frozen and not host_positions:
+            self._tensor_table = self._tensor_rows(trainable)
         # The operator calls of one step: with the operator's arithmetic every trainable tensor is one, with the torch
         # arithmetic only those whose optimizer state lives in host memory (fp16_cpu_adam.py:415-443).
         if self.arithmetic == "torch":
@@ -251,11 +238,131 @@ class FP16Adam(torch.optim.Optimizer):
             )
         table = _lib.chunk_array(dev_rows) if dev_rows else None
         self._tables = (table, len(dev_rows), host_positions)
+        self._stages = None
         if host_positions:
             from .hybrid import HostChunkStreamer
 
-            self._streamer = HostChunkStreamer(self.client, host_positions, n_slots=self.staging_slots)
+            if partly_frozen:
+                self._plan_stages(trainable, chunk_of, where, host_positions, called, live_ids)
+            else:
+                self._streamer = HostChunkStreamer(self.client, host_positions, n_slots=self.staging_slots)
         return self._tables
+
+    def _tensor_rows(self, params, slot=None):
+        """(ps_chunk rows, numels, count) of a tensor list for ``ps_adam_step_tensors``: the four addresses of every
+        parameter's fp32 master, exp_avg, exp_avg_sq and fp16 slot.  ``slot``: (payloads of the parameters' chunk
+        position, staging tensors) when the step works on a staged copy of a host-resident position: addresses are then
+        taken at the tensors' offsets inside the staging tensors (inside the real fp16 payload if that one lives in HBM)."""
+        index = self.client.chunk_tensor_index
+        rows, numels = [], []
+        for p in params:
+            st = self.state[p]
+            quad = (self.client.param_fp16_to_param_fp32_map[p], dict.__getitem__(st, "exp_avg"),
+                    dict.__getitem__(st, "exp_avg_sq"), p)
+            if slot is None:
+                rows.append([self.client.access_data(q).data_ptr() for q in quad])
+            else:
+                payloads, staging = slot
+                row = []
+                for k, q in enumerate(quad):
+                    base = staging[k] if payloads[k].device.type == "cpu" else payloads[k]
+                    row.append(base.data_ptr() + index.get_tensor_info(q.ps_attr.data_id()).start_offset * base.element_size())
+                rows.append(row)
+            numels.append(p.ps_attr.numel)
+        return _lib.chunk_array(rows), (ctypes.c_size_t * len(numels))(*numels), len(numels)
+
+    def _plan_stages(self, trainable, chunk_of, where, host_positions, called, live_ids):
+        """Chunks that mix trainable and frozen tensors TOGETHER WITH host-resident positions: the step is spread over
+        several entry-point calls, all under one call pattern (the stage that holds the step's first operator call
+        goes first and names it):
+          * the trainable tensors of HBM-resident chunks: one tensor-list call;
+          * host-resident positions whose tensors are all trainable: streamed as whole chunks;
+          * host-resident positions that hold frozen tensors too: copied into a staging slot, their trainable tensors
+            updated there by a tensor-list call with the operator's arithmetic, and copied back, on the caller's stream.
+        """
+        from .hybrid import HostChunkStreamer
+
+        cl, index = self.client.chunk_list, self.client.chunk_tensor_index
+        whole, part = [], []
+        for k, pos in enumerate(host_positions):
+            frozen_here = any(info.tensor_id not in live_ids for info in index.generate_tensor_info_in_order(pos.fp16))
+            (part if frozen_here else whole).append(k)
+        self._streamer = HostChunkStreamer(self.client, host_positions, n_slots=self.staging_slots, step_indices=whole)
+        n_calls = len(called)
+        first = called[0] if called else None
+        first_info = index.get_tensor_info(first.ps_attr.data_id()) if first is not None else None
+
+        def pattern():
+            """For a stage that does not hold the step's first operator call."""
+            return _lib.call_pattern(n_calls, 0, 0, 0) if n_calls else None
+
+        def position_of(params, wanted):
+            for i, q in enumerate(params):
+                if q is wanted:
+                    return i
+            return None
+
+        stages = []  # (holds the first call, stage)
+        resident = [p for p in trainable if where[chunk_of[p]][0] == "hbm"]
+        if resident:
+            i = position_of(resident, first)
+            pat = pattern() if i is None else _lib.call_pattern(n_calls, i, 0, first.ps_attr.numel)
+            stages.append((i is not None, ("tensors", self._tensor_rows(resident), pat)))
+        if whole:
+            i = None
+            if first is not None and where[first_info.chunk_id][0] == "host" and where[first_info.chunk_id][1] in whole:
+                i = whole.index(where[first_info.chunk_id][1])
+            pat = pattern() if i is None else _lib.call_pattern(n_calls, i, first_info.start_offset, first_info.numel)
+            stages.append((i is not None, ("stream", pat)))
+        for k in part:
+            pos = host_positions[k]
+            here = [p for p in trainable if chunk_of[p] == pos.fp16]
+            payloads = [cl[c].payload for c in (pos.fp32, pos.exp_avg, pos.exp_avg_sq, pos.fp16)]
+            staging = self._streamer._slots[0]
+            i = position_of(here, first)
+            pat = pattern() if i is None else _lib.call_pattern(n_calls, i, 0, first.ps_attr.numel)
+            stages.append((i is not None, ("staged", payloads, staging, self._tensor_rows(here, (payloads, staging)), pat)))
+        stages.sort(key=lambda e: not e[0])  # stable: the stage with the first call moves to the front
+        self._stages = [stage for _, stage in stages]
+
+    def _run_stages(self, step_no, hyper, loss_scale, scaler, stream):
+        """Queue the stages of a step that is spread over several entry-point calls (see ``_plan_stages``).
+        ``scaler``: the device-resident scaler of a device-decided step, else None."""
+        lr, (beta1, beta2), eps, weight_decay = hyper
+        state_ptr = scaler.state_ptr if scaler is not None else None
+
+        def tensors(table, pat):
+            rows, numels, n = table
+            _lib.check(
+                self._lib.ps_adam_step_tensors(
+                    self.opt_id, step_no, lr, beta1, beta2, eps, weight_decay, 1, rows, numels, n, pat, float(loss_scale),
+                    state_ptr, stream,
+                ),
+                "ps_adam_step_tensors",
+            )
+
+        for stage in self._stages:
+            if stage[0] == "tensors":
+                tensors(stage[1], stage[2])
+            elif stage[0] == "stream":
+                self._streamer.step(self.opt_id, step_no, lr, beta1, beta2, eps, weight_decay, loss_scale, None, 0,
+                                    stage[1], scaler)
+            else:
+                _, payloads, staging, table, pat = stage
+                moved = [(s, h) for s, h in zip(staging, payloads) if h.device.type == "cpu"]
+                for s, h in moved:
+                    s.copy_(h, non_blocking=True)
+                # a host-resident position is updated with the operator's arithmetic whatever the optimizer's own is
+                # (the reference runs its CPU operator on it, fp16_cpu_adam.py:415-428)
+                if self.arithmetic == "torch":
+                    _lib.check(self._lib.ps_adam_set_arithmetic(self.opt_id, _lib.PS_ARITH_OPERATOR), "ps_adam_set_arithmetic")
+                try:
+                    tensors(table, pat)
+                finally:
+                    if self.arithmetic == "torch":
+                        _lib.check(self._lib.ps_adam_set_arithmetic(self.opt_id, _lib.PS_ARITH_TORCH), "ps_adam_set_arithmetic")
+                for s, h in moved:
+                    h.copy_(s, non_blocking=True)
 
     def invalidate_tables(self):
         """Call after re-allocating chunk payloads."""
@@ -346,11 +453,13 @@ class FP16Adam(torch.optim.Optimizer):
                 scaler = self.loss_scaler
                 if self.scan_in_step:
                     self.check_overflow_chunks()
-                if self._tensor_table is not None:
+                if self._stages is not None:
+                    self._run_stages(0, hyper, -1.0, scaler, stream)
+                elif self._tensor_table is not None:
                     rows, numels, n_tensors = self._tensor_table
                     _lib.check(
                         self._lib.ps_adam_step_tensors(
-                            self.opt_id, 0, lr, beta1, beta2, eps, weight_decay, 1, rows, numels, n_tensors, -1.0,
+                            self.opt_id, 0, lr, beta1, beta2, eps, weight_decay, 1, rows, numels, n_tensors, None, -1.0,
                             scaler.state_ptr, stream,
                         ),
                         "ps_adam_step_tensors",
@@ -381,11 +490,13 @@ class FP16Adam(torch.optim.Optimizer):
             self._steps_dirty = True
             step_no = self._host_step
             loss_scale = self.loss_scaler.loss_scale if self.loss_scaler is not None else -1
-            if self._tensor_table is not None:
+            if self._stages is not None:
+                self._run_stages(step_no, hyper, loss_scale, None, stream)
+            elif self._tensor_table is not None:
                 rows, numels, n_tensors = self._tensor_table
                 _lib.check(
                     self._lib.ps_adam_step_tensors(
-                        self.opt_id, step_no, lr, beta1, beta2, eps, weight_decay, 1, rows, numels, n_tensors,
+                        self.opt_id, step_no, lr, beta1, beta2, eps, weight_decay, 1, rows, numels, n_tensors, None,
                         float(loss_scale), None, stream,
                     ),
                     "ps_adam_step_tensors",

@@ -16,7 +16,9 @@ from . import _lib
 
 
 class HostChunkStreamer:
-    def __init__(self, client, host_positions, n_slots=2):
+    def __init__(self, client, host_positions, n_slots=2, step_indices=None):
+        """``step_indices``: which of ``host_positions`` ``step()`` streams (default: all of them); the gradient probe
+        always covers every position."""
         self.client = client
         self.n_slots = n_slots
         self.chunk_numel = client.default_chunk_size
@@ -36,6 +38,11 @@ class HostChunkStreamer:
             rows.append([t.data_ptr() for t in payloads])
         self.host_table = _lib.chunk_array(rows)
         self.n_host = len(rows)
+        if step_indices is None:
+            self.step_table, self.n_step = self.host_table, self.n_host
+        else:
+            picked = [rows[k] for k in step_indices]
+            self.step_table, self.n_step = (_lib.chunk_array(picked) if picked else None), len(picked)
         dev = client.device
         n = self.chunk_numel
         # staging lives for the life of the optimizer: allocating it per step (as the reference does with
@@ -61,8 +68,8 @@ class HostChunkStreamer:
         ``scaler`` (a device-resident DynamicLossScaler) selects the device-gated form."""
         _lib.check(
             self._lib.ps_adam_step_hybrid(
-                opt_id, step_no, lr, beta1, beta2, eps, weight_decay, 1, resident, n_resident, self.host_table,
-                self.n_host, self.chunk_numel, self.staging, self.n_slots, calls, float(loss_scale),
+                opt_id, step_no, lr, beta1, beta2, eps, weight_decay, 1, resident, n_resident, self.step_table,
+                self.n_step, self.chunk_numel, self.staging, self.n_slots, calls, float(loss_scale),
                 scaler.state_ptr if scaler is not None else None, _lib.current_stream_handle(),
             ),
             "ps_adam_step_hybrid",

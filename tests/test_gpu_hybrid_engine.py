@@ -567,3 +567,73 @@ def test_two_host_threads_stream_host_chunks_on_one_gpu_at_the_same_time():
         h.compare(oc, what=f"thread {t}")
         if t == 1:
             assert h.opt.loss_scaler.loss_scale == oscaler.loss_scale and h.opt.loss_scaler.cur_iter == steps
+
+
+class _DeepPartlyFrozen(_Deep):
+    """Six 272-element layers, one per 300-element chunk position.  Frozen: layer 0's weight (so the step's first
+    operator call is a bias in the middle of a chunk that also holds a frozen tensor), the biases of layers 1 and 4,
+    and all of layer 2 (a position that drops out of the step)."""
+
+    def __init__(self):
+        super().__init__()
+        for p in (self.layers[0].weight, self.layers[1].bias, self.layers[4].bias, *self.layers[2].parameters()):
+            p.requires_grad_(False)
+
+
+@pytest.mark.parametrize("arithmetic", ["operator", "torch"])
+@pytest.mark.parametrize("loss_scale", [0, 64])
+@pytest.mark.parametrize("host", [(0, 1), (3, 5), (1, 3, 4), (0, 3), (0, 1, 2, 3, 4, 5)])
+def test_frozen_parameters_together_with_host_resident_positions(host, loss_scale, arithmetic):
+    """Chunks that mix frozen and trainable tensors, some of them with their optimizer state in host memory: the step
+    is spread over a tensor-list call (resident tensors), the streamed whole-chunk form (host positions without frozen
+    tensors) and staged tensor-list calls (host positions with frozen tensors), under ONE call pattern.  Bit for bit
+    what the reference computes under that placement; frozen tensors do not move."""
+    torch.manual_seed(1)
+    config = {
+        "optimizer": {"type": "AdamW", "params": {"lr": 1e-3, "betas": (0.9, 0.999), "eps": 1e-8, "weight_decay": 0.05,
+                                                  "arithmetic": arithmetic}},
+        "fp16": {"enabled": True, "loss_scale": loss_scale, "initial_scale_power": 7, "loss_scale_window": 3, "hysteresis": 2, "min_loss_scale": 1},
+        "default_chunk_size": 300,
+        "client": {"host_chunk_policy": lambda position: position in host},
+    }
+    engine, optimizer = ps.initialize_engine(model_func=_DeepPartlyFrozen, local_rank=0, config=config)
+    client = engine.client
+    cl = client.chunk_list
+    pos = client.positions()
+    assert [q.on_host for q in pos] == [i in host for i in range(6)]
+    frozen = [p for p in engine.module.parameters() if not p.requires_grad]
+    assert len(frozen) == 5
+    masters = [client.access_data(client.param_fp16_to_param_fp32_map[p]) for p in frozen]
+    frozen_before = [(p.detach().clone(), m.clone()) for p, m in zip(frozen, masters)]
+    spans = tensor_spans(client, optimizer)
+    assert len(spans) == 7 and spans[0] == (0, 256, 16)  # layer 0's bias comes first
+    mirror = [{"p32": _snap(cl[q.fp32].payload), "m": _snap(cl[q.exp_avg].payload),
+               "v": _snap(cl[q.exp_avg_sq].payload), "p16": _snap(cl[q.fp16].payload)} for q in pos]
+    oscaler = oracle.scaler_from_config(config["fp16"])
+    oopt = oracle.OptimizerStepOracle(mirror, oscaler, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.05,
+                                      use_adamw=True, tensors=spans, arithmetic=arithmetic, operator_chunks=host)
+    x = torch.randn(8, 16, device="cuda").half()
+    for it in range(6):
+        loss = engine(x * (1.0 if it != 2 or loss_scale else 6e4))  # dynamic scaler: iteration 2 overflows
+        engine.backward(loss)
+        for q, c in zip(pos, mirror):
+            c["p16"][...] = _snap(cl[q.fp16].payload)
+        optimizer.step()
+        torch.cuda.synchronize()
+        oopt.check_overflow()
+        assert oopt.step() == (it == 2 and loss_scale == 0)
+        for p, m, (p0, m0) in zip(frozen, masters, frozen_before):
+            assert torch.equal(p.detach(), p0) and torch.equal(m, m0), "a frozen parameter moved"
+        for i, (q, c) in enumerate(zip(pos, mirror)):
+            for key, cid in (("p32", q.fp32), ("m", q.exp_avg), ("v", q.exp_avg_sq), ("p16", q.fp16)):
+                assert_bits_equal(_snap(cl[cid].payload), c[key], f"host={host} iteration {it} position {i} {key}")
+        assert optimizer.loss_scaler.loss_scale == oscaler.loss_scale
+    kinds = [s[0] for s in optimizer._stages]
+    whole_on_host = [i for i in host if i in (3, 5)]
+    part_on_host = [i for i in host if i in (0, 1, 4)]
+    assert kinds.count("stream") == bool(whole_on_host) and kinds.count("staged") == len(part_on_host)
+    assert kinds.count("tensors") == (len(host) < 6)
+    # the stage that holds the step's first operator call goes first: the first trainable tensor (position 0), or,
+    # with the torch formula on resident state, the first one whose state lives in host memory
+    first = 0 if arithmetic == "operator" else min(i for i in host if i != 2)
+    assert kinds[0] == ("tensors" if first not in host else "staged" if first in part_on_host else "stream")

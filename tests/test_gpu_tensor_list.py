@@ -84,7 +84,7 @@ def test_host_decided_steps_over_a_permuted_layout(arithmetic, adamw, wd, scale)
         if step > 1:
             L.new_grads(rng, scale or 1.0)
         _lib.check(
-            lib.ps_adam_step_tensors(oid, step, lr, b1, b2, eps, wd, 1, L.table, L.numels, len(SIZES),
+            lib.ps_adam_step_tensors(oid, step, lr, b1, b2, eps, wd, 1, L.table, L.numels, len(SIZES), None,
                                      float(scale) if scale is not None else -1.0, None, _lib.current_stream_handle()),
             "ps_adam_step_tensors",
         )
@@ -128,7 +128,7 @@ def test_device_gated_steps_over_a_permuted_layout(arithmetic):
             L.dev["h"].copy_(torch.from_numpy(L.host["h"]))
         scaler.scan(L.dev["h"])
         _lib.check(
-            lib.ps_adam_step_tensors(oid, 0, lr, b1, b2, eps, wd, 1, L.table, L.numels, 50, -1.0, scaler.state_ptr,
+            lib.ps_adam_step_tensors(oid, 0, lr, b1, b2, eps, wd, 1, L.table, L.numels, 50, None, -1.0, scaler.state_ptr,
                                      _lib.current_stream_handle()),
             "ps_adam_step_tensors",
         )
@@ -162,18 +162,72 @@ def test_tensor_list_argument_checks_and_empty_lists():
     lib = _lib.load()
     lib.ps_adam_create(822, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, 0)
     s = _lib.current_stream_handle()
-    assert lib.ps_adam_step_tensors(822, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, None, 0, -1.0, None, s) == 0
-    assert lib.ps_adam_step_tensors(822, 2, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, None, 3, -1.0, None, s) == _lib.PS_ERR_BAD_ARG
-    assert lib.ps_adam_step_tensors(822, 2, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, None, -1, -1.0, None, s) == _lib.PS_ERR_BAD_ARG
+    assert lib.ps_adam_step_tensors(822, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, None, 0, None, -1.0, None, s) == 0
+    assert lib.ps_adam_step_tensors(822, 2, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, None, 3, None, -1.0, None, s) == _lib.PS_ERR_BAD_ARG
+    assert lib.ps_adam_step_tensors(822, 2, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, None, -1, None, -1.0, None, s) == _lib.PS_ERR_BAD_ARG
     x = torch.ones(8, device="cuda")
     h = torch.zeros(8, dtype=torch.half, device="cuda")
     rows = _lib.chunk_array([[x.data_ptr(), x.data_ptr(), 0, h.data_ptr()], [x.data_ptr(), 0, 0, 0]])
     numels = (ctypes.c_size_t * 2)(8, 0)
-    assert lib.ps_adam_step_tensors(822, 2, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, rows, numels, 2, -1.0, None, s) == _lib.PS_ERR_BAD_ARG
+    assert lib.ps_adam_step_tensors(822, 2, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, rows, numels, 2, None, -1.0, None, s) == _lib.PS_ERR_BAD_ARG
     assert b"tensor 0" in lib.ps_last_error()
     numels = (ctypes.c_size_t * 2)(0, 0)  # zero-length tensors may carry NULL addresses and are skipped
-    assert lib.ps_adam_step_tensors(822, 2, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, rows, numels, 2, -1.0, None, s) == 0
-    assert lib.ps_adam_step_tensors(4711, 2, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, rows, numels, 2, -1.0, None, s) == _lib.PS_ERR_UNKNOWN_ID
+    assert lib.ps_adam_step_tensors(822, 2, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, rows, numels, 2, None, -1.0, None, s) == 0
+    assert lib.ps_adam_step_tensors(4711, 2, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, rows, numels, 2, None, -1.0, None, s) == _lib.PS_ERR_UNKNOWN_ID
     torch.cuda.synchronize()
     assert torch.equal(x, torch.ones(8, device="cuda"))
     lib.ps_adam_destroy(822)
+
+
+@pytest.mark.parametrize("gated", [False, True])
+def test_one_step_spread_over_two_tensor_list_calls_under_one_call_pattern(gated):
+    """A step of 20 operator calls made through two entry-point calls: the first list holds the step's first call
+    (reference tensor 0, here at index 2 of a shuffled list) and names it; the second list says that the first call is
+    not among its tensors.  Tensor 0 takes the running product, all 19 others pow, as in one call over all 20."""
+    lib = _lib.load()
+    lr, b1, b2, eps, wd = 1e-3, 0.9, 0.999, 1e-8, 0.01
+    sizes = SIZES[:20]
+    L = PermutedLayout(sizes, seed=21, scale=2.0**8)
+    rng = np.random.default_rng(22)
+    oid = 823
+    _lib.check(lib.ps_adam_create(oid, lr, b1, b2, eps, wd, 1, 0), "create")
+    first_list = [7, 3, 0, 12, 19, 8]
+    second_list = [i for i in range(20) if i not in first_list]
+
+    def sub(indices):
+        rows = _lib.chunk_array([[L.table[i].param_fp32, L.table[i].exp_avg, L.table[i].exp_avg_sq, L.table[i].param_fp16] for i in indices])
+        return rows, (ctypes.c_size_t * len(indices))(*[sizes[i] for i in indices]), len(indices)
+
+    a, b = sub(first_list), sub(second_list)
+    kw = dict(init_scale=2**8, scale_factor=2, scale_window=1000)
+    scaler = ps.DynamicLossScaler(**kw)
+    scaler.materialize("cuda:0", betas=(b1, b2))
+    state = scaler.state_ptr if gated else None
+    native = oracle.AdamOracle(lr, b1, b2, eps, wd, True)
+    s = _lib.current_stream_handle()
+    steps = (1, 2, 3, 4) if gated else (1, 2, 3, 50, 51)
+    for step in steps:
+        if step > 1:
+            L.new_grads(rng, 2.0**8)
+        for (rows, numels, n), pat in ((a, _lib.call_pattern(20, 2, 0, sizes[0])), (b, _lib.call_pattern(20, 0, 0, 0))):
+            _lib.check(lib.ps_adam_step_tensors(oid, 0 if gated else step, lr, b1, b2, eps, wd, 1, rows, numels, n, pat,
+                                                -1.0 if gated else 2.0**8, state, s), "ps_adam_step_tensors")
+        if gated:
+            scaler.update_scale(None, operator_calls=20)
+        torch.cuda.synchronize()
+        for i in range(20):
+            p, h, m, v = L.views(i)
+            pc, mc, vc, hc = p.copy(), m.copy(), v.copy(), h.copy()
+            native.update(step, lr, b1, b2, eps, wd, True, pc, hc, mc, vc, 2.0**8)
+            p[...], m[...], v[...] = pc, mc, vc
+            h[...] = oracle.cast_fp32_to_fp16(pc)
+        L.compare(f"gated={gated} step {step}")
+    # a pattern that does not describe a whole tensor of the list is refused before anything is queued
+    rows, numels, n = a
+    E = _lib.PS_ERR_BAD_ARG
+    for bad in (_lib.call_pattern(0, 2, 0, sizes[0]), _lib.call_pattern(20, 6, 0, 5), _lib.call_pattern(20, -1, 0, 5),
+                _lib.call_pattern(20, 2, 1, sizes[0]), _lib.call_pattern(20, 2, 0, sizes[0] + 1)):
+        assert lib.ps_adam_step_tensors(oid, 60, lr, b1, b2, eps, wd, 1, rows, numels, n, bad, 2.0**8, None, s) == E
+    torch.cuda.synchronize()
+    L.compare("after the refused calls")
+    lib.ps_adam_destroy(oid)

@@ -185,7 +185,7 @@ def test_library_loads_and_exports_every_declared_symbol():
     lib = _lib.load()
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.ps_abi_version() == 3
+    assert lib.ps_abi_version() == _lib.PS_ABI_VERSION == 4
     # host-only entry points: registry and argument checks work without a GPU
     assert lib.ps_adam_create(77, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, 0) == 0
     assert lib.ps_adam_destroy(77) == 0
