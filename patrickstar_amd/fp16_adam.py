@@ -57,6 +57,13 @@ class _ParamState(dict):
             self._sync()
         return super().__getitem__(key)
 
+    def __setitem__(self, key, value):
+        super().__setitem__(key, value)
+        if key in ("lr", "betas", "eps", "weight_decay"):
+            owner = self._owner()
+            if owner is not None:
+                owner._hyper_checked = False  # the next step() looks at every parameter's entries again
+
     def items(self):
         self._sync()
         return super().items()
@@ -113,6 +120,7 @@ class FP16Adam(torch.optim.Optimizer):
         self._dynamic = isinstance(loss_scaler, DynamicLossScaler)
         self._host_overflow = False
         self._steps_dirty = False
+        self._hyper_checked = False  # every trainable parameter's state entries hold the same hyper-parameters
         self._host_step = None  # shared step counter of the host-decided path; taken from state[p]["step"] at first use
         self.staging_slots = 2  # HBM staging slots for host-resident chunks (double buffering)
 
@@ -408,13 +416,28 @@ class FP16Adam(torch.optim.Optimizer):
 
     # -- the step -----------------------------------------------------------------
     def _hyper(self):
+        """(lr, betas, eps, weight_decay) of the step: the entries of ``state[p]``, as the reference reads them per
+        tensor (``fp16_cpu_adam.py:593-598``).  The fused step applies ONE set to every tensor, so entries that differ
+        between parameters (somebody wrote ``state[p]["lr"]`` for some parameters only) are refused, not ignored."""
+        g = dict.__getitem__
+        first = None
         for group in self.param_groups:
             for p in group["params"]:
-                if p.requires_grad:
-                    st = self.state[p]
-                    g = dict.__getitem__
-                    return g(st, "lr"), g(st, "betas"), g(st, "eps"), g(st, "weight_decay")
-        return None
+                if not p.requires_grad:
+                    continue
+                st = self.state[p]
+                mine = (g(st, "lr"), g(st, "betas"), g(st, "eps"), g(st, "weight_decay"))
+                if first is None:
+                    first = mine
+                    if self._hyper_checked:
+                        return first
+                elif (mine[0], tuple(mine[1]), mine[2], mine[3]) != (first[0], tuple(first[1]), first[2], first[3]):
+                    raise ValueError(
+                        "optimizer.state holds different hyper-parameters for different parameters "
+                        f"({first} and {mine}); this step applies one lr / betas / eps / weight_decay to all of them"
+                    )
+        self._hyper_checked = True
+        return first
 
     def _first_step_entry(self):
         for group in self.param_groups:
@@ -556,6 +579,7 @@ class FP16Adam(torch.optim.Optimizer):
                     dict.__setitem__(mine, k, saved[k])
                     if k == "step":
                         step_seen = saved[k]
+        self._hyper_checked = False
         self._host_step = step_seen
         if self._dynamic:
             self.loss_scaler.materialize(self.client.device)

@@ -421,6 +421,30 @@ def test_step_tables_follow_the_reference_call_order_and_skip_frozen_parameters(
     assert (pat.n_calls, pat.first_chunk, pat.first_offset, pat.first_numel) == (3, 0, 14, 3)
 
 
+@pytest.mark.skipif(not os.path.exists(_lib.LIB_PATH), reason="HIP library not built")
+def test_hyper_parameters_are_read_from_the_state_entries_and_must_agree():
+    """The reference reads lr / betas / eps / weight_decay from state[p] per tensor (fp16_cpu_adam.py:593-598), not
+    from param_groups.  The fused step applies one set: rewriting every parameter's entry takes effect at the next
+    step, entries that differ between trainable parameters are refused, frozen parameters are not looked at."""
+    client = ps.PatrickStarClient(0, 32, device="cpu")
+    model = _Tiny()
+    model.a.bias.requires_grad_(False)
+    client.register_model(model)
+    opt = ps.FP16Adam(client, model.parameters(), lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=0.1)
+    assert opt._hyper() == (1e-3, (0.9, 0.99), 1e-6, 0.1)
+    opt.param_groups[0]["lr"] = 7.0  # ignored, as in the reference
+    assert opt._hyper()[0] == 1e-3
+    opt.state[model.b.weight]["lr"] = 5e-4
+    with pytest.raises(ValueError, match="different hyper-parameters"):
+        opt._hyper()
+    for p in model.parameters():
+        if p.requires_grad:
+            opt.state[p]["lr"] = 5e-4
+    assert opt._hyper()[0] == 5e-4
+    opt.state[model.a.bias]["weight_decay"] = 0.5  # frozen: never handed to the operator
+    assert opt._hyper() == (5e-4, (0.9, 0.99), 1e-6, 0.1)
+
+
 def test_placement_is_decided_from_the_free_hbm_when_the_model_is_registered():
     """use_hybrid_adam + a memory margin decide where optimizer state lives (fp16_cpu_adam.py:523-528,
     memtracer.py:190-214, chunk_io_buff.py:234-239): everything resident when it fits, the FIRST positions resident
