@@ -992,7 +992,7 @@ int ps_overflow_scan_host_chunks(const ps_chunk* host_chunks, int n_chunks, size
     // fp16 payloads that live in HBM are probed in place on the caller's stream
     for (int k = 0; k < n_chunks; ++k) {
         if (!fp16_in_hbm[k]) continue;
-        hipLaunchKernelGGL(scan_f16_kernel, dim3(grid_1d(n_tiles)), dim3(kAuxBlock), 0, caller,
+        hipLaunchKernelGGL(scan_f16_kernel, dim3(grid_1d(n_tiles)), dim3(kScanBlock), kScanLdsBytes, caller,
                            host_chunks[k].param_fp16, chunk_numel, n_tiles, d_state);
         PS_HIP(hipGetLastError());
     }
@@ -1010,7 +1010,7 @@ int ps_overflow_scan_host_chunks(const ps_chunk* host_chunks, int n_chunks, size
                               hipMemcpyHostToDevice, p->h2d));
         PS_HIP(hipEventRecord(p->h2d_done[s], p->h2d));
         PS_HIP(hipStreamWaitEvent(p->compute, p->h2d_done[s], 0));
-        hipLaunchKernelGGL(scan_f16_kernel, dim3(grid_1d(n_tiles)), dim3(kAuxBlock), 0, p->compute,
+        hipLaunchKernelGGL(scan_f16_kernel, dim3(grid_1d(n_tiles)), dim3(kScanBlock), kScanLdsBytes, p->compute,
                            staging[s].param_fp16, chunk_numel, n_tiles, d_state);
         PS_HIP(hipGetLastError());
         PS_HIP(hipEventRecord(p->compute_done[s], p->compute));
@@ -1110,7 +1110,7 @@ int ps_overflow_scan(const uint16_t* d_grads_fp16, size_t numel, ps_step_state* 
     if (numel == 0) return 0;
     if (!d_grads_fp16) return fail(PS_ERR_BAD_ARG, "d_grads_fp16 is NULL");
     size_t n_tiles = (numel + kScanTile - 1) / kScanTile;
-    hipLaunchKernelGGL(scan_f16_kernel, dim3(grid_1d(n_tiles)), dim3(kAuxBlock), 0,
+    hipLaunchKernelGGL(scan_f16_kernel, dim3(grid_1d(n_tiles)), dim3(kScanBlock), kScanLdsBytes,
                        static_cast<hipStream_t>(stream), d_grads_fp16, numel, n_tiles, d_state);
     PS_HIP(hipGetLastError());
     return 0;
@@ -1137,7 +1137,7 @@ int ps_overflow_scan_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_n
     if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, kScanTile)) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid, int) {
-        hipLaunchKernelGGL(scan_chunks_kernel, grid, dim3(kAuxBlock), 0, s, b, chunk_numel, d_state);
+        hipLaunchKernelGGL(scan_chunks_kernel, grid, dim3(kScanBlock), kScanLdsBytes, s, b, chunk_numel, d_state);
     });
 }
 
@@ -1146,7 +1146,7 @@ int ps_overflow_scan_chunks_noalloc(const ps_chunk* chunks, int n_chunks, size_t
 {
     if (!d_flag) return fail(PS_ERR_BAD_ARG, "d_flag is NULL");
     ChunkList a;
-    if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, kScanTile)) return rc;
+    if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, kPartialTile)) return rc;
     if (n_chunks == 0 || a.tiles_per_chunk == 0) return 0;
     // one scratch word per workgroup of the first kernel
     const size_t max_chunks = kScratchWords / a.tiles_per_chunk;  // 0 when one chunk alone is too long
@@ -1155,7 +1155,7 @@ int ps_overflow_scan_chunks_noalloc(const ps_chunk* chunks, int n_chunks, size_t
                     "%d chunks of %zu elements need %zu scratch words; this entry point holds %zu (at most %zu "
                     "elements per call): split the list or use ps_overflow_scan_chunks",
                     n_chunks, chunk_numel, (size_t)n_chunks * a.tiles_per_chunk, kScratchWords,
-                    kScratchWords * (size_t)kScanTile);
+                    kScratchWords * (size_t)kPartialTile);
     uint32_t* scratch = nullptr;
     if (int rc = scratch_address(&scratch)) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);

@@ -20,6 +20,18 @@
 #ifndef PS_STREAMING
 #define PS_STREAMING 0  // bit 0: non-temporal loads, bit 1: non-temporal stores of chunk payloads (both slower on MI355X)
 #endif
+// Launch shape of the inf/nan probe kernels (pure read streams).  Measured on 3.2 GB of fp16 payloads: single-wave
+// workgroups with 8 loads per lane and 6 resident workgroups per CU read 6.85 TB/s; 256 threads x 4 loads, uncapped,
+// 6.29 TB/s.
+#ifndef PS_SCAN_BLOCK
+#define PS_SCAN_BLOCK 64  // threads per workgroup (64 or a multiple of it)
+#endif
+#ifndef PS_SCAN_UNROLL
+#define PS_SCAN_UNROLL 8  // 16-byte loads per lane per tile
+#endif
+#ifndef PS_SCAN_LDS_KB
+#define PS_SCAN_LDS_KB 26  // KiB of unused dynamic LDS per workgroup (0: no cap on resident workgroups)
+#endif
 #if PS_MAX_WAVES_PER_EU > 0
 #define PS_OCCUPANCY __attribute__((amdgpu_waves_per_eu(1, PS_MAX_WAVES_PER_EU)))
 #else

@@ -348,57 +348,71 @@ __device__ __forceinline__ uint32_t nonfinite_halves(uint32_t w)
 }
 
 // OR across the block: shuffle butterfly inside each wave, LDS across the
-// four waves, then at most one atomic per block (none when nothing was seen).
+// waves of the block (if it has several), then at most one atomic per block (none when nothing was seen).
+template <int BLOCK = kAuxBlock>
 __device__ __forceinline__ void block_flag_commit(uint32_t hit, uint32_t* flag)
 {
-    __shared__ uint32_t wave_hit[kAuxBlock / 64];
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) hit |= (uint32_t)__shfl_xor((int)hit, off, 64);
+    if (BLOCK == 64) {
+        if (threadIdx.x == 0 && hit) atomicOr(flag, 1u);
+        return;
+    }
+    __shared__ uint32_t wave_hit[BLOCK / 64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     if (lane == 0) wave_hit[wave] = hit;
     __syncthreads();
     if (threadIdx.x == 0) {
         uint32_t any = 0;
 #pragma unroll
-        for (int w = 0; w < kAuxBlock / 64; ++w) any |= wave_hit[w];
+        for (int w = 0; w < BLOCK / 64; ++w) any |= wave_hit[w];
         if (any) atomicOr(flag, 1u);
     }
 }
 
-constexpr int kScanUnroll = 4;
-constexpr int kScanTile = kAuxBlock * 8 * kScanUnroll;  // 16-byte loads of 8 halves: 8192 halves = 16 KiB per tile
+// Launch shape of the probe kernels that commit to the device flag: threads per workgroup, 16-byte loads per lane,
+// and an unused dynamic-LDS request that caps the resident workgroups per CU (0: no cap).
+constexpr int kScanBlock = PS_SCAN_BLOCK;
+constexpr int kScanUnroll = PS_SCAN_UNROLL;
+constexpr int kScanTile = kScanBlock * 8 * kScanUnroll;  // halves per tile
+constexpr size_t kScanLdsBytes = (size_t)PS_SCAN_LDS_KB * 1024;
+// The two-stage probe keeps one partial word per tile: large tiles, so that the word array stays small.
+constexpr int kPartialUnroll = 4;
+constexpr int kPartialTile = kAuxBlock * 8 * kPartialUnroll;  // 8192 halves = 16 KiB per tile
 
-// One scan tile of a fp16 buffer.
+// One scan tile of a fp16 buffer, by a workgroup of BLOCK threads: UNROLL 16-byte loads of 8 halves per lane.
+template <int BLOCK, int UNROLL>
 __device__ __forceinline__ uint32_t scan_tile_f16(const uint16_t* __restrict__ h, size_t numel,
                                                   size_t tile)
 {
+    constexpr size_t kTileHalves = (size_t)BLOCK * 8 * UNROLL;
     uint32_t hit = 0;
-    const size_t base = tile * (size_t)kScanTile;
+    const size_t base = tile * kTileHalves;
     if (base >= numel) return 0;
-    if ((((uintptr_t)h) & 15u) == 0 && base + kScanTile <= numel) {
-        uint4v w[kScanUnroll];
+    if ((((uintptr_t)h) & 15u) == 0 && base + kTileHalves <= numel) {
+        uint4v w[UNROLL];
 #pragma unroll
-        for (int u = 0; u < kScanUnroll; ++u)
-            w[u] = ld_u4(h + base + ((size_t)u * kAuxBlock + threadIdx.x) * 8);
+        for (int u = 0; u < UNROLL; ++u)
+            w[u] = ld_u4(h + base + ((size_t)u * BLOCK + threadIdx.x) * 8);
 #pragma unroll
-        for (int u = 0; u < kScanUnroll; ++u)
+        for (int u = 0; u < UNROLL; ++u)
             hit |= nonfinite_halves(w[u][0]) | nonfinite_halves(w[u][1]) |
                    nonfinite_halves(w[u][2]) | nonfinite_halves(w[u][3]);
     } else {
-        size_t end = base + kScanTile < numel ? base + kScanTile : numel;
-        for (size_t i = base + threadIdx.x; i < end; i += kAuxBlock)
+        size_t end = base + kTileHalves < numel ? base + kTileHalves : numel;
+        for (size_t i = base + threadIdx.x; i < end; i += BLOCK)
             hit |= ((h[i] & 0x7C00u) == 0x7C00u) ? 1u : 0u;
     }
     return hit;
 }
 
-__global__ void __launch_bounds__(kAuxBlock)
+__global__ void __launch_bounds__(kScanBlock)
     scan_f16_kernel(const uint16_t* __restrict__ h, size_t numel, size_t n_tiles,
                     ps_step_state* st)
 {
     uint32_t hit = 0;
-    for (size_t t = blockIdx.x; t < n_tiles; t += gridDim.x) hit |= scan_tile_f16(h, numel, t);
-    block_flag_commit(hit, &st->overflow);
+    for (size_t t = blockIdx.x; t < n_tiles; t += gridDim.x) hit |= scan_tile_f16<kScanBlock, kScanUnroll>(h, numel, t);
+    block_flag_commit<kScanBlock>(hit, &st->overflow);
 }
 
 __global__ void __launch_bounds__(kAuxBlock)
@@ -412,11 +426,11 @@ __global__ void __launch_bounds__(kAuxBlock)
     block_flag_commit(hit, &st->overflow);
 }
 
-__global__ void __launch_bounds__(kAuxBlock)
+__global__ void __launch_bounds__(kScanBlock)
     scan_chunks_kernel(ChunkBatch b, size_t chunk_numel, ps_step_state* st)
 {
-    uint32_t hit = scan_tile_f16(b.c[blockIdx.y].param_fp16, chunk_numel, blockIdx.x);
-    block_flag_commit(hit, &st->overflow);
+    uint32_t hit = scan_tile_f16<kScanBlock, kScanUnroll>(b.c[blockIdx.y].param_fp16, chunk_numel, blockIdx.x);
+    block_flag_commit<kScanBlock>(hit, &st->overflow);
 }
 
 // The same probe without atomics and without a caller-side state: every workgroup leaves the OR over its tile in
@@ -425,7 +439,7 @@ __global__ void __launch_bounds__(kAuxBlock)
     scan_chunks_partial_kernel(ChunkBatch b, size_t chunk_numel, uint32_t* __restrict__ partial)
 {
     __shared__ uint32_t wave_hit[kAuxBlock / 64];
-    uint32_t hit = scan_tile_f16(b.c[blockIdx.y].param_fp16, chunk_numel, blockIdx.x);
+    uint32_t hit = scan_tile_f16<kAuxBlock, kPartialUnroll>(b.c[blockIdx.y].param_fp16, chunk_numel, blockIdx.x);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) hit |= (uint32_t)__shfl_xor((int)hit, off, 64);
     if ((threadIdx.x & 63) == 0) wave_hit[threadIdx.x >> 6] = hit;

@@ -21,7 +21,7 @@ def same_typed(a, b):
 
 # ---------------------------------------------------------------- probe
 
-@pytest.mark.parametrize("n", [1, 7, 2047, 2048, 8192, 8192 * 3 + 5, 1 << 20])
+@pytest.mark.parametrize("n", [1, 7, 2047, 2048, 4095, 4096, 4097, 8192, 8192 * 3 + 5, 1 << 20])
 def test_overflow_scan_positions_and_values(n):
     base = (torch.randn(n, device="cuda") * 100).half()
     assert ps.DynamicLossScaler._has_inf_or_nan(base) is False
