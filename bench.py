@@ -639,7 +639,7 @@ def ceiling(args):
             results["probe_update4_step_shape"] = entry(measure(lambda: fn(1, 17)), nbytes, reads, writes, tiles_per_workgroup=1, lds_kb=17,
                                                         resident_workgroups_per_cu=9)
     # Is the limit the DRAM or the path to it?  (1) The pure-read kernel over a window small enough to stay in the
-    # memory-side cache (256 MiB on this GPU), launched again and again: data that never leaves the chip.  (2) A window
+    # memory-side cache (256 MiB on this GPU), launched again and again: data that need not leave the chip.  (2) A window
     # read once (so that it sits in that cache) and then copied, window after window over the whole list, against plain
     # copies of the same windows: would keeping a step's DRAM reads and DRAM writes apart in time pay?
     windows = {}
@@ -690,7 +690,7 @@ def ceiling(args):
         "note": "probe_*: best launch shape of the sweep (sweeps_GBps holds every shape); time_sliced_bound: 14 B/element read at the "
         "pure-read rate plus 14 B/element written at the pure-write rate, as if reads and writes never met on the memory bus; "
         "probe_update4 is the step's access pattern without its arithmetic; windows: reread = the pure-read kernel launched repeatedly "
-        "over one window of that size (a window of up to 256 MiB stays in the memory-side cache), plain_copy / read_then_copy = 4 GiB "
+        "over one window of that size (a window of up to 256 MiB fits the memory-side cache), plain_copy / read_then_copy = 4 GiB "
         "copied window by window, without and with a pure-read pass over each window just before its copy (GB/s of the copy's bytes)",
     }
     print(json.dumps(out))
