@@ -169,6 +169,7 @@ class FP16Adam(torch.optim.Optimizer):
         self._tensor_table = None  # (ps_chunk rows, numels, count) when the step has to go tensor by tensor
         self._calls = None  # ps_call_pattern of one step (None: no operator call at all)
         self._stages = None  # the entry-point calls of a step that cannot be made as one (see _plan_stages)
+        self._trainable_seen = None  # requires_grad of every parameter when the tables were built
         self._operator_calls = 0
         if self._dynamic and torch.cuda.is_available():
             self.loss_scaler.materialize(self.client.device, betas=betas)
@@ -439,23 +440,51 @@ class FP16Adam(torch.optim.Optimizer):
         self._hyper_checked = True
         return first
 
+    def _stepped_params(self):
+        """The parameters the steps so far have updated: those that were trainable when the tables were last built
+        (before the first step: those that are trainable now)."""
+        params = self.param_groups[0]["params"]
+        flags = self._trainable_seen if self._trainable_seen is not None else [p.requires_grad for p in params]
+        return [p for p, on in zip(params, flags) if on]
+
     def _first_step_entry(self):
-        for group in self.param_groups:
-            for p in group["params"]:
-                if p.requires_grad:
-                    return dict.__getitem__(self.state[p], "step")
+        for p in self._stepped_params():
+            return dict.__getitem__(self.state[p], "step")
         return 0
 
     def _sync_steps(self):
-        """Write the shared step counter (device-resident or host-side) into every state[p]["step"]."""
+        """Write the shared step counter (device-resident or host-side) into state[p]["step"] of every parameter that
+        the steps so far have updated."""
         if not self._steps_dirty:
             return
         self._steps_dirty = False
         step = self.loss_scaler.adam_step if self._dynamic else self._host_step
-        for group in self.param_groups:
-            for p in group["params"]:
-                if p.requires_grad:
-                    dict.__setitem__(self.state[p], "step", step)
+        for p in self._stepped_params():
+            dict.__setitem__(self.state[p], "step", step)
+
+    def _trainable_changed(self, now):
+        """requires_grad of some parameter changed since the last step.  The reference counts ``state[p]["step"]`` per
+        parameter and hands each tensor's own count to the operator (fp16_cpu_adam.py:571-574,603); the fused step has
+        ONE counter.  Freezing a parameter is therefore fine at any time; a parameter that becomes trainable must
+        stand at the common count (true before the first step, or if it was trainable for every step so far)."""
+        before = self._trainable_seen
+        if before is not None:
+            self._sync_steps()
+            if self._dynamic:
+                common = self.loss_scaler.adam_step
+            else:
+                common = self._host_step if self._host_step is not None else self._first_step_entry()
+            for p, was, on in zip(self.param_groups[0]["params"], before, now):
+                own = dict.__getitem__(self.state[p], "step")
+                if on and not was and own != common:
+                    raise NotImplementedError(
+                        f"parameter {p.ps_attr.name} became trainable after {own} steps of its own while the others "
+                        f"have made {common}: the reference would hand the operator a different step number for it, "
+                        "which one fused step cannot do"
+                    )
+        self._trainable_seen = now
+        self._tables = None
+        self._hyper_checked = False
 
     @torch.no_grad()
     def step(self, closure=None):
@@ -464,6 +493,11 @@ class FP16Adam(torch.optim.Optimizer):
         if closure is not None:
             with torch.enable_grad():
                 loss = closure()
+        # which parameters are trainable is looked at every step, as the reference does (fp16_cpu_adam.py:569-571):
+        # freezing or unfreezing a parameter between steps rebuilds the descriptor tables and the call pattern
+        trainable_now = tuple(p.requires_grad for p in self.param_groups[0]["params"])
+        if trainable_now != self._trainable_seen:
+            self._trainable_changed(trainable_now)
         hyper = self._hyper()
         if hyper is None:
             return loss

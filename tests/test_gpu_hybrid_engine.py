@@ -637,3 +637,57 @@ def test_frozen_parameters_together_with_host_resident_positions(host, loss_scal
     # with the torch formula on resident state, the first one whose state lives in host memory
     first = 0 if arithmetic == "operator" else min(i for i in host if i != 2)
     assert kinds[0] == ("tensors" if first not in host else "staged" if first in part_on_host else "stream")
+
+
+def test_freezing_and_unfreezing_parameters_between_steps():
+    """requires_grad is looked at every step (fp16_cpu_adam.py:569-571).  Unfreezing before the first step and freezing
+    later both follow the reference (oracle with the matching tensor list); a parameter that comes back after it missed
+    steps would need its own step number, which is refused loudly instead of being updated with the common one."""
+    torch.manual_seed(0)
+    config = {
+        "optimizer": {"type": "AdamW", "params": {"lr": 1e-2, "betas": (0.9, 0.999), "eps": 1e-8, "weight_decay": 0.1}},
+        "fp16": {"enabled": True, "loss_scale": 128},
+        "default_chunk_size": 2000,
+    }
+    engine, optimizer = ps.initialize_engine(model_func=_PartlyFrozen, local_rank=0, config=config)
+    client = engine.client
+    cl = client.chunk_list
+    pos = client.positions()
+    module = engine.module
+    for p in module.fc1.parameters():  # frozen when the engine was built (no backward hook): trainable from step 1 on
+        p.requires_grad_(True)
+    mirror = [{"p32": _snap(cl[q.fp32].payload), "m": _snap(cl[q.exp_avg].payload),
+               "v": _snap(cl[q.exp_avg_sq].payload), "p16": _snap(cl[q.fp16].payload)} for q in pos]
+    oopt = oracle.OptimizerStepOracle(mirror, oracle.StaticScalerOracle(128), lr=1e-2, betas=(0.9, 0.999), eps=1e-8,
+                                      weight_decay=0.1, use_adamw=True, tensors=tensor_spans(client, optimizer))
+    assert len(oopt.tensors) == 5
+    x = torch.randn(16, 24, device="cuda").half()
+
+    def iterate(what):
+        loss = engine(x)
+        engine.backward(loss)
+        for q, c in zip(pos, mirror):
+            c["p16"][...] = _snap(cl[q.fp16].payload)
+        optimizer.step()
+        torch.cuda.synchronize()
+        oopt.step()
+        for q, c in zip(pos, mirror):
+            for key, cid in (("p32", q.fp32), ("m", q.exp_avg), ("v", q.exp_avg_sq), ("p16", q.fp16)):
+                assert_bits_equal(_snap(cl[cid].payload), c[key], f"{what} {key}")
+
+    iterate("all five trainable, step 1")
+    iterate("all five trainable, step 2")
+    module.gain.requires_grad_(False)  # the first tensor of the step drops out: the call pattern moves on
+    module.fc2.bias.requires_grad_(False)
+    oopt.tensors = tensor_spans(client, optimizer)
+    assert len(oopt.tensors) == 3 and optimizer.state[module.gain]["step"] == 2
+    gain_before = client.access_data(module.gain).clone()
+    iterate("two frozen, step 3")
+    iterate("two frozen, step 4")
+    assert torch.equal(client.access_data(module.gain), gain_before)
+    assert optimizer.state[module.gain]["step"] == 2 and optimizer.state[module.fc2.weight]["step"] == 4
+    module.gain.requires_grad_(True)  # stands at 2 steps, the others at 4
+    loss = engine(x)
+    engine.backward(loss)
+    with pytest.raises(NotImplementedError, match="became trainable after 2 steps"):
+        optimizer.step()
