@@ -188,6 +188,21 @@ class FP16Adam(torch.optim.Optimizer):
         for group in self.param_groups:
             group.setdefault("amsgrad", False)
 
+    # -- the operator on one tensor ------------------------------------------------
+    def ds_cpu_adam_update(self, data, grad, momentum, variance, step, lr, beta1, beta2, eps, weight_decay,
+                           bias_correction):
+        """One operator call on one tensor, in place on ``data``, ``momentum`` and ``variance``, with the loss scaler's
+        current scale (or -1): ``fp16_cpu_adam.py:205-243`` under its own name.  The reference asserts CPU tensors
+        here; these are GPU tensors.  ``step()`` does not go through this method (it hands whole chunk lists to the
+        library); it is the per-tensor form for callers that drive the operator themselves."""
+        for name, t in (("data", data), ("grad", grad), ("momentum", momentum), ("variance", variance)):
+            assert t.device.type == "cuda", f"{name} must live on the GPU"
+        loss_scale = self.loss_scaler.loss_scale if self.loss_scaler is not None else -1
+        self.ds_opt_adam.adam_update(
+            self.opt_id, step, lr, beta1, beta2, eps, weight_decay, bias_correction,
+            data.view(-1), grad.view(-1), momentum.view(-1), variance.view(-1), loss_scale,
+        )
+
     # -- chunk descriptor tables -------------------------------------------------
     def _trainable(self):
         """The parameters ``step()`` updates, in the order the reference visits them (``fp16_cpu_adam.py:566-605``)."""

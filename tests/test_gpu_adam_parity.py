@@ -106,6 +106,31 @@ def test_operator_module_argument_checks():
         op.adam_update(901, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, True, x, x, x, x, -1)
 
 
+def test_ds_cpu_adam_update_method_hands_the_scalers_scale_to_the_operator():
+    """FP16Adam.ds_cpu_adam_update (fp16_cpu_adam.py:205-243): one operator call on 2-D tensors, flattened, with the
+    loss scaler's scale or -1; two calls with the same step number take the two branches of IncrementStep."""
+    rng = np.random.default_rng(17)
+    for scaler, scale in ((None, -1.0), (ps.LossScaler(32), 32.0)):
+        client = ps.PatrickStarClient(0, 64)
+        opt = ps.FP16Adam(client, client.append_flat_chunks(1), loss_scaler=scaler, lr=1e-2, weight_decay=0.001, use_adamw=True)
+        native = oracle.AdamOracle(1e-2, 0.9, 0.999, 1e-8, 0.001, True)
+        for call, shape in enumerate([(1024, 32), (1023,), (7, 9)]):
+            host = [rng.normal(0, 0.02, shape).astype(np.float32), (rng.normal(0, 1e-3, shape) * abs(scale)).astype(np.float16),
+                    rng.normal(0, 1e-4, shape).astype(np.float32), np.abs(rng.normal(0, 1e-6, shape)).astype(np.float32)]
+            dev = [_dev(x.copy()) for x in host]
+            step = 1 if call < 2 else 2  # same step twice (running product, then pow), then the next step (running product)
+            opt.ds_cpu_adam_update(dev[0], dev[1], dev[2], dev[3], step, 1e-2, 0.9, 0.999, 1e-8, 0.001, True)
+            torch.cuda.synchronize()
+            p, g, m, v = (x.reshape(-1).copy() for x in host)
+            native.update(step, 1e-2, 0.9, 0.999, 1e-8, 0.001, True, p, g, m, v, scale)
+            assert_bits_equal(dev[0].cpu().numpy().reshape(-1), p, f"call {call} param")
+            assert_bits_equal(dev[2].cpu().numpy().reshape(-1), m, f"call {call} exp_avg")
+            assert_bits_equal(dev[3].cpu().numpy().reshape(-1), v, f"call {call} exp_avg_sq")
+            assert_bits_equal(dev[1].cpu().numpy().reshape(-1), g, f"call {call} gradient untouched")
+    with pytest.raises(AssertionError, match="GPU"):
+        opt.ds_cpu_adam_update(torch.zeros(4), dev[1], dev[2], dev[3], 3, 1e-2, 0.9, 0.999, 1e-8, 0.0, True)
+
+
 def test_adam_update_unaligned_views_fp16_out_and_errors():
     lib = _lib.load()
     rng = np.random.default_rng(5)
