@@ -414,6 +414,31 @@ class FP16Adam(torch.optim.Optimizer):
         if self._dynamic and param.grad is not None:
             self.loss_scaler.scan(param.grad)
 
+    def has_overflow_and_reset_param(self, write_chunk_buff=None):
+        """``fp16_cpu_adam.py:287-310`` under its own name: if the sticky flag is set, rewrite every chunk's fp16
+        parameters from the fp32 masters (frozen parameters included, as the reference rewrites every chunk-based
+        parameter), clear the flag and return True.  ``step()`` does not come through here (its gate is decided on the
+        device); this form reads the flag back, i.e. it synchronises.  ``write_chunk_buff`` is accepted and ignored."""
+        if not self.has_overflow:
+            return False
+        cl = self.client.chunk_list
+        rows = [
+            [cl[pos.fp32].payload.data_ptr(), 16, 16, cl[pos.fp16].payload.data_ptr()]  # m and v are not touched
+            for pos in self.client.positions()
+            if pos.fp32 is not None and cl[pos.fp32].payload is not None
+        ]
+        if rows:
+            with torch.cuda.device(self.client.device):
+                # pinned host payloads of host-resident positions are device-accessible: the kernel reads / writes them in place
+                _lib.check(
+                    self._lib.ps_restore_fp16_chunks(
+                        _lib.chunk_array(rows), len(rows), self.client.default_chunk_size, None, _lib.current_stream_handle()
+                    ),
+                    "ps_restore_fp16_chunks",
+                )
+        self.has_overflow = False
+        return True
+
     def check_overflow_chunks(self):
         """Probe the fp16 gradient payload of every chunk (asynchronous)."""
         if not self._dynamic:

@@ -115,3 +115,38 @@ def test_restore_chunks_with_and_without_the_device_flag(n_chunks, n, mode):
         assert_bits_equal(got[gap], old[gap], f"gap behind chunk {c}")
     if state is not None:
         assert state.overflow_flag == (mode == "flag set")  # the restore does not consume the flag
+
+
+@pytest.mark.parametrize("host_positions,host_keeps_fp16", [((), True), ((1, 3), True), ((0, 2), False)])
+def test_has_overflow_and_reset_param_restores_every_chunk(host_positions, host_keeps_fp16):
+    """FP16Adam.has_overflow_and_reset_param (fp16_cpu_adam.py:287-310) as a call of its own: a set flag rewrites the
+    fp16 payload of EVERY position from its fp32 master (RNE, padding included), clears the flag and reports True; a
+    clear flag changes nothing.  Positions in pinned host memory are rewritten in place by the same kernel."""
+    import oracle
+    import patrickstar_amd as ps
+    from _harness import HybridHarness, assert_bits_equal
+
+    h = HybridHarness(4, 2048 + 77, list(host_positions), ps.DynamicLossScaler(init_scale=2**8), seed=3,
+                      host_keeps_fp16=host_keeps_fp16, lr=1e-3)
+    h.fill_state()
+    h.fill_grads(1e-3, 2.0**8)
+    before = [h.download(i) for i in range(4)]
+    assert h.opt.has_overflow_and_reset_param() is False
+    torch.cuda.synchronize()
+    for i in range(4):
+        assert_bits_equal(h.download(i)[3], before[i][3], f"clear flag: position {i} fp16 untouched")
+    h.payloads(2)[3][17] = float("nan")
+    h.opt.check_overflow_chunks()
+    assert h.opt.has_overflow is True
+    assert h.opt.has_overflow_and_reset_param() is True
+    torch.cuda.synchronize()
+    assert h.opt.has_overflow is False
+    for i in range(4):
+        p, m, v, f16 = h.download(i)
+        assert_bits_equal(f16, oracle.cast_fp32_to_fp16(before[i][0]), f"position {i} fp16 = RNE(fp32 master)")
+        for got, want, name in ((p, before[i][0], "fp32"), (m, before[i][1], "exp_avg"), (v, before[i][2], "exp_avg_sq")):
+            assert_bits_equal(got, want, f"position {i} {name} untouched")
+    assert h.opt.has_overflow_and_reset_param() is False
+    # a static scaler never reports overflow (loss_scaler.py:63-65)
+    s = HybridHarness(2, 512, [], ps.LossScaler(8), seed=4, lr=1e-3)
+    assert s.opt.has_overflow_and_reset_param() is False
