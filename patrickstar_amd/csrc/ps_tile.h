@@ -54,6 +54,24 @@ __device__ __forceinline__ void st_u4(uint16_t* p, uint4v v)
 #endif
 }
 
+// 16 bytes at an address that is only 4-byte aligned (multi-dword global accesses need dword alignment only): for
+// momentum / variance tensors that sit at another 16-byte phase than their parameter.
+typedef float4v __attribute__((aligned(4))) float4v_dword_aligned;
+template <bool DWORD_ALIGNED>
+__device__ __forceinline__ float4v ld_f4_as(const float* p)
+{
+    if (DWORD_ALIGNED) return *(const PS_GLOBAL float4v_dword_aligned*)(p);
+    return ld_f4(p);
+}
+template <bool DWORD_ALIGNED>
+__device__ __forceinline__ void st_f4_as(float* p, float4v v)
+{
+    if (DWORD_ALIGNED)
+        *(PS_GLOBAL float4v_dword_aligned*)(p) = v;
+    else
+        st_f4(p, v);
+}
+
 constexpr int kBlock = PS_BLOCK;
 constexpr unsigned kLdsBytes = PS_LDS_KB * 1024u;
 // Elements per lane per vector step.  8: one 16-byte access of fp16 and two
@@ -151,6 +169,8 @@ __device__ __forceinline__ void lane_math(const StepConsts& c, float step_size, 
 // before the first use.  Loads and stores are written once, outside any
 // branch on the arithmetic variant.
 // The loads of one whole, aligned tile: all of them issued back to back, nothing waited for.
+// STATE_DWORD_ALIGNED: exp_avg / exp_avg_sq are only 4-byte aligned (the parameter lists are aligned as always).
+template <bool STATE_DWORD_ALIGNED = false>
 __device__ __forceinline__ void tile_load(LaneTile& r, const float* __restrict__ p32, const float* __restrict__ m32,
                                           const float* __restrict__ v32, const uint16_t* __restrict__ h16, size_t base)
 {
@@ -161,14 +181,14 @@ __device__ __forceinline__ void tile_load(LaneTile& r, const float* __restrict__
 #pragma unroll
         for (int q = 0; q < kQuads; ++q) r.p[u][q] = ld_f4(p32 + i + 4 * q);
 #pragma unroll
-        for (int q = 0; q < kQuads; ++q) r.m[u][q] = ld_f4(m32 + i + 4 * q);
+        for (int q = 0; q < kQuads; ++q) r.m[u][q] = ld_f4_as<STATE_DWORD_ALIGNED>(m32 + i + 4 * q);
 #pragma unroll
-        for (int q = 0; q < kQuads; ++q) r.v[u][q] = ld_f4(v32 + i + 4 * q);
+        for (int q = 0; q < kQuads; ++q) r.v[u][q] = ld_f4_as<STATE_DWORD_ALIGNED>(v32 + i + 4 * q);
     }
 }
 
 // Arithmetic and stores of a tile whose loads are under way.
-template <int ARITH, int WD, int UNS>
+template <int ARITH, int WD, int UNS, bool STATE_DWORD_ALIGNED = false>
 __device__ __forceinline__ void tile_finish(const StepConsts& c, float step_size, float bc2inv, LaneTile& r,
                                             float* __restrict__ p32, float* __restrict__ m32,
                                             float* __restrict__ v32, uint16_t* __restrict__ h16, size_t base)
@@ -188,22 +208,22 @@ __device__ __forceinline__ void tile_finish(const StepConsts& c, float step_size
 #pragma unroll
         for (int q = 0; q < kQuads; ++q) st_f4(p32 + i + 4 * q, r.p[u][q]);
 #pragma unroll
-        for (int q = 0; q < kQuads; ++q) st_f4(m32 + i + 4 * q, r.m[u][q]);
+        for (int q = 0; q < kQuads; ++q) st_f4_as<STATE_DWORD_ALIGNED>(m32 + i + 4 * q, r.m[u][q]);
 #pragma unroll
-        for (int q = 0; q < kQuads; ++q) st_f4(v32 + i + 4 * q, r.v[u][q]);
+        for (int q = 0; q < kQuads; ++q) st_f4_as<STATE_DWORD_ALIGNED>(v32 + i + 4 * q, r.v[u][q]);
         st_halves(h16 + i, r.h[u]);
     }
 }
 
-template <int ARITH, int WD, int UNS>
+template <int ARITH, int WD, int UNS, bool STATE_DWORD_ALIGNED = false>
 __device__ __forceinline__ void adam_tile_vec(const StepConsts& c, float step_size, float bc2inv,
                                               float* __restrict__ p32, float* __restrict__ m32,
                                               float* __restrict__ v32, uint16_t* __restrict__ h16,
                                               size_t base)
 {
     LaneTile r;
-    tile_load(r, p32, m32, v32, h16, base);
-    tile_finish<ARITH, WD, UNS>(c, step_size, bc2inv, r, p32, m32, v32, h16, base);
+    tile_load<STATE_DWORD_ALIGNED>(r, p32, m32, v32, h16, base);
+    tile_finish<ARITH, WD, UNS, STATE_DWORD_ALIGNED>(c, step_size, bc2inv, r, p32, m32, v32, h16, base);
 }
 
 // Same elements, one at a time: ragged tile ends, unaligned bases and tiles that an operator call's
@@ -232,6 +252,20 @@ __device__ __forceinline__ bool aligned16(const void* a, const void* b, const vo
     return (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)d) & 15u) == 0;
 }
 
+// How a whole tile of this chunk / tensor can be accessed: all four lists 16-byte aligned; or the two parameter
+// lists aligned (fp32 to 16 bytes, fp16 to the 8 or 16 bytes of its access) and momentum / variance, which sit at
+// another phase, only to the 4 bytes of an element; or element by element.
+enum { TILE_ALIGNED = 0, TILE_STATE_DWORD_ALIGNED = 1, TILE_ELEMENTWISE = 2 };
+__device__ __forceinline__ int tile_access(const ps_chunk& ch)
+{
+    if (aligned16(ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16)) return TILE_ALIGNED;
+    const uintptr_t half_mask = kWords == 4 ? 15u : 7u;
+    if ((((uintptr_t)ch.param_fp32) & 15u) == 0 && (((uintptr_t)ch.param_fp16) & half_mask) == 0 &&
+        ((((uintptr_t)ch.exp_avg) | ((uintptr_t)ch.exp_avg_sq)) & 3u) == 0)
+        return TILE_STATE_DWORD_ALIGNED;
+    return TILE_ELEMENTWISE;
+}
+
 // first_lo .. first_hi: the elements of THIS chunk that the step's first operator call covers
 // (first_hi <= first_lo: none).  Whole tiles inside or outside that span are uniform and keep the vector
 // path; the at most two tiles that its ends run through go element by element.
@@ -246,12 +280,19 @@ __device__ __forceinline__ void adam_tile_late_consts(MakeConsts make_consts, co
     const size_t last = end < chunk_numel ? end : chunk_numel;
     const bool inside = base >= first_lo && last <= first_hi;
     const bool cut = !inside && base < first_hi && last > first_lo;
-    if (!cut && end <= chunk_numel && aligned16(ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16)) {
+    const int access = (!cut && end <= chunk_numel) ? tile_access(ch) : TILE_ELEMENTWISE;
+    if (access == TILE_ALIGNED) {
         LaneTile r;
         tile_load(r, ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16, base);
         const StepConsts c = make_consts();
         tile_finish<ARITH, WD, UNS>(c, inside ? c.first_step_size : c.step_size, inside ? c.first_bc2inv : c.bc2inv, r,
                                     ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16, base);
+    } else if (access == TILE_STATE_DWORD_ALIGNED) {
+        LaneTile r;
+        tile_load<true>(r, ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16, base);
+        const StepConsts c = make_consts();
+        tile_finish<ARITH, WD, UNS, true>(c, inside ? c.first_step_size : c.step_size, inside ? c.first_bc2inv : c.bc2inv,
+                                          r, ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16, base);
     } else {
         const StepConsts c = make_consts();
         adam_tile_scalar<ARITH, WD, UNS>(c, ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16, base, last,
@@ -267,10 +308,15 @@ __device__ __forceinline__ void adam_tile(const StepConsts& c, const ps_chunk& c
     const size_t last = end < chunk_numel ? end : chunk_numel;  // one past the tile's last element
     const bool inside = base >= first_lo && last <= first_hi;
     const bool cut = !inside && base < first_hi && last > first_lo;
-    if (!cut && end <= chunk_numel && aligned16(ch.param_fp32, ch.exp_avg, ch.exp_avg_sq, ch.param_fp16)) {
+    const int access = (!cut && end <= chunk_numel) ? tile_access(ch) : TILE_ELEMENTWISE;
+    if (access == TILE_ALIGNED) {
         adam_tile_vec<ARITH, WD, UNS>(c, inside ? c.first_step_size : c.step_size,
                                       inside ? c.first_bc2inv : c.bc2inv, ch.param_fp32, ch.exp_avg,
                                       ch.exp_avg_sq, ch.param_fp16, base);
+    } else if (access == TILE_STATE_DWORD_ALIGNED) {
+        adam_tile_vec<ARITH, WD, UNS, true>(c, inside ? c.first_step_size : c.step_size,
+                                            inside ? c.first_bc2inv : c.bc2inv, ch.param_fp32, ch.exp_avg,
+                                            ch.exp_avg_sq, ch.param_fp16, base);
     } else {
         adam_tile_scalar<ARITH, WD, UNS>(c, ch.param_fp32, ch.exp_avg, ch.exp_avg_sq,
                                          ch.param_fp16, base, last, first_lo, first_hi);
