@@ -663,10 +663,13 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
         if (u % elem_size) return -1;
         return (int)((u / elem_size) & 3u);
     };
+    // (momentum and variance may sit at any other element phase: the reference packs them in another order than the
+    // parameters; their 16-byte accesses then go to 4-byte-aligned addresses)
     const int ph = elem_phase(d_params, 4);
-    bool vec_ok = ph >= 0 && numel >= 4096 && elem_phase(d_exp_avg, 4) == ph &&
-                  elem_phase(d_exp_avg_sq, 4) == ph && elem_phase(d_grads, gsz) == ph &&
-                  (d_param_fp16_out == nullptr || elem_phase(d_param_fp16_out, 2) == ph);
+    const bool vec_ok = ph >= 0 && numel >= 4096 && elem_phase(d_exp_avg, 4) >= 0 && elem_phase(d_exp_avg_sq, 4) >= 0 &&
+                        elem_phase(d_grads, gsz) == ph &&
+                        (d_param_fp16_out == nullptr || elem_phase(d_param_fp16_out, 2) == ph);
+    const bool state_aligned = elem_phase(d_exp_avg, 4) == ph && elem_phase(d_exp_avg_sq, 4) == ph;
     if (!vec_ok) {
         scalar_span(0, numel);
     } else {
@@ -675,10 +678,17 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
         const int tail = (int)(numel - head - n_tiles * 256);
         dim3 grid(grid_1d(n_tiles + 1)), block(64);  // + 1: the workgroup that does head and tail
         uint16_t* out = d_param_fp16_out ? d_param_fp16_out + head : nullptr;
-#define PS_FLAT_VEC(WD, HALF)                                                                     \
-    hipLaunchKernelGGL((adam_flat_vec_kernel<WD, HALF>), grid, block, kLdsBytes, s, c,            \
+#define PS_FLAT_VEC_AS(WD, HALF, DWORD)                                                           \
+    hipLaunchKernelGGL((adam_flat_vec_kernel<WD, HALF, DWORD>), grid, block, kLdsBytes, s, c,     \
                        d_params + head, static_cast<const void*>(gbytes + head * gsz),            \
                        d_exp_avg + head, d_exp_avg_sq + head, out, n_tiles, (int)head, tail)
+#define PS_FLAT_VEC(WD, HALF)                       \
+    do {                                            \
+        if (state_aligned)                          \
+            PS_FLAT_VEC_AS(WD, HALF, false);        \
+        else                                        \
+            PS_FLAT_VEC_AS(WD, HALF, true);         \
+    } while (0)
         if (grads_are_half) {
             if (c.wd_mode == WD_DECOUPLED) PS_FLAT_VEC(WD_DECOUPLED, true);
             else if (c.wd_mode == WD_L2) PS_FLAT_VEC(WD_L2, true);
@@ -689,6 +699,7 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
             else PS_FLAT_VEC(WD_NONE, false);
         }
 #undef PS_FLAT_VEC
+#undef PS_FLAT_VEC_AS
     }
     PS_HIP(hipGetLastError());
     return 0;

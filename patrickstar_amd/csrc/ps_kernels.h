@@ -281,7 +281,8 @@ __device__ __forceinline__ void flat_tile_math(const StepConsts& c, const float 
     }
 }
 
-template <int WD, bool GRAD_HALF>
+// STATE_DWORD_ALIGNED: exp_avg / exp_avg_sq sit at another 16-byte phase than the parameter (any element offset).
+template <int WD, bool GRAD_HALF, bool STATE_DWORD_ALIGNED>
 __global__ void __launch_bounds__(64)
     adam_flat_vec_kernel(StepConsts c, float* p32, const void* grads, float* m32, float* v32,
                          uint16_t* out16,  // may alias grads (fp16 gradients overwritten by fp16 parameters)
@@ -316,7 +317,7 @@ __global__ void __launch_bounds__(64)
 #pragma unroll
             for (int e = 0; e < 4; ++e) g[e] = gv[e];
         }
-        float4v p = ld_f4(p32 + i), m = ld_f4(m32 + i), v = ld_f4(v32 + i);
+        float4v p = ld_f4(p32 + i), m = ld_f4_as<STATE_DWORD_ALIGNED>(m32 + i), v = ld_f4_as<STATE_DWORD_ALIGNED>(v32 + i);
         uint32_t h[4];
         // the unscale form is uniform: branch once around the arithmetic, not per element
         if (c.unscale == UNSCALE_MUL)
@@ -326,8 +327,8 @@ __global__ void __launch_bounds__(64)
         else
             flat_tile_math<WD, UNSCALE_NONE, GRAD_HALF>(c, g, p, m, v, h);
         st_f4(p32 + i, p);
-        st_f4(m32 + i, m);
-        st_f4(v32 + i, v);
+        st_f4_as<STATE_DWORD_ALIGNED>(m32 + i, m);
+        st_f4_as<STATE_DWORD_ALIGNED>(v32 + i, v);
         if (out16 != nullptr) {
             uint2v o;
             o[0] = h[0] | (h[1] << 16);

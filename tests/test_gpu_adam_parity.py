@@ -431,7 +431,7 @@ def test_adam_update_vector_path_all_phases(phase, grad_dtype):
         assert_bits_equal(t.cpu().numpy()[:phase], ref[:phase], "elements before the view")
 
 
-def test_adam_update_mismatched_phases_fall_back_to_elementwise():
+def test_adam_update_with_parameter_and_gradient_at_different_phases_goes_elementwise():
     lib = _lib.load()
     rng = np.random.default_rng(9)
     n = 9000
@@ -452,6 +452,39 @@ def test_adam_update_mismatched_phases_fall_back_to_elementwise():
     assert_bits_equal(dp.cpu().numpy()[1:1 + n], po, "param")
     assert_bits_equal(dm.cpu().numpy()[2:2 + n], mo, "exp_avg")
     assert_bits_equal(dv.cpu().numpy()[:n], vo, "exp_avg_sq")
+
+
+@pytest.mark.parametrize("grads_half", [True, False])
+@pytest.mark.parametrize("po,mo,vo", [(0, 1, 2), (3, 0, 1), (2, 2, 5), (1, 6, 3)])
+def test_adam_update_with_state_at_other_phases_than_the_parameter(po, mo, vo, grads_half):
+    """The reference packs momentum / variance tensors in another order than the parameters, so the views handed to one
+    operator call may start at different element phases: parameter and gradient share one (they share a layout), the
+    two state tensors have their own.  Long enough for the vector path; everything around the views stays untouched."""
+    lib = _lib.load()
+    rng = np.random.default_rng(90 + po + 4 * mo + 16 * vo)
+    n, pad = 256 * 40 + 77, 8
+    p = rng.normal(0, 0.02, n + 2 * pad).astype(np.float32)
+    m = rng.normal(0, 1e-4, n + 2 * pad).astype(np.float32)
+    v = np.abs(rng.normal(0, 1e-6, n + 2 * pad)).astype(np.float32)
+    g = (rng.normal(0, 1e-3, n + 2 * pad) * 64).astype(np.float16 if grads_half else np.float32)
+    out = np.zeros(n + 2 * pad, np.float16)
+    dp, dm, dv, dg, dout = (_dev(x.copy()) for x in (p, m, v, g, out))
+    oid = 906
+    lib.ps_adam_create(oid, 1e-3, 0.9, 0.999, 1e-8, 0.01, 1, 0)
+    rc = lib.ps_adam_update(oid, 3, 1e-3, 0.9, 0.999, 1e-8, 0.01, 1, dp[po:].data_ptr(), dg[po:].data_ptr(), int(grads_half),
+                            dm[mo:].data_ptr(), dv[vo:].data_ptr(), n, 64.0, dout[po:].data_ptr(), _lib.current_stream_handle())
+    assert rc == 0, lib.ps_last_error()
+    torch.cuda.synchronize()
+    lib.ps_adam_destroy(oid)
+    pw, mw, vw = p[po:po + n].copy(), m[mo:mo + n].copy(), v[vo:vo + n].copy()
+    oracle.AdamOracle(1e-3, 0.9, 0.999, 1e-8, 0.01, True).update(3, 1e-3, 0.9, 0.999, 1e-8, 0.01, True, pw, g[po:po + n].copy(), mw, vw, 64.0)
+    for got, src, off, want, name in ((dp, p, po, pw, "param"), (dm, m, mo, mw, "exp_avg"), (dv, v, vo, vw, "exp_avg_sq"),
+                                      (dout, out, po, oracle.cast_fp32_to_fp16(pw), "fp16 out")):
+        got = got.cpu().numpy()
+        assert_bits_equal(got[off:off + n], want, name)
+        assert_bits_equal(got[:off], src[:off], f"{name}: before the view")
+        assert_bits_equal(got[off + n:], src[off + n:], f"{name}: behind the view")
+    assert_bits_equal(dg.cpu().numpy(), g, "gradients are never written")
 
 
 def test_randomised_call_sequences_match_the_oracle_state_machine():
