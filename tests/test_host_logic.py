@@ -303,6 +303,26 @@ def test_argument_checks_happen_before_any_gpu_work():
     assert lib.ps_scaler_update(ctypes.c_void_p(16), 3, None, 0, 1, None) == E
     assert lib.ps_scaler_update(ctypes.c_void_p(16), 0, None, 0, -1, None) == E
     assert lib.ps_state_seed_step(ctypes.c_void_p(16), -1, 0.9, 0.999, 1, None) == E
+    # sizes beyond what one launch grid can cover (2^31 - 1 tiles per chunk) are refused by every chunk-list entry point;
+    # 2^62 elements is beyond the limit of each of them, whatever its tile size
+    huge = 2**62
+    flag = ctypes.c_void_p(16)
+    assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, 1, huge, None, 1.0, None) == E
+    assert b"beyond the launch grid" in lib.ps_last_error()
+    assert lib.ps_adam_step_chunks_gated(88, 1e-3, 1e-8, 0.0, 1, fake, 1, huge, None, flag, None) == E
+    assert lib.ps_overflow_scan_chunks(fake, 1, huge, flag, None) == E
+    assert lib.ps_overflow_scan_chunks_noalloc(fake, 1, huge, flag, None) == E
+    assert lib.ps_restore_fp16_chunks(fake, 1, huge, None, None) == E
+    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, 1, None, 0, huge, None, 0, None, 1.0, None, None) == E
+    one = (ctypes.c_size_t * 1)(huge)
+    assert lib.ps_adam_step_tensors(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, one, 1, None, 1.0, None, None) == E
+    assert b"beyond the launch grid" in lib.ps_last_error()
+    # negative counts and a call pattern that does not fit the list
+    assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, -1, 1024, None, 1.0, None) == E
+    assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, 1, 1024, _lib.call_pattern(2, 1, 0, 10), 1.0, None) == E
+    assert b"first_chunk" in lib.ps_last_error()
+    assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, 1, 1024, _lib.call_pattern(2, 0, 1000, 25), 1.0, None) == E
+    assert b"does not fit a chunk" in lib.ps_last_error()
     lib.ps_adam_destroy(88)
 
 
