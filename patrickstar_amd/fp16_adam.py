@@ -540,6 +540,9 @@ class FP16Adam(torch.optim.Optimizer):
             self._trainable_changed(trainable_now)
         hyper = self._hyper()
         if hyper is None:
+            # nothing is trainable: the reference still runs its scale update (fp16_cpu_adam.py:549-558,624-625)
+            if self._dynamic:
+                self.loss_scaler.update_scale(None, operator_calls=0)
             return loss
         lr, (beta1, beta2), eps, weight_decay = hyper
         table, n_dev, host_positions = self._tables or self._build_tables()
