@@ -1,0 +1,144 @@
+"""Seeded randomised parity of the fused steps under random operator-call patterns.
+
+Every case draws a chunk list (1 to 70 chunks, so that some lists need two launches), cuts every chunk into tensors at random
+places, visits the tensors in a random order (the first of them is the step's first operator call, wherever it lies), picks
+hyper-parameters, decay form, clamp, scale kind and base misalignments, sprinkles zeros, subnormals and huge values over
+the state, and runs a few steps (consecutive and jumping step numbers; device-decided cases get poisoned iterations).
+Bar: bit-exact against the step-level oracle, which makes one operator call per tensor."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import patrickstar_amd as ps
+from patrickstar_amd import _lib
+from test_gpu_call_pattern import RawChunks
+from test_gpu_tensor_list import PermutedLayout
+
+pytestmark = pytest.mark.gpu
+
+
+def _sprinkle(a, rng, kinds):
+    idx = rng.integers(0, a.size, max(1, a.size // 50))
+    a[idx] = rng.choice(kinds, idx.size).astype(a.dtype)
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_chunk_lists_under_random_call_patterns(seed):
+    lib = _lib.load()
+    rng = np.random.default_rng(seed)
+    for case in range(40):
+        C = int(rng.choice([1, 2, 3, 5, 65, 70])) if rng.random() < 0.8 else int(rng.integers(1, 9))
+        n = int(rng.choice([1, 2, 255, 256, 257, 511, 1024, int(rng.integers(1, 2500))]))
+        offs = tuple(int(x) for x in rng.integers(0, 4, 4)) if rng.random() < 0.5 else (0, 0, 0, 0)
+        R = RawChunks(C, n, seed=int(rng.integers(1 << 30)), offs=offs)
+        for c, bufs in zip(R.host, R.dev):
+            if rng.random() < 0.5:
+                _sprinkle(c["p32"], rng, [0.0, -0.0, 1e-41, -3e-42, 1e30, -1e-30, 65504.0, 1.0])
+                _sprinkle(c["m"], rng, [0.0, 1e-42, -1e-41, 1e20, -1e-25])
+                _sprinkle(c["v"], rng, [0.0, 1e-44, 1e-38, 1e25, 3e-41])
+                for key, t, off in zip(("p32", "m", "v"), bufs, R.offs):
+                    t[off:off + n].copy_(torch.from_numpy(c[key]))
+        tensors = []
+        for ci in range(C):
+            cuts = sorted(set([0, n] + [int(x) for x in rng.integers(0, n + 1, int(rng.integers(0, 4)))]))
+            tensors += [(ci, a, b - a) for a, b in zip(cuts[:-1], cuts[1:])]
+        tensors = [tensors[i] for i in rng.permutation(len(tensors))]
+        lr, eps = float(rng.choice([1e-3, 1e-4, 0.1])), float(rng.choice([1e-8, 1e-6, 1e-3]))
+        b1, b2 = float(rng.choice([0.9, 0.0, 0.5])), float(rng.choice([0.999, 0.9, 0.99]))
+        wd, adamw = float(rng.choice([0.0, 0.01, 0.3])), bool(rng.integers(0, 2))
+        gated = bool(rng.integers(0, 2))
+        clip = float(rng.choice([-1, -1, 0.5, 1e-3]))
+        oid = 5000 + case
+        _lib.check(lib.ps_adam_create(oid, lr, b1, b2, eps, wd, int(adamw), 0), "create")
+        if clip > 0:
+            _lib.check(lib.ps_adam_set_grad_clamp(oid, clip), "clamp")
+        calls = _lib.call_pattern(len(tensors), *tensors[0])
+        what = (f"seed {seed} case {case}: C={C} n={n} offs={offs} tensors={len(tensors)} first={tensors[0]} lr={lr} eps={eps} "
+                f"betas=({b1},{b2}) wd={wd} adamw={adamw} gated={gated} clip={clip}")
+        stream = _lib.current_stream_handle()
+        if gated:
+            kw = dict(init_scale=float(rng.choice([2.0**10, 1000.0, 3.0])), scale_factor=2, scale_window=int(rng.integers(1, 4)), min_scale=1)
+            scaler = ps.DynamicLossScaler(**kw)
+            scaler.materialize("cuda:0", betas=(b1, b2))
+            oscaler = oracle.ScalerOracle(**kw)
+            oopt = oracle.OptimizerStepOracle(R.host, oscaler, lr=lr, betas=(b1, b2), eps=eps, weight_decay=wd, use_adamw=adamw,
+                                              tensors=tensors, gradient_clipping=clip)
+            for it in range(int(rng.integers(2, 6))):
+                poison = (int(rng.integers(0, C)), int(rng.integers(0, n))) if rng.random() < 0.25 else None
+                R.new_grads(rng, float(oscaler.loss_scale), poison=poison)
+                _lib.check(lib.ps_overflow_scan_chunks(R.table, C, n, scaler.state_ptr, stream), "scan")
+                _lib.check(lib.ps_adam_step_chunks_gated(oid, lr, eps, wd, 1, R.table, C, n, calls, scaler.state_ptr, stream), "gated")
+                scaler.update_scale(None, operator_calls=len(tensors))
+                oopt.check_overflow()
+                assert oopt.step() == (poison is not None), what
+                R.compare(f"{what} iteration {it}")
+                assert scaler.loss_scale == oscaler.loss_scale, what
+        else:
+            scale = [None, 8.0, 2.0**12, 1000.0, 12345.678][int(rng.integers(0, 5))]
+            oopt = oracle.OptimizerStepOracle(R.host, oracle.StaticScalerOracle(scale) if scale else None, lr=lr, betas=(b1, b2), eps=eps,
+                                              weight_decay=wd, use_adamw=adamw, tensors=tensors, gradient_clipping=clip)
+            step = 0
+            for _ in range(int(rng.integers(2, 6))):
+                step = step + 1 if rng.random() < 0.7 else int(rng.integers(1, 3000))
+                R.new_grads(rng, scale or 1.0)
+                oopt.step_count = step - 1
+                _lib.check(lib.ps_adam_step_chunks(oid, step, lr, b1, b2, eps, wd, 1, R.table, C, n, calls, scale if scale else -1.0, stream),
+                           "chunks")
+                oopt.step()
+                R.compare(f"{what} step {step}")
+        lib.ps_adam_destroy(oid)
+
+
+@pytest.mark.parametrize("seed", [4, 5])
+def test_tensor_lists_in_any_order_and_over_two_calls(seed):
+    """The tensor-list entry point with tensors of random lengths (zero and one element included) whose momentum and
+    variance sit at other element phases than the parameters, listed in another order than the reference visits them and
+    split over one or two calls under one call pattern."""
+    lib = _lib.load()
+    rng = np.random.default_rng(seed)
+    pool = [1, 2, 3, 63, 64, 255, 256, 257, 300, 1000, 4099, 65536, 70001]
+    for case in range(25):
+        k = int(rng.choice([7, 8, 20, 64, 65, 130]))
+        sizes = [int(rng.choice(pool)) if rng.random() < 0.8 else int(rng.integers(1, 5000)) for _ in range(k)]
+        scale = [None, 8.0, 2.0**12, 1000.0][int(rng.integers(0, 4))]
+        L = PermutedLayout(sizes, seed=int(rng.integers(1 << 30)), scale=scale or 1.0)
+        lr, eps, wd = float(rng.choice([1e-3, 1e-4])), float(rng.choice([1e-8, 1e-6])), float(rng.choice([0.0, 0.01]))
+        adamw, b1, b2 = bool(rng.integers(0, 2)), 0.9, float(rng.choice([0.999, 0.95]))
+        torch_arith = rng.random() < 0.3
+        oid = 7000 + case
+        _lib.check(lib.ps_adam_create(oid, lr, b1, b2, eps, wd, int(adamw), 0), "create")
+        if torch_arith:
+            _lib.check(lib.ps_adam_set_arithmetic(oid, _lib.PS_ARITH_TORCH), "arithmetic")
+        ref_order = [int(i) for i in rng.permutation(k)]  # the order of the reference's operator calls
+        listed = [int(i) for i in rng.permutation(k)]     # the order of the list(s) handed over
+        cut = int(rng.integers(1, k)) if rng.random() < 0.5 else k
+        first = ref_order[0]
+        parts = sorted([part for part in (listed[:cut], listed[cut:]) if part], key=lambda part: first not in part)
+        native = oracle.AdamOracle(lr, b1, b2, eps, wd, adamw)
+        what = f"seed {seed} case {case}: k={k} scale={scale} torch={torch_arith} adamw={adamw} wd={wd} parts={[len(x) for x in parts]}"
+        step = 0
+        for it in range(int(rng.integers(1, 4))):
+            step = step + 1 if rng.random() < 0.7 else int(rng.integers(1, 3000))
+            if it:
+                L.new_grads(rng, scale or 1.0)
+            for part in parts:
+                rows = _lib.chunk_array([[L.table[i].param_fp32, L.table[i].exp_avg, L.table[i].exp_avg_sq, L.table[i].param_fp16] for i in part])
+                numels = (ctypes.c_size_t * len(part))(*[sizes[i] for i in part])
+                pattern = _lib.call_pattern(k, part.index(first), 0, sizes[first]) if first in part else _lib.call_pattern(k, 0, 0, 0)
+                _lib.check(lib.ps_adam_step_tensors(oid, step, lr, b1, b2, eps, wd, 1, rows, numels, len(part), pattern,
+                                                    float(scale) if scale else -1.0, None, _lib.current_stream_handle()), what)
+            torch.cuda.synchronize()
+            for i in ref_order:
+                p, h, m, v = L.views(i)
+                pc, mc, vc, hc = p.copy(), m.copy(), v.copy(), h.copy()
+                if torch_arith:
+                    oracle.torch_formula_update(pc, hc, mc, vc, step, lr, b1, b2, eps, wd, adamw, scale)
+                else:
+                    native.update(step, lr, b1, b2, eps, wd, True, pc, hc, mc, vc, float(scale) if scale else -1.0)
+                p[...], m[...], v[...] = pc, mc, vc
+                h[...] = oracle.cast_fp32_to_fp16(np.ascontiguousarray(pc))
+            L.compare(f"{what} step {step}")
+        lib.ps_adam_destroy(oid)
