@@ -14,6 +14,7 @@ import torch
 import oracle
 import patrickstar_amd as ps
 from patrickstar_amd import _lib
+from _harness import assert_bits_equal
 from test_gpu_call_pattern import RawChunks
 from test_gpu_tensor_list import PermutedLayout
 
@@ -142,3 +143,93 @@ def test_tensor_lists_in_any_order_and_over_two_calls(seed):
                 h[...] = oracle.cast_fp32_to_fp16(np.ascontiguousarray(pc))
             L.compare(f"{what} step {step}")
         lib.ps_adam_destroy(oid)
+
+
+@pytest.mark.parametrize("seed", [6, 7])
+def test_engine_with_random_frozen_sets_and_host_placements(seed):
+    """initialize_engine over small random MLPs: layer widths (some odd), chunk size (one to several layers per chunk),
+    frozen parameters, which positions keep their optimizer state in pinned host memory, arithmetic, optimizer type and
+    scaler kind are drawn per case; dynamic cases overflow now and then.  Whatever combination of entry points one
+    step turns into (whole chunks, tensor list, streamed chunks, staged tensor lists), every payload matches the oracle
+    that makes one operator call per trainable tensor under the same placement."""
+    from _harness import tensor_spans
+
+    def snap(t):
+        return t.detach().to("cpu", copy=True).numpy().copy()
+
+    rng = np.random.default_rng(seed)
+    seen = set()
+    for case in range(30):
+        widths = [int(rng.choice([8, 12, 16, 24, 33])) for _ in range(int(rng.integers(3, 8)))]
+        with_gain = rng.random() < 0.5
+
+        class Net(torch.nn.Module):
+            def __init__(self):
+                super().__init__()
+                self.layers = torch.nn.ModuleList([torch.nn.Linear(a, b) for a, b in zip(widths[:-1], widths[1:])])
+                if with_gain:
+                    self.gain = torch.nn.Parameter(torch.ones(widths[-1]))
+
+            def forward(self, x):
+                for layer in self.layers:
+                    x = torch.tanh(layer(x))
+                if with_gain:
+                    x = x * self.gain
+                return x.float().pow(2).mean()
+
+        names = [n for n, _ in Net().named_parameters()]
+        per_module = max(a * b + b for a, b in zip(widths[:-1], widths[1:]))
+        chunk = int(per_module * rng.choice([1.0, 1.3, 2.2, 3.5])) + int(rng.integers(0, 20))
+        frozen = set(n for n in names if rng.random() < 0.3)
+        if len(frozen) == len(names):
+            frozen.pop()
+        arithmetic = "operator" if rng.random() < 0.6 else "torch"
+        loss_scale = int(rng.choice([0, 64]))
+        optim_type = "AdamW" if rng.random() < 0.5 else "Adam"
+        host_share, host_draw = float(rng.choice([0.0, 0.3, 0.6, 1.0])), rng.random(64)
+
+        def model_func():
+            torch.manual_seed(1000 * seed + case)
+            m = Net()
+            for n, p in m.named_parameters():
+                if n in frozen:
+                    p.requires_grad_(False)
+            return m
+
+        config = {
+            "optimizer": {"type": optim_type, "params": {"lr": 1e-3, "betas": (0.9, 0.999), "eps": 1e-8, "weight_decay": 0.05,
+                                                         "arithmetic": arithmetic}},
+            "fp16": {"enabled": True, "loss_scale": loss_scale, "initial_scale_power": 7, "loss_scale_window": 3, "hysteresis": 2, "min_loss_scale": 1},
+            "default_chunk_size": chunk,
+            "client": {"host_chunk_policy": lambda position: host_draw[position % 64] < host_share},
+        }
+        what = f"seed {seed} case {case}: widths={widths} chunk={chunk} frozen={sorted(frozen)} {arithmetic} {optim_type} loss_scale={loss_scale}"
+        engine, optimizer = ps.initialize_engine(model_func=model_func, local_rank=0, config=config)
+        client = engine.client
+        cl, pos = client.chunk_list, client.positions()
+        host = [i for i, q in enumerate(pos) if q.on_host]
+        mirror = [{"p32": snap(cl[q.fp32].payload), "m": snap(cl[q.exp_avg].payload), "v": snap(cl[q.exp_avg_sq].payload),
+                   "p16": snap(cl[q.fp16].payload)} for q in pos]
+        oscaler = oracle.scaler_from_config(config["fp16"])
+        oopt = oracle.OptimizerStepOracle(mirror, oscaler, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.05,
+                                          use_adamw=(optim_type == "AdamW"), tensors=tensor_spans(client, optimizer),
+                                          arithmetic=arithmetic, operator_chunks=host)
+        x = torch.randn(8, widths[0], device="cuda").half()
+        for it in range(4):
+            blow_up = loss_scale == 0 and rng.random() < 0.25
+            loss = engine(x * (6e4 if blow_up else 1.0))
+            engine.backward(loss)
+            for q, c in zip(pos, mirror):
+                c["p16"][...] = snap(cl[q.fp16].payload)
+            optimizer.step()
+            torch.cuda.synchronize()
+            oopt.check_overflow()
+            oopt.step()
+            for i, (q, c) in enumerate(zip(pos, mirror)):
+                for key, cid in (("p32", q.fp32), ("m", q.exp_avg), ("v", q.exp_avg_sq), ("p16", q.fp16)):
+                    assert_bits_equal(snap(cl[cid].payload), c[key], f"{what} host={host} iteration {it} position {i} {key}")
+            assert optimizer.loss_scaler.loss_scale == oscaler.loss_scale, what
+        seen.update([s[0] for s in optimizer._stages] if optimizer._stages else
+                    ["one tensor list" if optimizer._tensor_table else "whole chunks"])
+    # the draw covers every way a step can be put together
+    assert {"tensors", "stream", "staged", "one tensor list", "whole chunks"} <= seen, seen
