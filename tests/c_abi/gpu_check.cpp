@@ -301,7 +301,83 @@ int main()
         return 6;
     }
     PS_OK(ps_adam_destroy(33));
+
+    // ---- tensor list: the chunks cut into tensors (two per chunk, the second at an odd element offset), listed in
+    //      another order than the reference visits them and handed over in two calls under one call pattern; the
+    //      reference's first call is the SECOND tensor of chunk 1
+    {
+        const size_t cut = 256 * 5 + 3;
+        struct Span { int chunk; size_t off, len; };
+        const Span order[6] = {{1, cut, n - cut}, {0, 0, cut}, {2, 0, cut}, {0, cut, n - cut}, {1, 0, cut}, {2, cut, n - cut}};  // reference order
+        const int listed_a[2] = {3, 0}, listed_b[4] = {5, 4, 2, 1};  // indices into order[]; the first call is listed_a[1]
+        PS_OK(ps_adam_create(34, lr, b1, b2, eps, wd, 1, 0));
+        oracle_adam_init(&native, lr, b1, b2, eps, wd, 1);
+        for (int c = 0; c < C; ++c)
+            if (upload(host[c], dev[c], n)) return 2;
+        for (uint64_t step = 1; step < 4; ++step) {
+            for (int c = 0; c < C; ++c) {
+                new_gradients(rng, host[c], scale);
+                if (upload(host[c], dev[c], n)) return 2;
+            }
+            auto describe = [&](const int* idx, int count, ps_chunk* rows, size_t* lens) {
+                for (int k = 0; k < count; ++k) {
+                    const Span& t = order[idx[k]];
+                    rows[k].param_fp32 = dev[t.chunk].p + t.off;
+                    rows[k].exp_avg = dev[t.chunk].m + t.off;
+                    rows[k].exp_avg_sq = dev[t.chunk].v + t.off;
+                    rows[k].param_fp16 = dev[t.chunk].h + t.off;
+                    lens[k] = t.len;
+                }
+            };
+            ps_chunk rows_a[2], rows_b[4];
+            size_t len_a[2], len_b[4];
+            describe(listed_a, 2, rows_a, len_a);
+            describe(listed_b, 4, rows_b, len_b);
+            const ps_call_pattern first_here = {6, 1, 0, len_a[1]}, first_elsewhere = {6, 0, 0, 0};
+            PS_OK(ps_adam_step_tensors(34, step, lr, b1, b2, eps, wd, 1, rows_a, len_a, 2, &first_here, scale, NULL, stream));
+            PS_OK(ps_adam_step_tensors(34, step, lr, b1, b2, eps, wd, 1, rows_b, len_b, 4, &first_elsewhere, scale, NULL, stream));
+            HIP_OK(hipStreamSynchronize(stream));
+            for (const Span& t : order) {
+                oracle_adam_advance(&native, step, b1, b2);
+                oracle_adam_set(&native, lr, eps, wd, 1);
+                HostChunk& hc = host[t.chunk];
+                if (t.len && oracle_adam_span(&native, hc.p.data() + t.off, hc.h.data() + t.off, 1, hc.m.data() + t.off,
+                                              hc.v.data() + t.off, t.len, (float)scale, 0) <= 0)
+                    return 5;
+            }
+            for (int c = 0; c < C; ++c) {
+                oracle_cast_f32_to_f16(host[c].p.data(), host[c].h.data(), n);
+                if (int rc = compare(host[c], dev[c], n, "tensor-list step", c)) return rc;
+            }
+        }
+        PS_OK(ps_adam_destroy(34));
+    }
+
+    // ---- the probe that allocates nothing: same answer as the probe with a caller-side state
+    {
+        uint32_t* d_flag = nullptr;
+        HIP_OK(hipMalloc((void**)&d_flag, sizeof(uint32_t)));
+        HIP_OK(hipMemsetAsync(d_flag, 0, sizeof(uint32_t), stream));
+        uint32_t flag = 7;
+        PS_OK(ps_overflow_scan_chunks_noalloc(table, C, n, d_flag, stream));
+        HIP_OK(hipMemcpyAsync(&flag, d_flag, sizeof(flag), hipMemcpyDeviceToHost, stream));
+        HIP_OK(hipStreamSynchronize(stream));
+        if (flag != 0) {
+            fprintf(stderr, "the allocation-free probe saw an inf / nan in finite payloads\n");
+            return 7;
+        }
+        const uint16_t nan16 = 0x7E00;
+        HIP_OK(hipMemcpyAsync(dev[C - 1].h + (n - 1), &nan16, sizeof(nan16), hipMemcpyHostToDevice, stream));
+        PS_OK(ps_overflow_scan_chunks_noalloc(table, C, n, d_flag, stream));
+        HIP_OK(hipMemcpyAsync(&flag, d_flag, sizeof(flag), hipMemcpyDeviceToHost, stream));
+        HIP_OK(hipStreamSynchronize(stream));
+        if (flag != 1) {
+            fprintf(stderr, "the allocation-free probe missed a nan in the last element of the last chunk\n");
+            return 7;
+        }
+        HIP_OK(hipFree(d_flag));
+    }
     printf("c abi gpu check ok: 3 host-decided and 8 device-decided steps (2 skipped), 3 steps with host-resident chunks, "
-           "over %d x %zu elements\n", C, n);
+           "3 tensor-list steps in two calls each, the allocation-free probe, over %d x %zu elements\n", C, n);
     return 0;
 }
