@@ -22,8 +22,10 @@
  *     (-hipError_t for a HIP runtime error, PS_ERR_* otherwise);
  *     ps_last_error() gives the text.  Nothing throws across this boundary.
  *   - vector (16-byte) accesses are used when the four base addresses of a
- *     chunk / tensor are 16-byte aligned; otherwise a slower element-wise path
- *     produces the same bits.
+ *     chunk / tensor are 16-byte aligned, and also when only momentum and
+ *     variance sit at another element phase than the two parameter lists
+ *     (their 16-byte accesses then go to 4-byte-aligned addresses); otherwise a
+ *     slower element-wise path produces the same bits.
  */
 #ifndef PS_ADAM_H
 #define PS_ADAM_H
