@@ -496,3 +496,83 @@ def test_placement_is_decided_from_the_free_hbm_when_the_model_is_registered():
     c = client_with()
     c.plan_placement()
     assert c.host_chunk_policy is None
+
+
+@pytest.mark.skipif(not os.path.exists(_lib.LIB_PATH), reason="HIP library not built")
+def test_layout_invariants_hold_for_random_models():
+    """Random stacks of Linear layers (with and without bias, some with a parameter of the parent's own) and random chunk
+    sizes: every parameter gets a span inside one chunk, spans of a chunk do not overlap and appear in insertion order,
+    the parameters of one module share a chunk (first-fit by module, core/client.py:246-280), the fp32 master and
+    both optimizer states of a parameter sit at the parameter's own chunk position and offset, payloads start with the
+    initial values and are zero behind the last tensor, and what FP16Adam hands to the library names every trainable
+    tensor exactly once."""
+    from hypothesis import given, settings, strategies as st
+
+    @settings(max_examples=40, deadline=None)
+    @given(widths=st.lists(st.integers(1, 9), min_size=2, max_size=7), slack=st.integers(0, 40), biases=st.integers(0, 127),
+           own=st.booleans(), frozen=st.integers(0, 1 << 14))
+    def check(widths, slack, biases, own, frozen):
+        ran.append(1)
+
+        class Net(torch.nn.Module):
+            def __init__(self):
+                super().__init__()
+                self.layers = torch.nn.ModuleList(
+                    [torch.nn.Linear(a, b, bias=bool((biases >> i) & 1)) for i, (a, b) in enumerate(zip(widths[:-1], widths[1:]))])
+                if own:
+                    self.own = torch.nn.Parameter(torch.arange(3.0))
+
+        torch.manual_seed(0)
+        model = Net()
+        params = list(model.parameters())
+        for i, p in enumerate(params):
+            if (frozen >> i) & 1 and i:  # the first parameter stays trainable
+                p.requires_grad_(False)
+        chunk = max(sum(q.numel() for q in layer.parameters()) for layer in model.layers) + slack
+        chunk = max(chunk, 3)
+        init = {n: p.detach().clone() for n, p in model.named_parameters()}
+        client = ps.PatrickStarClient(0, chunk, device="cpu")
+        client.register_model(model)
+        opt = ps.FP16Adam(client, model.parameters(), lr=1e-3)
+        idx = client.chunk_tensor_index
+        info = lambda p: idx.get_tensor_info(p.ps_attr.data_id())
+        position_of = {q.fp16: i for i, q in enumerate(client.positions())}
+        # spans: inside the chunk, disjoint, in insertion order
+        for q in client.positions():
+            end = 0
+            for t in idx.generate_tensor_info_in_order(q.fp16):
+                assert t.start_offset >= end and t.start_offset + t.numel <= chunk
+                end = t.start_offset + t.numel
+            assert not client.chunk_list[q.fp16].payload[end:].any() and not client.chunk_list[q.fp32].payload[end:].any()
+        for layer in model.layers:
+            assert len({info(p).chunk_id for p in layer.parameters()}) == 1
+        for name, p in model.named_parameters():
+            assert torch.equal(client.access_data(p), init[name].half())
+            master = client.param_fp16_to_param_fp32_map[p]
+            assert torch.equal(client.access_data(master), init[name])
+            pos = client.positions()[position_of[info(p).chunk_id]]
+            for shadow, cid in ((master, pos.fp32), (dict.__getitem__(opt.state[p], "exp_avg"), pos.exp_avg),
+                                (dict.__getitem__(opt.state[p], "exp_avg_sq"), pos.exp_avg_sq)):
+                assert (info(shadow).chunk_id, info(shadow).start_offset, info(shadow).numel) == (cid, info(p).start_offset, p.numel())
+        # what one step covers: every trainable element exactly once, no frozen one
+        table, n_dev, host_positions = opt._build_tables()
+        assert not host_positions
+        trainable = [p for p in params if p.requires_grad]
+        if opt._tensor_table is not None:
+            rows, numels, n = opt._tensor_table
+            assert n == len(trainable) and list(numels) == [p.numel() for p in trainable]
+            assert [rows[i].param_fp16 for i in range(n)] == [client.access_data(p).data_ptr() for p in trainable]
+        else:
+            live = {info(p).chunk_id for p in trainable}
+            assert n_dev == len(live)
+            for cid in live:  # a whole-chunk step is only taken when nothing frozen shares a live chunk
+                assert all(t.param.requires_grad for t in idx.generate_tensor_info_in_order(cid))
+        assert opt._operator_calls == len(trainable)
+        first = opt._calls._obj
+        live_positions = [q for q in client.positions() if any(t.param.requires_grad for t in idx.generate_tensor_info_in_order(q.fp16))]
+        assert live_positions[first.first_chunk].fp16 == info(trainable[0]).chunk_id
+        assert (first.n_calls, first.first_offset, first.first_numel) == (len(trainable), info(trainable[0]).start_offset, trainable[0].numel())
+
+    ran = []
+    check()
+    assert len(ran) >= 20
