@@ -315,9 +315,9 @@ def run_streamed(args, with_cpu_baseline=True):
     def kernels():
         s = _lib.current_stream_handle()
         if res_rows:
-            lib.ps_adam_step_chunks(991, 1, 1e-4, 0.9, 0.999, 1e-8, 0.01, 1, res, len(res_rows), N, None, 4096.0, s)
+            lib.ps_adam_step_chunks(991, 1, 1e-4, 0.9, 0.999, 1e-8, 0.01, 1, res, len(res_rows), N, None, None, 4096.0, s)
         for _ in host_pos:
-            lib.ps_adam_step_chunks(991, 1, 1e-4, 0.9, 0.999, 1e-8, 0.01, 1, one, 1, N, None, 4096.0, s)
+            lib.ps_adam_step_chunks(991, 1, 1e-4, 0.9, 0.999, 1e-8, 0.01, 1, one, 1, N, None, None, 4096.0, s)
 
     t_h2d, t_d2h = timed(h2d), timed(d2h)
     h2d()  # leave finite data in the slot for the kernel leg
@@ -558,8 +558,8 @@ def dynamic_leg(cfg, steps, warmup):
 
     def step():
         s = _lib.current_stream_handle()
-        _lib.check(lib.ps_overflow_scan_chunks(table, n_dev, cfg.N, scaler.state_ptr, s), "scan")
-        _lib.check(lib.ps_adam_step_chunks_gated(992, HYPER["lr"], HYPER["eps"], HYPER["weight_decay"], 1, table, n_dev, cfg.N,
+        _lib.check(lib.ps_overflow_scan_chunks(table, n_dev, cfg.N, None, scaler.state_ptr, s), "scan")
+        _lib.check(lib.ps_adam_step_chunks_gated(992, HYPER["lr"], HYPER["eps"], HYPER["weight_decay"], 1, table, n_dev, cfg.N, None,
                                                  calls, scaler.state_ptr, s), "gated")
         scaler.update_scale(None, operator_calls=cfg.C)
 
@@ -642,19 +642,31 @@ def tensor_list_leg(cfg, steps, warmup):
     return out
 
 
+PROBE_SOURCE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "bench_kernels", "ps_stream_probe.hip")
+PROBE_PATH = os.path.join(os.path.dirname(PROBE_SOURCE), "libps_stream_probe.so")
+
+
+def build_stream_probe(force=False):
+    """Compile the plain streaming kernels `--mode ceiling` measures the memory system with (a measurement instrument
+    of this script, not part of the optimizer library) into bench_kernels/libps_stream_probe.so, unless already there."""
+    if force or not os.path.exists(PROBE_PATH) or os.path.getmtime(PROBE_PATH) < os.path.getmtime(PROBE_SOURCE):
+        from patrickstar_amd.build import compile_shared
+
+        compile_shared([PROBE_SOURCE], PROBE_PATH)
+    return PROBE_PATH
+
+
 def ceiling(args):
     """Streaming ceilings on the buffers of the 1.5 B configuration: plain kernels of libps_stream_probe.so, swept over
     their launch shape (tiles per workgroup x resident-workgroup cap), beside the library's own kernels.  One JSON line;
     every entry is a median over `--steps` launches."""
+    probe_path = build_stream_probe()  # before anything touches the GPU: the compiler runs as a child process
     import torch
 
     import patrickstar_amd as ps
     from patrickstar_amd import _lib
-    from patrickstar_amd.build import PROBE_PATH
 
-    if not os.path.exists(PROBE_PATH):
-        sys.exit(f"bench.py: {PROBE_PATH} not found: build it with `python -m patrickstar_amd.build`")
-    probe = ctypes.CDLL(PROBE_PATH)
+    probe = ctypes.CDLL(probe_path)
     vp, sz, i32 = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
     probe.ps_probe_read.argtypes = [vp, sz, vp, i32, i32, vp]
     probe.ps_probe_write.argtypes = [vp, sz, ctypes.c_float, i32, i32, vp]
@@ -750,7 +762,7 @@ def ceiling(args):
             h[c * cfg.N:(c + 1) * cfg.N].copy_(half_chunk)
 
     refill_fp16()
-    results["library_scan_chunks"] = entry(measure(lambda: lib.ps_overflow_scan_chunks(table, n_dev, cfg.N, state.state_ptr, s())), 2 * n, 1, 0)
+    results["library_scan_chunks"] = entry(measure(lambda: lib.ps_overflow_scan_chunks(table, n_dev, cfg.N, None, state.state_ptr, s())), 2 * n, 1, 0)
     results["library_cast_fp32_to_fp16"] = entry(measure(lambda: lib.ps_cast_fp32_to_fp16(p.data_ptr(), h.data_ptr(), n, s())), 6 * n, 1, 1)
     results["library_restore_fp16_chunks"] = entry(measure(lambda: lib.ps_restore_fp16_chunks(table, n_dev, cfg.N, None, s())), 6 * n, 1, 1)
     refill_fp16()

@@ -9,8 +9,8 @@
 //   - one read stream copied into one write stream (1 : 1),
 //   - the optimizer step's own access pattern with its arithmetic removed: four arrays (three
 //     binary32, one binary16) read and written in place, 28 bytes per element,
-// on the same buffers the step runs on.  Built into libps_stream_probe.so by patrickstar_amd/build.py;
-// nothing in the package loads it.
+// on the same buffers the step runs on.  Built into bench_kernels/libps_stream_probe.so by bench.py
+// (build_stream_probe) when `--mode ceiling` first needs it; nothing in the package loads it.
 #include <hip/hip_runtime.h>
 
 #include <cstddef>

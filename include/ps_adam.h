@@ -37,7 +37,7 @@
 extern "C" {
 #endif
 
-#define PS_ABI_VERSION 4
+#define PS_ABI_VERSION 5
 
 #define PS_ERR_BAD_ARG (-10001)     /* null pointer, negative count, unknown mode */
 #define PS_ERR_UNKNOWN_ID (-10002)  /* optimizer id was never created (the reference dereferences null here) */
@@ -67,7 +67,7 @@ typedef struct ps_chunk {
  * (fp16_cpu_adam.py:279-285) and the Adam step counter with its float
  * beta^t running products (cpu_adam.h:143-162).  It lives in device memory
  * so that "was there an overflow -> skip, restore, halve" needs no host
- * round trip.  192 bytes, 16-byte aligned.
+ * round trip.  256 bytes, 16-byte aligned.
  */
 typedef struct ps_step_state {
     double cur_scale;           /* loss_scale; Python float semantics (binary64) */
@@ -86,8 +86,8 @@ typedef struct ps_step_state {
     int32_t min_is_int;
     uint32_t overflow;          /* sticky flag of the step being assembled (0/1) */
     uint32_t last_skipped;      /* what the latest ps_scaler_update decided */
-    float beta1;
-    float beta2;
+    float beta1;                /* the betas of the NEXT step over whole chunk lists (the device-decided entry points */
+    float beta2;                /* take none); ps_state_seed_step sets them */
     float beta1_t_next;         /* beta1^t that the FIRST operator call of step t = adam_step + 1 uses */
     float beta2_t_next;
     uint32_t reserved[4];
@@ -107,6 +107,17 @@ typedef struct ps_step_state {
     float beta1_t_rest;         /* (float)pow((double)beta, adam_step + 1): what every operator call */
     float beta2_t_rest;         /* of step adam_step + 1 after the first one uses */
     uint32_t reserved2[2];
+    float operator_beta1;       /* its _betta1 / _betta2: the betas of its latest call (create_adam's before any) */
+    float operator_beta2;
+    /* What the operator object holds after the last call of a step queued by ps_adam_step_tensors_each (every
+     * tensor its own step number and betas).  ps_scaler_update adopts it if the step turns out clean and drops
+     * it if the step is skipped.  pending_operator_step == 0: nothing is pending. */
+    int64_t pending_operator_step;
+    float pending_beta1_t;
+    float pending_beta2_t;
+    float pending_beta1;
+    float pending_beta2;
+    uint32_t reserved3[8];
 } ps_step_state;
 
 /*
@@ -201,9 +212,21 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
 
 /* One fused pass over a whole chunk list: for every element of every chunk
  * read fp16 grad, fp32 param, m, v once; write fp32 param, m, v and the fp16
- * param (over the grad) once: 28 bytes per element.  Host scalar state is
- * advanced ONCE for the call (the chunk list is one flat tensor for the
- * operator).  chunks is a host array of n_chunks descriptors.
+ * param (over the grad) once: 28 bytes per element.  chunks is a host array of
+ * n_chunks descriptors.
+ *   calls       how the reference would have cut the step into operator calls (ps_call_pattern).
+ *               NULL: the whole list is one flat tensor for the operator and its host scalar state
+ *               (cpu_adam.h:143-162) advances once; with n_calls >= 2 it is taken through the first
+ *               call and one further call, from which on the object no longer moves.
+ *   used_numel  NULL: every chunk is updated over all chunk_numel elements.  Else a host array of
+ *               n_chunks lengths: chunk i holds tensors in its first used_numel[i] elements only and
+ *               ZEROS behind them in all four payloads (the reference allocates payloads with
+ *               torch.zeros and only ever writes tensor spans, patrickstar/core/chunk_data.py:148-154).
+ *               Zeros are a fixed point of the update (g = m = v = p = 0 gives m = v = 0 and
+ *               p = 0 under L2 and decoupled decay alike, fp16 0), so the pass leaves the tail alone:
+ *               same bits, fewer bytes.  The one case where the reference's arithmetic does not keep
+ *               the zeros (a denominator of 0: eps == 0, or a non-finite step size: it writes NaNs into
+ *               the padding) is detected and the tail is then computed like everything else.
  * Hyper-parameters and loss_scale are the Python numbers (binary64).  The operator's
  * arithmetic narrows them to float first, as the pybind signature of adam_update does
  * (cpu_adam.cpp:700-712); the torch arithmetic uses them as torch does.
@@ -211,18 +234,21 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
 int ps_adam_step_chunks(int optimizer_id, size_t step, double lr, double beta1, double beta2,
                         double epsilon, double weight_decay, int bias_correction,
                         const ps_chunk* chunks, int n_chunks, size_t chunk_numel,
-                        const ps_call_pattern* calls, double loss_scale, ps_stream_t stream);
+                        const size_t* used_numel, const ps_call_pattern* calls, double loss_scale,
+                        ps_stream_t stream);
 
 /* Same pass, decided on the device: if d_state->overflow is set, every chunk's
  * fp16 payload is restored from the fp32 master copy (fp16_cpu_adam.py:298-309)
  * and nothing else changes; otherwise the Adam update runs with
  * loss_scale = d_state->cur_scale and t = d_state->adam_step + 1 (beta^t of the first and of the
- * later operator calls, or the binary64 bias corrections of the torch arithmetic, from d_state).
+ * later operator calls, or the binary64 bias corrections of the torch arithmetic, from d_state; the
+ * betas are d_state's: ps_state_seed_step changes them).  used_numel as for ps_adam_step_chunks.
  * Follow with ps_scaler_update(..., PS_FLAG_FROM_DEVICE, ..., calls ? calls->n_calls : 1). */
 int ps_adam_step_chunks_gated(int optimizer_id, double lr, double epsilon, double weight_decay,
                               int bias_correction, const ps_chunk* chunks, int n_chunks,
-                              size_t chunk_numel, const ps_call_pattern* calls,
-                              const ps_step_state* d_state, ps_stream_t stream);
+                              size_t chunk_numel, const size_t* used_numel,
+                              const ps_call_pattern* calls, const ps_step_state* d_state,
+                              ps_stream_t stream);
 
 /* The per-tensor loop of FP16Adam.fp16_chunk_adam_ops (fp16_cpu_adam.py:336-468) as ONE call, for chunk layouts
  * in which a parameter's exp_avg / exp_avg_sq do not sit at the parameter's own offset inside their chunks (the
@@ -247,6 +273,50 @@ int ps_adam_step_tensors(int optimizer_id, size_t step, double lr, double beta1,
                          const ps_chunk* tensors, const size_t* numels, int n_tensors,
                          const ps_call_pattern* calls, double loss_scale, const ps_step_state* d_state,
                          ps_stream_t stream);
+
+/* One adam_update call of the reference's per-tensor loop with the numbers of ITS tensor: FP16Adam.step counts
+ * state[p]["step"] per parameter and reads lr / betas / eps / weight_decay from state[p] per parameter
+ * (patrickstar/ops/fp16_cpu_adam.py:571-606), and fp16_chunk_adam_ops hands each call its own (:403-428).  They
+ * differ between tensors when a parameter was frozen for some steps (its count stays behind) or when somebody
+ * wrote state[p]["lr"] for some parameters only. */
+typedef struct ps_tensor_call {
+    double lr, beta1, beta2, eps, weight_decay;
+    int64_t step;       /* host-decided step: this tensor's step number (state[p]["step"] after its increment, >= 1);
+                           device-decided step: its distance d from the device's counter, the tensor's step number
+                           then being d_state->adam_step + 1 + d (which must come out >= 1) */
+    int32_t arithmetic; /* PS_ARITH_OPERATOR, PS_ARITH_TORCH, or -1 for the optimizer's own (ps_adam_set_arithmetic) */
+    int32_t reserved;
+} ps_tensor_call;
+
+/* Device memory ps_adam_step_tensors_each needs for a device-decided step over n_tensors tensors (the step
+ * constants of every distinct call, formed on the device): 64 bytes per tensor at most. */
+size_t ps_tensors_each_workspace_bytes(int n_tensors);
+
+/* ps_adam_step_tensors with per-tensor step numbers and hyper-parameters: tensors[i] is updated with each[i].
+ * The list is the WHOLE step, in the reference's call order (param_groups order): the native operator object is
+ * taken through every call that uses the operator's arithmetic, in that order, exactly as
+ * Adam_Optimizer::IncrementStep (cpu_adam.h:143-162) moves: a call continues the running float product beta^t
+ * only if its step number is the previous call's plus one and its betas are the previous call's, and evaluates
+ * (float)pow((double)beta, step) otherwise.  Calls with the torch arithmetic form 1 - beta ** step in binary64
+ * from their own numbers and leave the object alone.  Tensors whose calls come out with the same constants
+ * share launches (sorted by length as in ps_adam_step_tensors), so the common cases (one thawed layer, two
+ * learning rates) take two or three launches more than the uniform step.
+ *   d_state == NULL  host-decided: each[i].step is the step number; loss_scale as for ps_adam_step_chunks;
+ *                    d_workspace is not used
+ *   d_state != NULL  device-decided: a flagged step restores the fp16 slots from fp32; else every call's
+ *                    constants are formed ON THE DEVICE from d_state (adam_step, cur_scale, the operator
+ *                    object's state) by a small kernel in front of the update kernels, into d_workspace (at
+ *                    least ps_tensors_each_workspace_bytes(n_tensors) bytes of device memory, 16-byte aligned,
+ *                    owned by the caller and left alone by it until the step has run).  loss_scale is ignored.
+ *                    The object's state after the step's last call is left in d_state's pending_* fields: follow
+ *                    with ps_scaler_update (operator_calls = the number of operator-arithmetic calls), which
+ *                    adopts it on a clean step and drops it on a skipped one.
+ * Addresses may be pinned host memory (host-resident optimizer state is then read and written over the link in
+ * place).  The clamp of ps_adam_set_grad_clamp applies. */
+int ps_adam_step_tensors_each(int optimizer_id, int bias_correction, const ps_chunk* tensors,
+                              const size_t* numels, const ps_tensor_call* each, int n_tensors,
+                              double loss_scale, ps_step_state* d_state, void* d_workspace,
+                              size_t workspace_bytes, ps_stream_t stream);
 
 /* Unconditional restore p16 = RNE(p32) of a chunk list (FP16ChunkWriteBuffer,
  * chunk_io_buff.py:85-151), or only when d_state->overflow is set if d_state != NULL. */
@@ -273,6 +343,8 @@ int ps_restore_fp16_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_nu
  *   staging      host array of n_slots (1..8) descriptors of DEVICE buffers of
  *                chunk_numel elements each, owned by the caller; param_fp16 may be NULL when
  *                every host chunk keeps its fp16 payload in HBM
+ *   used_numel   as for ps_adam_step_chunks, over chunks[] followed by host_chunks[] (NULL: all full);
+ *                only the used part of a host chunk crosses the link
  *   calls        as for ps_adam_step_chunks, over chunks[] followed by host_chunks[]; with
  *                PS_ARITH_TORCH only host_chunks[] reach the operator and the pattern describes those
  *                (first_chunk >= n_chunks).  NULL: one operator call for everything
@@ -288,16 +360,17 @@ int ps_restore_fp16_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_nu
 int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, double beta2,
                         double epsilon, double weight_decay, int bias_correction,
                         const ps_chunk* chunks, int n_chunks, const ps_chunk* host_chunks,
-                        int n_host_chunks, size_t chunk_numel, const ps_chunk* staging, int n_slots,
-                        const ps_call_pattern* calls, double loss_scale, const ps_step_state* d_state,
-                        ps_stream_t stream);
+                        int n_host_chunks, size_t chunk_numel, const size_t* used_numel,
+                        const ps_chunk* staging, int n_slots, const ps_call_pattern* calls,
+                        double loss_scale, const ps_step_state* d_state, ps_stream_t stream);
 
 /* The inf/nan probe for host-resident chunks: only the fp16 payloads are
  * streamed (2 B/element) through staging[i].param_fp16; fp16 payloads that
- * live in HBM are probed in place. */
+ * live in HBM are probed in place.  used_numel (NULL: all full): only the first used_numel[i] elements
+ * of chunk i can hold anything but zeros and only they are looked at. */
 int ps_overflow_scan_host_chunks(const ps_chunk* host_chunks, int n_chunks, size_t chunk_numel,
-                                 const ps_chunk* staging, int n_slots, ps_step_state* d_state,
-                                 ps_stream_t stream);
+                                 const size_t* used_numel, const ps_chunk* staging, int n_slots,
+                                 ps_step_state* d_state, ps_stream_t stream);
 
 /* Whole-buffer RNE cast (payload_fp16.copy_(payload_fp32), chunk_io_buff.py:116-126). */
 int ps_cast_fp32_to_fp16(const float* d_src, uint16_t* d_dst, size_t numel, ps_stream_t stream);
@@ -313,7 +386,9 @@ int ps_state_init(ps_step_state* d_state, double init_scale, int init_is_int, do
                   int delayed_shift, int consecutive_hysteresis, double beta1, double beta2,
                   ps_stream_t stream);
 
-/* Set the Adam step counter (load_state_dict, fp16_cpu_adam.py:660-694) and betas.
+/* Set the Adam step counter (load_state_dict, fp16_cpu_adam.py:660-694) and the betas of the next step (the
+ * reference hands state[p]["betas"] to the operator with every call, fp16_cpu_adam.py:404-407: betas that
+ * differ from the object's restart beta^t from pow, cpu_adam.h:145-150).
  *   fresh_operator != 0  a new operator object stands behind them (step 0, beta^t = 1, as create_adam leaves
  *                        it): its first call, for step adam_step + 1, multiplies only if adam_step is 0 and
  *                        otherwise evaluates pow((float)beta, adam_step + 1) in double and narrows, i.e. the
@@ -338,8 +413,10 @@ int ps_overflow_scan(const uint16_t* d_grads_fp16, size_t numel, ps_step_state* 
                      ps_stream_t stream);
 int ps_overflow_scan_f32(const float* d_grads_fp32, size_t numel, ps_step_state* d_state,
                          ps_stream_t stream);
+/* ... over the fp16 payloads of a chunk list; used_numel as for ps_adam_step_chunks (the zeros behind a
+ * chunk's last tensor are finite: they are not read). */
 int ps_overflow_scan_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_numel,
-                            ps_step_state* d_state, ps_stream_t stream);
+                            const size_t* used_numel, ps_step_state* d_state, ps_stream_t stream);
 
 /* ps_overflow_scan_chunks for callers that cannot allocate device memory.  It has no counterpart in the
  * reference: it exists for code running under HIP graph capture, tight serving loops and harnesses that
@@ -376,7 +453,8 @@ int ps_grad_to_chunk(const void* d_grad, int grad_is_half, uint16_t* d_slot_fp16
  * the torch arithmetic.  operator_calls says how often the step that was just
  * queued called the operator in the reference's terms: the n_calls of its
  * ps_call_pattern (1 without one, the tensor count of ps_adam_step_tensors, 0 if
- * every chunk took the torch formula).  Clears the sticky flag.  If d_log
+ * every chunk took the torch formula); a pending record left by ps_adam_step_tensors_each takes its place.
+ * Clears the sticky flag and the pending record.  If d_log
  * is not NULL, entry [cur_iter % log_capacity] (cur_iter before the
  * increment) records the decision. */
 int ps_scaler_update(ps_step_state* d_state, int flag_mode, ps_scale_record* d_log,

@@ -361,7 +361,6 @@ class OptimizerStepOracle:
         self.loss_scaler = loss_scaler
         self.lr, self.betas, self.eps, self.weight_decay = lr, betas, eps, weight_decay
         self.use_adamw = use_adamw
-        self.step_count = 0
         self.has_overflow = False
         self.isa = isa
         self.gradient_clipping = gradient_clipping
@@ -377,7 +376,32 @@ class OptimizerStepOracle:
         for ci, off, numel in tensors:
             assert 0 <= ci < len(chunks) and 0 <= off and off + numel <= chunks[ci]["p32"].size, (ci, off, numel)
         self.tensors = list(tensors)
+        # state[p] of the reference (fp16_cpu_adam.py:111-131): every parameter carries its OWN step number and
+        # its own copy of the hyper-parameters, and step() hands each operator call its tensor's own numbers
+        # (:571-606, :406-410).  Keyed by the tensor's span; made on first use with the constructor's values.
+        self._default_step = 0
+        self._state = {}
         self.native = AdamOracle(lr, betas[0], betas[1], eps, weight_decay, use_adamw)
+
+    def state(self, span):
+        """The reference's ``state[p]`` entries of the tensor at ``span = (chunk, offset, numel)``: ``step``, ``lr``,
+        ``betas``, ``eps``, ``weight_decay``.  Writable, like the reference's."""
+        span = tuple(span)
+        if span not in self._state:
+            self._state[span] = {"step": self._default_step, "lr": self.lr, "betas": self.betas, "eps": self.eps,
+                                 "weight_decay": self.weight_decay}
+        return self._state[span]
+
+    @property
+    def step_count(self):
+        """``state[p]["step"]`` of the first listed tensor (every tensor's, while all of them are stepped together)."""
+        return self.state(self.tensors[0])["step"] if self.tensors else self._default_step
+
+    @step_count.setter
+    def step_count(self, value):
+        self._default_step = value
+        for st in self._state.values():
+            st["step"] = value
 
     def check_overflow(self):
         """Sticky OR over every chunk's gradients (``fp16_cpu_adam.py:279-285``)."""
@@ -408,23 +432,27 @@ class OptimizerStepOracle:
             self.has_overflow = False
             self.loss_scaler.update_scale(True)
             return True
-        self.step_count += 1
         scaler_scale = self.loss_scaler.loss_scale if self.loss_scaler is not None else None
+        if not self.tensors:
+            self._default_step += 1
+        # :569-606: every trainable parameter's own step advances, then the lists are built
+        calls = []
+        for span in self.tensors:
+            st = self.state(span)
+            st["step"] += 1
+            calls.append((span, st["step"], st["lr"], st["betas"], st["eps"], st["weight_decay"]))
         visited = []
-        for ci, off, numel in self.tensors:
+        for (ci, off, numel), step, lr, (beta1, beta2), eps, weight_decay in calls:
             c = self.chunks[ci]
             p, g, m, v = (c[k][off : off + numel] for k in ("p32", "p16", "m", "v"))
             if self.gradient_clipping > 0:
                 self._clamp(g)
             if self.arithmetic == "torch" and ci not in self.operator_chunks:
-                torch_formula_update(
-                    p, g, m, v, self.step_count, self.lr, self.betas[0], self.betas[1],
-                    self.eps, self.weight_decay, self.use_adamw, scaler_scale,
-                )
+                torch_formula_update(p, g, m, v, step, lr, beta1, beta2, eps, weight_decay, self.use_adamw, scaler_scale)
             else:
                 # one adam_update of the native operator: IncrementStep, update_state, Step
                 self.native.update(
-                    self.step_count, self.lr, self.betas[0], self.betas[1], self.eps, self.weight_decay, True,
+                    step, lr, beta1, beta2, eps, weight_decay, True,
                     p, g, m, v, float(scaler_scale if scaler_scale is not None else -1), self.isa,
                 )
             if ci not in visited:

@@ -11,7 +11,7 @@ LIB_PATH = os.path.join(PKG_DIR, "libps_adam.so")
 PS_FLAG_FALSE, PS_FLAG_TRUE, PS_FLAG_FROM_DEVICE = 0, 1, 2
 PS_ERR_BAD_ARG, PS_ERR_UNKNOWN_ID, PS_ERR_NO_DEVICE = -10001, -10002, -10003
 PS_ARITH_OPERATOR, PS_ARITH_TORCH = 0, 1
-PS_ABI_VERSION = 4
+PS_ABI_VERSION = 5
 
 
 class ps_chunk(ctypes.Structure):
@@ -56,6 +56,14 @@ class ps_step_state(ctypes.Structure):
         ("beta1_t_rest", ctypes.c_float),
         ("beta2_t_rest", ctypes.c_float),
         ("reserved2", ctypes.c_uint32 * 2),
+        ("operator_beta1", ctypes.c_float),
+        ("operator_beta2", ctypes.c_float),
+        ("pending_operator_step", ctypes.c_int64),
+        ("pending_beta1_t", ctypes.c_float),
+        ("pending_beta2_t", ctypes.c_float),
+        ("pending_beta1", ctypes.c_float),
+        ("pending_beta2", ctypes.c_float),
+        ("reserved3", ctypes.c_uint32 * 8),
     ]
 
 
@@ -68,6 +76,19 @@ class ps_call_pattern(ctypes.Structure):
     ]
 
 
+class ps_tensor_call(ctypes.Structure):
+    _fields_ = [
+        ("lr", ctypes.c_double),
+        ("beta1", ctypes.c_double),
+        ("beta2", ctypes.c_double),
+        ("eps", ctypes.c_double),
+        ("weight_decay", ctypes.c_double),
+        ("step", ctypes.c_int64),
+        ("arithmetic", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+    ]
+
+
 class ps_scale_record(ctypes.Structure):
     _fields_ = [
         ("scale_after", ctypes.c_double),
@@ -77,9 +98,10 @@ class ps_scale_record(ctypes.Structure):
 
 
 assert ctypes.sizeof(ps_chunk) == 32
-assert ctypes.sizeof(ps_step_state) == 192
+assert ctypes.sizeof(ps_step_state) == 256
 assert ctypes.sizeof(ps_call_pattern) == 32
 assert ctypes.sizeof(ps_scale_record) == 16
+assert ctypes.sizeof(ps_tensor_call) == 56
 
 _f, _d, _i, _i64, _sz, _vp = (
     ctypes.c_float,
@@ -99,11 +121,13 @@ SIGNATURES = {
     "ps_adam_set_arithmetic": (_i, [_i, _i]),
     "ps_adam_destroy": (_i, [_i]),
     "ps_adam_update": (_i, [_i, _sz, _f, _f, _f, _f, _f, _i, _vp, _vp, _i, _vp, _vp, _sz, _f, _vp, _vp]),
-    "ps_adam_step_chunks": (_i, [_i, _sz, _d, _d, _d, _d, _d, _i, _vp, _i, _sz, _vp, _d, _vp]),
-    "ps_adam_step_chunks_gated": (_i, [_i, _d, _d, _d, _i, _vp, _i, _sz, _vp, _vp, _vp]),
+    "ps_adam_step_chunks": (_i, [_i, _sz, _d, _d, _d, _d, _d, _i, _vp, _i, _sz, _vp, _vp, _d, _vp]),
+    "ps_adam_step_chunks_gated": (_i, [_i, _d, _d, _d, _i, _vp, _i, _sz, _vp, _vp, _vp, _vp]),
     "ps_adam_step_tensors": (_i, [_i, _sz, _d, _d, _d, _d, _d, _i, _vp, _vp, _i, _vp, _d, _vp, _vp]),
-    "ps_adam_step_hybrid": (_i, [_i, _sz, _d, _d, _d, _d, _d, _i, _vp, _i, _vp, _i, _sz, _vp, _i, _vp, _d, _vp, _vp]),
-    "ps_overflow_scan_host_chunks": (_i, [_vp, _i, _sz, _vp, _i, _vp, _vp]),
+    "ps_tensors_each_workspace_bytes": (_sz, [_i]),
+    "ps_adam_step_tensors_each": (_i, [_i, _i, _vp, _vp, _vp, _i, _d, _vp, _vp, _sz, _vp]),
+    "ps_adam_step_hybrid": (_i, [_i, _sz, _d, _d, _d, _d, _d, _i, _vp, _i, _vp, _i, _sz, _vp, _vp, _i, _vp, _d, _vp, _vp]),
+    "ps_overflow_scan_host_chunks": (_i, [_vp, _i, _sz, _vp, _vp, _i, _vp, _vp]),
     "ps_restore_fp16_chunks": (_i, [_vp, _i, _sz, _vp, _vp]),
     "ps_cast_fp32_to_fp16": (_i, [_vp, _vp, _sz, _vp]),
     "ps_state_init": (_i, [_vp, _d, _i, _d, _i, _i64, _d, _i, _i, _i, _d, _d, _vp]),
@@ -111,7 +135,7 @@ SIGNATURES = {
     "ps_state_set_scaler": (_i, [_vp, _d, _i, _i64, _i64, _i, _vp]),
     "ps_overflow_scan": (_i, [_vp, _sz, _vp, _vp]),
     "ps_overflow_scan_f32": (_i, [_vp, _sz, _vp, _vp]),
-    "ps_overflow_scan_chunks": (_i, [_vp, _i, _sz, _vp, _vp]),
+    "ps_overflow_scan_chunks": (_i, [_vp, _i, _sz, _vp, _vp, _vp]),
     "ps_overflow_scan_chunks_noalloc": (_i, [_vp, _i, _sz, _vp, _vp]),
     "ps_grad_to_chunk": (_i, [_vp, _i, _vp, _sz, _vp, _vp]),
     "ps_scaler_update": (_i, [_vp, _i, _vp, _i64, _i64, _vp]),
@@ -164,6 +188,11 @@ def current_stream_handle():
 def call_pattern(n_calls, first_chunk=0, first_offset=0, first_numel=0):
     """A ps_call_pattern, by reference, for the `calls` argument of the step entry points."""
     return ctypes.byref(ps_call_pattern(int(n_calls), int(first_chunk), int(first_offset), int(first_numel)))
+
+
+def size_array(values):
+    """Host array of size_t, or None for an empty / absent list."""
+    return (ctypes.c_size_t * len(values))(*values) if values else None
 
 
 def chunk_array(rows):

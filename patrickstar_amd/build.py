@@ -1,5 +1,4 @@
-"""Builds libps_adam.so (the C-ABI HIP library) and libps_stream_probe.so (the streaming kernels `bench.py --mode
-ceiling` measures the memory system with; not loaded by the package) for gfx950 with hipcc, in-tree."""
+"""Builds libps_adam.so (the C-ABI HIP library) for gfx950 with hipcc, in-tree."""
 import os
 import shutil
 import subprocess
@@ -8,8 +7,6 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(PKG_DIR)
 LIB_PATH = os.path.join(PKG_DIR, "libps_adam.so")
 SOURCES = [os.path.join(PKG_DIR, "csrc", "ps_adam.hip")]
-PROBE_PATH = os.path.join(PKG_DIR, "libps_stream_probe.so")
-PROBE_SOURCES = [os.path.join(PKG_DIR, "csrc", "ps_stream_probe.hip")]
 INCLUDE = os.path.join(ROOT, "include")
 
 # -ffp-contract=off: fused multiply-adds are written out explicitly; the compiler must not add or remove any.
@@ -42,7 +39,8 @@ def hipcc_path():
     raise RuntimeError("hipcc not found: the HIP library cannot be built")
 
 
-def _compile(sources, target, verbose, extra_flags):
+def compile_shared(sources, target, verbose=False, extra_flags=()):
+    """hipcc the given sources into one shared library with this package's flags."""
     # compile beside the target and rename: a process that has the old library mapped keeps its own copy
     tmp = target + f".{os.getpid()}.tmp"
     cmd = [hipcc_path(), *HIPCC_FLAGS, *extra_flags, "-I", INCLUDE, *sources, "-o", tmp]
@@ -58,9 +56,8 @@ def _compile(sources, target, verbose, extra_flags):
 
 
 def build(verbose=False, extra_flags=()):
-    """Compile every HIP source: patrickstar_amd/libps_adam.so (returned) and libps_stream_probe.so."""
-    _compile(PROBE_SOURCES, PROBE_PATH, verbose, ())
-    return _compile(SOURCES, LIB_PATH, verbose, extra_flags)
+    """Compile the package's HIP sources into patrickstar_amd/libps_adam.so (returned)."""
+    return compile_shared(SOURCES, LIB_PATH, verbose, extra_flags)
 
 
 if __name__ == "__main__":

@@ -150,11 +150,14 @@ struct ChunkList {
     const ps_chunk* chunks;
     int n_chunks;
     size_t chunk_numel;
-    size_t tiles_per_chunk;  // of kTile elements
+    const size_t* used;  // per chunk: elements in front of the zero padding; nullptr: every chunk is full
+    size_t tile;         // elements per workgroup of the kernel that will run over the list
+
+    size_t numel_of(int i) const { return used ? used[i] : chunk_numel; }
 };
 
 // All descriptors are checked here, before anything is enqueued or any host state advances.
-int make_chunk_list(ChunkList& a, const ps_chunk* chunks, int n_chunks, size_t chunk_numel,
+int make_chunk_list(ChunkList& a, const ps_chunk* chunks, int n_chunks, size_t chunk_numel, const size_t* used_numel,
                     size_t tile, bool fp16_only = false, const char* what = "chunk")
 {
     if (n_chunks < 0) return fail(PS_ERR_BAD_ARG, "n_chunks = %d is negative", n_chunks);
@@ -163,27 +166,37 @@ int make_chunk_list(ChunkList& a, const ps_chunk* chunks, int n_chunks, size_t c
         const ps_chunk& c = chunks[i];
         if (!c.param_fp16 || (!fp16_only && (!c.param_fp32 || !c.exp_avg || !c.exp_avg_sq)))
             return fail(PS_ERR_BAD_ARG, "%s %d has a NULL payload address", what, i);
+        if (used_numel && used_numel[i] > chunk_numel)
+            return fail(PS_ERR_BAD_ARG, "%s %d: used_numel = %zu is beyond chunk_numel = %zu", what, i, used_numel[i],
+                        chunk_numel);
     }
     a.chunks = chunks;
     a.n_chunks = n_chunks;
     a.chunk_numel = chunk_numel;
-    a.tiles_per_chunk = (chunk_numel + tile - 1) / tile;
-    if (a.tiles_per_chunk > kMaxGridX)
+    a.used = used_numel;
+    a.tile = tile;
+    if ((chunk_numel + tile - 1) / tile > kMaxGridX)
         return fail(PS_ERR_BAD_ARG, "chunk_numel = %zu is beyond the launch grid", chunk_numel);
     return 0;
 }
 
-// Calls launch(batch, grid, index of the batch's first chunk) for every group of up to kBatch chunks.
+// Calls launch(batch, grid, index of the batch's first chunk) for every group of up to kBatch chunks.  The grid is
+// as wide as the longest chunk of the batch; workgroups beyond a shorter chunk's end leave at once.
 template <typename F>
 int for_each_batch(const ChunkList& a, F launch)
 {
-    if (a.n_chunks == 0 || a.tiles_per_chunk == 0) return 0;
     for (int first = 0; first < a.n_chunks; first += kBatch) {
         int n = a.n_chunks - first < kBatch ? a.n_chunks - first : kBatch;
         ChunkBatch b;
         memset(&b, 0, sizeof(b));
-        for (int i = 0; i < n; ++i) b.c[i] = a.chunks[first + i];
-        launch(b, dim3((unsigned)a.tiles_per_chunk, (unsigned)n), first);
+        size_t tiles = 0;
+        for (int i = 0; i < n; ++i) {
+            b.c[i] = a.chunks[first + i];
+            b.n[i] = a.numel_of(first + i);
+            tiles = std::max(tiles, (b.n[i] + a.tile - 1) / a.tile);
+        }
+        if (tiles == 0) continue;
+        launch(b, dim3((unsigned)tiles, (unsigned)n), first);
         PS_HIP(hipGetLastError());
     }
     return 0;
@@ -229,39 +242,37 @@ int make_calls(Calls& out, const ps_call_pattern* calls, int64_t n_chunks_total,
 }
 
 template <int ARITH, int WD>
-void launch_adam_batch_wd(const ChunkBatch& b, dim3 grid, size_t chunk_numel, const StepConsts& c,
-                          const FirstCall& fc, hipStream_t s)
+void launch_adam_batch_wd(const ChunkBatch& b, dim3 grid, const StepConsts& c, const FirstCall& fc, hipStream_t s)
 {
     dim3 block(kBlock);
     if (c.unscale == UNSCALE_MUL)
-        hipLaunchKernelGGL((adam_chunks_kernel<ARITH, WD, UNSCALE_MUL>), grid, block, kLdsBytes, s, b, chunk_numel, c, fc);
+        hipLaunchKernelGGL((adam_chunks_kernel<ARITH, WD, UNSCALE_MUL>), grid, block, kLdsBytes, s, b, c, fc);
     else if (ARITH == PS_ARITH_OPERATOR && c.unscale == UNSCALE_DIV)  // the torch formula never divides
-        hipLaunchKernelGGL((adam_chunks_kernel<ARITH, WD, UNSCALE_DIV>), grid, block, kLdsBytes, s, b, chunk_numel, c, fc);
+        hipLaunchKernelGGL((adam_chunks_kernel<ARITH, WD, UNSCALE_DIV>), grid, block, kLdsBytes, s, b, c, fc);
     else
-        hipLaunchKernelGGL((adam_chunks_kernel<ARITH, WD, UNSCALE_NONE>), grid, block, kLdsBytes, s, b, chunk_numel, c, fc);
+        hipLaunchKernelGGL((adam_chunks_kernel<ARITH, WD, UNSCALE_NONE>), grid, block, kLdsBytes, s, b, c, fc);
 }
 
 template <int ARITH>
-void launch_adam_batch_arith(const ChunkBatch& b, dim3 grid, size_t chunk_numel,
-                             const StepConsts& c, const FirstCall& fc, hipStream_t s)
+void launch_adam_batch_arith(const ChunkBatch& b, dim3 grid, const StepConsts& c, const FirstCall& fc, hipStream_t s)
 {
     if (c.wd_mode == WD_DECOUPLED)
-        launch_adam_batch_wd<ARITH, WD_DECOUPLED>(b, grid, chunk_numel, c, fc, s);
+        launch_adam_batch_wd<ARITH, WD_DECOUPLED>(b, grid, c, fc, s);
     else if (c.wd_mode == WD_L2)
-        launch_adam_batch_wd<ARITH, WD_L2>(b, grid, chunk_numel, c, fc, s);
+        launch_adam_batch_wd<ARITH, WD_L2>(b, grid, c, fc, s);
     else
-        launch_adam_batch_wd<ARITH, WD_NONE>(b, grid, chunk_numel, c, fc, s);
+        launch_adam_batch_wd<ARITH, WD_NONE>(b, grid, c, fc, s);
 }
 
 // `c` must have been built for `arith` (finish_consts / torch_consts).  `fc`: which elements of the
 // batch the step's first operator call covers; the torch formula has no such distinction.
-void launch_adam_batch(int arith, const ChunkBatch& b, dim3 grid, size_t chunk_numel,
-                       const StepConsts& c, const FirstCall& fc, hipStream_t s)
+void launch_adam_batch(int arith, const ChunkBatch& b, dim3 grid, const StepConsts& c, const FirstCall& fc,
+                       hipStream_t s)
 {
     if (arith == PS_ARITH_TORCH)
-        launch_adam_batch_arith<PS_ARITH_TORCH>(b, grid, chunk_numel, c, FirstCall{-1, 0, 0}, s);
+        launch_adam_batch_arith<PS_ARITH_TORCH>(b, grid, c, FirstCall{-1, 0, 0}, s);
     else
-        launch_adam_batch_arith<PS_ARITH_OPERATOR>(b, grid, chunk_numel, c, fc, s);
+        launch_adam_batch_arith<PS_ARITH_OPERATOR>(b, grid, c, fc, s);
 }
 
 template <int ARITH>
@@ -708,12 +719,13 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
 int ps_adam_step_chunks(int optimizer_id, size_t step, double lr, double beta1, double beta2,
                         double epsilon, double weight_decay, int bias_correction,
                         const ps_chunk* chunks, int n_chunks, size_t chunk_numel,
-                        const ps_call_pattern* calls, double loss_scale, ps_stream_t stream)
+                        const size_t* used_numel, const ps_call_pattern* calls, double loss_scale,
+                        ps_stream_t stream)
 {
     auto o = find_opt(optimizer_id);
     if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
     ChunkList a;
-    if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, kTile)) return rc;
+    if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, used_numel, kTile)) return rc;
     Calls k;
     if (int rc = make_calls(k, calls, n_chunks, chunk_numel)) return rc;
     const HyperParams hp{lr, beta1, beta2, epsilon, weight_decay, loss_scale, bias_correction != 0};
@@ -722,41 +734,53 @@ int ps_adam_step_chunks(int optimizer_id, size_t step, double lr, double beta1, 
         c = torch_step_consts(*o, step, hp);
     else
         c = operator_step_consts(*o, step, hp, k.n_calls);
+    if (!zeros_are_a_fixed_point(c)) a.used = nullptr;  // the padding is computed like everything else
     const int arith = o->arith;
     hipStream_t s = static_cast<hipStream_t>(stream);
     return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid, int first) {
-        launch_adam_batch(arith, b, grid, chunk_numel, c, k.in_batch(first, (int)grid.y), s);
+        launch_adam_batch(arith, b, grid, c, k.in_batch(first, (int)grid.y), s);
     });
 }
 
 int ps_adam_step_chunks_gated(int optimizer_id, double lr, double epsilon, double weight_decay,
                               int bias_correction, const ps_chunk* chunks, int n_chunks,
-                              size_t chunk_numel, const ps_call_pattern* calls,
-                              const ps_step_state* d_state, ps_stream_t stream)
+                              size_t chunk_numel, const size_t* used_numel,
+                              const ps_call_pattern* calls, const ps_step_state* d_state,
+                              ps_stream_t stream)
 {
     auto o = find_opt(optimizer_id);
     if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
     if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
     ChunkList a;
-    if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, kTile)) return rc;
+    if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, used_numel, kTile)) return rc;
     Calls k;
     if (int rc = make_calls(k, calls, n_chunks, chunk_numel)) return rc;
     const GatedArgs ga = gated_args(*o, lr, epsilon, weight_decay, bias_correction, k.n_calls);
     const int arith = o->arith;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    // (whether the padding may be left alone depends on the device-resident scalars: the kernel decides)
     return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid, int first) {
         launch_gated_batch(arith, b, grid, chunk_numel, ga, k.in_batch(first, (int)grid.y), d_state, s);
     });
 }
 
-int ps_adam_step_tensors(int optimizer_id, size_t step, double lr, double beta1, double beta2,
-                         double epsilon, double weight_decay, int bias_correction,
-                         const ps_chunk* tensors, const size_t* numels, int n_tensors,
-                         const ps_call_pattern* calls, double loss_scale, const ps_step_state* d_state,
-                         ps_stream_t stream)
+}  // extern "C"
+
+namespace {
+
+// ---------------------------------------------------------- tensor lists
+//
+// Where a tensor's tile grid starts (the fp32 parameter's first 1 KiB boundary; what lies in front of it is a tile of
+// its own) and how many tiles it has.  Addresses that are not even element-aligned keep the plain numbering.
+struct TensorItem {
+    int index;  // in the caller's list
+    uint32_t head;
+    size_t body, tiles;
+};
+static_assert(kTile <= 256, "TensorBatch::numel_head keeps the head length (up to kTile - 1 elements) in 8 bits");
+
+int check_tensor_list(const ps_chunk* tensors, const size_t* numels, int n_tensors)
 {
-    auto o = find_opt(optimizer_id);
-    if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
     if (n_tensors < 0) return fail(PS_ERR_BAD_ARG, "n_tensors = %d is negative", n_tensors);
     if (n_tensors > 0 && (!tensors || !numels)) return fail(PS_ERR_BAD_ARG, "tensors or numels is NULL");
     for (int i = 0; i < n_tensors; ++i) {
@@ -766,6 +790,88 @@ int ps_adam_step_tensors(int optimizer_id, size_t step, double lr, double beta1,
         if ((numels[i] + kTile - 1) / kTile >= kMaxGridX || numels[i] > kNumelMask)
             return fail(PS_ERR_BAD_ARG, "tensor %d: numel = %zu is beyond the launch grid", i, numels[i]);
     }
+    return 0;
+}
+
+TensorItem tensor_item(const ps_chunk* tensors, const size_t* numels, int i)
+{
+    const uintptr_t p_addr = reinterpret_cast<uintptr_t>(tensors[i].param_fp32);
+    size_t head = p_addr % sizeof(float) ? 0 : (kTile - (p_addr / sizeof(float)) % kTile) % kTile;
+    if (head > numels[i]) head = numels[i];
+    const size_t body = numels[i] - head;
+    return TensorItem{i, (uint32_t)head, body, (head ? 1 : 0) + (body + kTile - 1) / kTile};
+}
+
+// Calls launch(batch, grid) for groups of the given tensors (all of them non-empty): longest first; one launch
+// takes tensors of nearly the same length (its grid is as wide as the longest of them: at most a tenth of a
+// launch's workgroups find nothing to do), short tensors all together.  `first_tensor`: the index (in the caller's
+// list) of the tensor that is the step's first operator call, marked in its batch; -1: none.
+template <typename F>
+int for_each_tensor_batch(std::vector<TensorItem>& items, const ps_chunk* tensors, int first_tensor, F launch)
+{
+    std::stable_sort(items.begin(), items.end(), [](const TensorItem& a, const TensorItem& b) { return a.tiles > b.tiles; });
+    constexpr size_t kShortTensorTiles = 256;
+    TensorBatch b;
+    size_t next = 0;
+    while (next < items.size()) {
+        memset(&b, 0, sizeof(b));
+        b.first_call = -1;
+        const size_t widest = items[next].tiles;
+        int in_batch = 0;
+        while (next < items.size() && in_batch < kTensorBatch &&
+               (items[next].tiles * 10 >= widest * 9 || widest <= kShortTensorTiles)) {
+            const TensorItem& it = items[next];
+            ps_chunk t = tensors[it.index];
+            t.param_fp32 += it.head;
+            t.exp_avg += it.head;
+            t.exp_avg_sq += it.head;
+            t.param_fp16 += it.head;
+            b.t[in_batch] = t;
+            b.numel_head[in_batch] = (uint64_t)it.body | ((uint64_t)it.head << 56);
+            if (it.index == first_tensor) b.first_call = in_batch;
+            in_batch += 1;
+            next += 1;
+        }
+        launch(b, dim3((unsigned)widest, (unsigned)in_batch));
+        PS_HIP(hipGetLastError());
+    }
+    return 0;
+}
+
+// Weight-decay form of a call, as the two arithmetics decide it: the operator tests its float weight decay "> 0"
+// (cpu_adam.cpp:42), the torch formula the Python number "!= 0".
+int wd_mode_of(int arith, double wd, bool adamw)
+{
+    const bool decay = arith == PS_ARITH_OPERATOR ? (float)wd > 0.0f : wd != 0.0;
+    return decay ? (adamw ? WD_DECOUPLED : WD_L2) : WD_NONE;
+}
+
+template <int ARITH>
+void launch_tensors_planned_arith(const TensorBatch& b, dim3 grid, int wd_mode, const PlannedConsts* d_consts,
+                                  const ps_step_state* d_state, hipStream_t s)
+{
+    dim3 block(kBlock);
+    if (wd_mode == WD_DECOUPLED)
+        hipLaunchKernelGGL((adam_tensors_planned_kernel<ARITH, WD_DECOUPLED>), grid, block, kLdsBytes, s, b, d_consts, d_state);
+    else if (wd_mode == WD_L2)
+        hipLaunchKernelGGL((adam_tensors_planned_kernel<ARITH, WD_L2>), grid, block, kLdsBytes, s, b, d_consts, d_state);
+    else
+        hipLaunchKernelGGL((adam_tensors_planned_kernel<ARITH, WD_NONE>), grid, block, kLdsBytes, s, b, d_consts, d_state);
+}
+
+}  // namespace
+
+extern "C" {
+
+int ps_adam_step_tensors(int optimizer_id, size_t step, double lr, double beta1, double beta2,
+                         double epsilon, double weight_decay, int bias_correction,
+                         const ps_chunk* tensors, const size_t* numels, int n_tensors,
+                         const ps_call_pattern* calls, double loss_scale, const ps_step_state* d_state,
+                         ps_stream_t stream)
+{
+    auto o = find_opt(optimizer_id);
+    if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
+    if (int rc = check_tensor_list(tensors, numels, n_tensors)) return rc;
     const int arith = o->arith;
     // One operator call per tensor.  Without a pattern the list is the whole step and tensors[0] its first call;
     // a pattern says how many calls the step has in all and which tensor of THIS list, if any, is the first.
@@ -786,6 +892,7 @@ int ps_adam_step_tensors(int optimizer_id, size_t step, double lr, double beta1,
             first_tensor = (int)calls->first_chunk;
         }
     }
+    if (arith != PS_ARITH_OPERATOR) first_tensor = -1;  // the torch formula has no first call
     StepConsts c;
     GatedArgs ga = gated_args(*o, lr, epsilon, weight_decay, bias_correction, n_calls);
     if (d_state == nullptr && n_tensors > 0) {
@@ -793,54 +900,15 @@ int ps_adam_step_tensors(int optimizer_id, size_t step, double lr, double beta1,
         c = arith == PS_ARITH_TORCH ? torch_step_consts(*o, step, hp) : operator_step_consts(*o, step, hp, n_calls);
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    // Where each tensor's tile grid starts (the fp32 parameter's first 1 KiB boundary; what lies in front of it is a
-    // tile of its own) and how many tiles it has.  Addresses that are not even element-aligned keep the plain
-    // numbering.
-    struct Item {
-        int index;
-        uint32_t head;
-        size_t body, tiles;
-    };
-    std::vector<Item> items;
+    std::vector<TensorItem> items;
     try {
         items.reserve((size_t)n_tensors);
     } catch (const std::exception&) {  // nothing may throw across the boundary
         return fail(PS_ERR_BAD_ARG, "no host memory for a list of %d tensors", n_tensors);
     }
-    for (int i = 0; i < n_tensors; ++i) {
-        if (numels[i] == 0) continue;
-        const uintptr_t p_addr = reinterpret_cast<uintptr_t>(tensors[i].param_fp32);
-        size_t head = p_addr % sizeof(float) ? 0 : (kTile - (p_addr / sizeof(float)) % kTile) % kTile;
-        if (head > numels[i]) head = numels[i];
-        const size_t body = numels[i] - head;
-        items.push_back(Item{i, (uint32_t)head, body, (head ? 1 : 0) + (body + kTile - 1) / kTile});
-    }
-    // Longest first; one launch takes tensors of nearly the same length (its grid is as wide as the longest of
-    // them: at most a tenth of a launch's workgroups find nothing to do), short tensors all together.
-    std::stable_sort(items.begin(), items.end(), [](const Item& a, const Item& b) { return a.tiles > b.tiles; });
-    constexpr size_t kShortTensorTiles = 256;
-    TensorBatch b;
-    size_t next = 0;
-    while (next < items.size()) {
-        memset(&b, 0, sizeof(b));
-        b.first_call = -1;
-        const size_t widest = items[next].tiles;
-        int in_batch = 0;
-        while (next < items.size() && in_batch < kTensorBatch &&
-               (items[next].tiles * 10 >= widest * 9 || widest <= kShortTensorTiles)) {
-            const Item& it = items[next];
-            ps_chunk t = tensors[it.index];
-            t.param_fp32 += it.head;
-            t.exp_avg += it.head;
-            t.exp_avg_sq += it.head;
-            t.param_fp16 += it.head;
-            b.t[in_batch] = t;
-            b.numel_head[in_batch] = (uint64_t)it.body | ((uint64_t)it.head << 56);
-            if (it.index == first_tensor && arith == PS_ARITH_OPERATOR) b.first_call = in_batch;
-            in_batch += 1;
-            next += 1;
-        }
-        const dim3 grid((unsigned)widest, (unsigned)in_batch);
+    for (int i = 0; i < n_tensors; ++i)
+        if (numels[i] != 0) items.push_back(tensor_item(tensors, numels, i));
+    return for_each_tensor_batch(items, tensors, first_tensor, [&](const TensorBatch& b, dim3 grid) {
         if (d_state == nullptr) {
             if (arith == PS_ARITH_TORCH)
                 launch_tensors_arith<PS_ARITH_TORCH>(b, grid, c, s);
@@ -852,19 +920,176 @@ int ps_adam_step_tensors(int optimizer_id, size_t step, double lr, double beta1,
             else
                 launch_tensors_gated_arith<PS_ARITH_OPERATOR>(b, grid, ga, d_state, s);
         }
-        PS_HIP(hipGetLastError());
+    });
+}
+
+size_t ps_tensors_each_workspace_bytes(int n_tensors)
+{
+    return n_tensors > 0 ? (size_t)n_tensors * sizeof(PlannedConsts) : 0;
+}
+
+int ps_adam_step_tensors_each(int optimizer_id, int bias_correction, const ps_chunk* tensors,
+                              const size_t* numels, const ps_tensor_call* each, int n_tensors,
+                              double loss_scale, ps_step_state* d_state, void* d_workspace,
+                              size_t workspace_bytes, ps_stream_t stream)
+{
+    auto o = find_opt(optimizer_id);
+    if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
+    if (int rc = check_tensor_list(tensors, numels, n_tensors)) return rc;
+    if (n_tensors > 0 && !each) return fail(PS_ERR_BAD_ARG, "each is NULL");
+    for (int i = 0; i < n_tensors; ++i) {
+        const int a = each[i].arithmetic;
+        if (a != -1 && a != PS_ARITH_OPERATOR && a != PS_ARITH_TORCH)
+            return fail(PS_ERR_BAD_ARG, "each[%d].arithmetic = %d", i, a);
+        if (d_state == nullptr && each[i].step < 1)
+            return fail(PS_ERR_BAD_ARG, "each[%d].step = %lld: a host-decided step number is at least 1", i,
+                        (long long)each[i].step);
     }
-    return 0;
+    if (d_state != nullptr && n_tensors > 0) {
+        if (!d_workspace || workspace_bytes < ps_tensors_each_workspace_bytes(n_tensors))
+            return fail(PS_ERR_BAD_ARG, "d_workspace holds %zu bytes; a device-decided step over %d tensors needs %zu",
+                        d_workspace ? workspace_bytes : (size_t)0, n_tensors, ps_tensors_each_workspace_bytes(n_tensors));
+        if (reinterpret_cast<uintptr_t>(d_workspace) % 16)
+            return fail(PS_ERR_BAD_ARG, "d_workspace must be 16-byte aligned");
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool bias = bias_correction != 0;
+    auto arith_of = [&](int i) { return each[i].arithmetic < 0 ? o->arith : each[i].arithmetic; };
+    try {
+        // Calls that come out with the same constants form a class; class_of[i] says which one tensor i belongs to.
+        std::vector<int> class_of((size_t)n_tensors, -1);
+        std::vector<int> class_arith, class_wd;
+        if (d_state == nullptr) {
+            // ---- host-decided: the operator object goes through the calls, in order
+            std::vector<StepConsts> consts;
+            for (int i = 0; i < n_tensors; ++i) {
+                const ps_tensor_call& e = each[i];
+                const int arith = arith_of(i);
+                const HyperParams hp{e.lr, e.beta1, e.beta2, e.eps, e.weight_decay, loss_scale, bias};
+                StepConsts c;
+                memset(&c, 0, sizeof(c));
+                if (arith == PS_ARITH_TORCH)
+                    c = torch_step_consts(*o, (size_t)e.step, hp);
+                else
+                    c = operator_step_consts(*o, (size_t)e.step, hp, 1);
+                int k = 0;
+                for (; k < (int)consts.size(); ++k)
+                    if (class_arith[k] == arith && memcmp(&consts[k], &c, sizeof(c)) == 0) break;
+                if (k == (int)consts.size()) {
+                    consts.push_back(c);
+                    class_arith.push_back(arith);
+                    class_wd.push_back(c.wd_mode);
+                }
+                class_of[i] = k;
+            }
+            std::vector<TensorItem> items;
+            for (int k = 0; k < (int)consts.size(); ++k) {
+                items.clear();
+                for (int i = 0; i < n_tensors; ++i)
+                    if (class_of[i] == k && numels[i] != 0) items.push_back(tensor_item(tensors, numels, i));
+                const StepConsts& c = consts[k];
+                int rc = for_each_tensor_batch(items, tensors, -1, [&](const TensorBatch& b, dim3 grid) {
+                    if (class_arith[k] == PS_ARITH_TORCH)
+                        launch_tensors_arith<PS_ARITH_TORCH>(b, grid, c, s);
+                    else
+                        launch_tensors_arith<PS_ARITH_OPERATOR>(b, grid, c, s);
+                });
+                if (rc) return rc;
+            }
+            return 0;
+        }
+
+        // ---- device-decided: the step numbers (adam_step + 1 + d), the loss scale and the operator object live on
+        // the device.  The host knows how the calls relate to one another (IncrementStep, cpu_adam.h:143-162, looks
+        // only at differences between consecutive calls), which leaves three kinds of operator call and one
+        // torch call; the device turns each distinct one into constants.
+        std::vector<PlanClass> classes;
+        int prev_class = -1;  // of the previous operator call
+        int last_operator = -1;
+        for (int i = 0; i < n_tensors; ++i) {
+            const ps_tensor_call& e = each[i];
+            const int arith = arith_of(i);
+            PlanClass k;
+            memset(&k, 0, sizeof(k));
+            k.lr = e.lr, k.beta1 = e.beta1, k.beta2 = e.beta2, k.eps = e.eps, k.wd = e.weight_decay;
+            k.d = e.step;
+            k.prev = -1;
+            if (arith == PS_ARITH_TORCH) {
+                k.mode = PLAN_TORCH;
+            } else if (prev_class < 0) {
+                k.mode = PLAN_FIRST;  // continues the product only if the object, as the last clean step left it, allows
+            } else {
+                const PlanClass& q = classes[prev_class];
+                const bool same_betas = (float)q.beta1 == (float)e.beta1 && (float)q.beta2 == (float)e.beta2;
+                if (same_betas && e.step == q.d + 1) {
+                    k.mode = PLAN_MUL;
+                    k.prev = prev_class;
+                } else {
+                    k.mode = PLAN_POW;
+                }
+            }
+            int c = 0;
+            for (; c < (int)classes.size(); ++c)
+                if (class_arith[c] == arith && memcmp(&classes[c], &k, sizeof(k)) == 0) break;
+            if (c == (int)classes.size()) {
+                classes.push_back(k);
+                class_arith.push_back(arith);
+                class_wd.push_back(wd_mode_of(arith, e.weight_decay, o->adamw));
+            }
+            class_of[i] = c;
+            if (arith != PS_ARITH_TORCH) prev_class = last_operator = c;
+        }
+        PlannedConsts* table = static_cast<PlannedConsts*>(d_workspace);
+        const int n_classes = (int)classes.size();
+        for (int first = 0; first < n_classes || first == 0; first += kPlanBatch) {
+            PlanBatch pb;
+            memset(&pb, 0, sizeof(pb));
+            PlanArgs pa;
+            memset(&pa, 0, sizeof(pa));
+            pa.n = std::min(kPlanBatch, n_classes - first);
+            for (int j = 0; j < pa.n; ++j) pb.k[j] = classes[first + j];
+            pa.grad_clamp = o->grad_clamp;
+            pa.adamw = o->adamw ? 1 : 0;
+            pa.bias_correction = bias ? 1 : 0;
+            pa.first_class = first;
+            pa.is_last_launch = first + kPlanBatch >= n_classes;
+            pa.last_operator_class = last_operator;
+            if (last_operator >= 0) {
+                pa.last_d = classes[last_operator].d;
+                pa.last_beta1 = (float)classes[last_operator].beta1;
+                pa.last_beta2 = (float)classes[last_operator].beta2;
+            }
+            hipLaunchKernelGGL(plan_consts_kernel, dim3(1), dim3(64), 0, s, pb, pa, d_state, table);
+            PS_HIP(hipGetLastError());
+            if (n_classes == 0) break;
+        }
+        std::vector<TensorItem> items;
+        for (int k = 0; k < n_classes; ++k) {
+            items.clear();
+            for (int i = 0; i < n_tensors; ++i)
+                if (class_of[i] == k && numels[i] != 0) items.push_back(tensor_item(tensors, numels, i));
+            int rc = for_each_tensor_batch(items, tensors, -1, [&](const TensorBatch& b, dim3 grid) {
+                if (class_arith[k] == PS_ARITH_TORCH)
+                    launch_tensors_planned_arith<PS_ARITH_TORCH>(b, grid, class_wd[k], table + k, d_state, s);
+                else
+                    launch_tensors_planned_arith<PS_ARITH_OPERATOR>(b, grid, class_wd[k], table + k, d_state, s);
+            });
+            if (rc) return rc;
+        }
+        return 0;
+    } catch (const std::exception&) {  // nothing may throw across the boundary
+        return fail(PS_ERR_BAD_ARG, "no host memory for a list of %d tensors", n_tensors);
+    }
 }
 
 int ps_restore_fp16_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_numel,
                            const ps_step_state* d_state, ps_stream_t stream)
 {
     ChunkList a;
-    if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, kTile)) return rc;
+    if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, nullptr, kTile)) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid, int) {
-        hipLaunchKernelGGL(restore_chunks_kernel, grid, dim3(kBlock), 0, s, b, chunk_numel, d_state);
+        hipLaunchKernelGGL(restore_chunks_kernel, grid, dim3(kBlock), 0, s, b, d_state);
     });
 }
 
@@ -882,15 +1107,18 @@ int ps_cast_fp32_to_fp16(const float* d_src, uint16_t* d_dst, size_t numel, ps_s
 int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, double beta2,
                         double epsilon, double weight_decay, int bias_correction,
                         const ps_chunk* chunks, int n_chunks, const ps_chunk* host_chunks,
-                        int n_host_chunks, size_t chunk_numel, const ps_chunk* staging, int n_slots,
-                        const ps_call_pattern* calls, double loss_scale, const ps_step_state* d_state,
-                        ps_stream_t stream)
+                        int n_host_chunks, size_t chunk_numel, const size_t* used_numel,
+                        const ps_chunk* staging, int n_slots, const ps_call_pattern* calls,
+                        double loss_scale, const ps_step_state* d_state, ps_stream_t stream)
 {
     auto o = find_opt(optimizer_id);
     if (!o) return fail(PS_ERR_UNKNOWN_ID, "optimizer id %d was never created", optimizer_id);
+    if (n_chunks < 0) return fail(PS_ERR_BAD_ARG, "n_chunks = %d is negative", n_chunks);
     ChunkList resident, host;
-    if (int rc = make_chunk_list(resident, chunks, n_chunks, chunk_numel, kTile)) return rc;
-    if (int rc = make_chunk_list(host, host_chunks, n_host_chunks, chunk_numel, kTile, false, "host chunk")) return rc;
+    if (int rc = make_chunk_list(resident, chunks, n_chunks, chunk_numel, used_numel, kTile)) return rc;
+    if (int rc = make_chunk_list(host, host_chunks, n_host_chunks, chunk_numel, used_numel ? used_numel + n_chunks : nullptr,
+                                 kTile, false, "host chunk"))
+        return rc;
     std::unique_ptr<bool[]> fp16_in_hbm(new (std::nothrow) bool[n_host_chunks > 0 ? n_host_chunks : 1]);
     if (!fp16_in_hbm) return fail(PS_ERR_BAD_ARG, "no host memory for a list of %d host chunks", n_host_chunks);
     if (n_host_chunks > 0) {
@@ -915,9 +1143,19 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, 
         const HyperParams hp{lr, beta1, beta2, epsilon, weight_decay, loss_scale, bias_correction != 0};
         if (arith == PS_ARITH_OPERATOR || n_host_chunks > 0) c_host = operator_step_consts(*o, step, hp, k.n_calls);
         c_resident = arith == PS_ARITH_TORCH ? torch_step_consts(*o, step, hp) : c_host;
+        if (!zeros_are_a_fixed_point(c_resident)) resident.used = nullptr;
+        if (n_host_chunks > 0 && !zeros_are_a_fixed_point(c_host)) host.used = nullptr;
+    } else {
+        // Streamed chunks move only their used part over the link, so whether their padding may be left alone has
+        // to be known here, from the host's numbers (the kernel's own check, on the device-resident scalars, stays
+        // in force for the resident chunks): a positive eps and finite scalars, betas below one as floats.
+        const bool plain = (float)epsilon > 0.0f && std::isfinite((float)lr) && std::isfinite((float)weight_decay) &&
+                           std::isfinite((float)epsilon) && (float)beta1 < 1.0f && (float)beta2 < 1.0f;
+        if (!plain) host.used = nullptr;
     }
     hipStream_t caller = static_cast<hipStream_t>(stream);
-    const bool stream_host = n_host_chunks > 0 && chunk_numel > 0;
+    bool stream_host = false;
+    for (int i = 0; i < n_host_chunks; ++i) stream_host = stream_host || host.numel_of(i) > 0;
     Pipeline* p = nullptr;
     std::unique_lock<std::mutex> turn;
     if (stream_host) {
@@ -929,15 +1167,16 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, 
     int rc = for_each_batch(resident, [&](const ChunkBatch& b, dim3 grid, int first) {
         const FirstCall fc = k.in_batch(first, (int)grid.y);
         if (d_state == nullptr)
-            launch_adam_batch(arith, b, grid, chunk_numel, c_resident, fc, caller);
+            launch_adam_batch(arith, b, grid, c_resident, fc, caller);
         else
             launch_gated_batch(arith, b, grid, chunk_numel, ga, fc, d_state, caller);
     });
-    if (rc) return rc;
-    if (!stream_host) return 0;
+    if (!stream_host) return rc;
 
-    const size_t b32 = chunk_numel * sizeof(float), b16 = chunk_numel * sizeof(uint16_t);
     auto stream_chunk = [&](int k_host) -> int {
+        const size_t numel = host.numel_of(k_host);
+        if (numel == 0) return 0;
+        const size_t b32 = numel * sizeof(float), b16 = numel * sizeof(uint16_t);
         const int s = k_host % n_slots;
         const ps_chunk& h = host_chunks[k_host];
         ps_chunk d = staging[s];
@@ -958,12 +1197,13 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, 
         ChunkBatch b;
         memset(&b, 0, sizeof(b));
         b.c[0] = d;
-        dim3 grid((unsigned)host.tiles_per_chunk, 1);
+        b.n[0] = numel;
+        dim3 grid((unsigned)((numel + kTile - 1) / kTile), 1);
         const FirstCall fc = k.in_batch((int64_t)n_chunks + k_host, 1);
         if (d_state == nullptr)
-            launch_adam_batch(PS_ARITH_OPERATOR, b, grid, chunk_numel, c_host, fc, p->compute);
-        else
-            launch_gated_batch(PS_ARITH_OPERATOR, b, grid, chunk_numel, ga, fc, d_state, p->compute);
+            launch_adam_batch(PS_ARITH_OPERATOR, b, grid, c_host, fc, p->compute);
+        else  // the staged copy ends at `numel`: nothing behind it for the kernel to decide about
+            launch_gated_batch(PS_ARITH_OPERATOR, b, grid, numel, ga, fc, d_state, p->compute);
         PS_HIP(hipGetLastError());
         PS_HIP(hipEventRecord(p->compute_done[s], p->compute));
 
@@ -980,33 +1220,36 @@ int ps_adam_step_hybrid(int optimizer_id, size_t step, double lr, double beta1, 
         return 0;
     };
     for (int i = 0; i < n_host_chunks && rc == 0; ++i) rc = stream_chunk(i);
-    // later work on the caller's stream sees every chunk written back (also if queuing stopped half way)
+    // later work on the caller's stream sees every chunk written back (also if queuing stopped half way, or never
+    // started because a resident launch failed: the side streams already wait on the caller, the caller must wait
+    // on them)
     const int joined = p->join(caller);
     return rc ? rc : joined;
 }
 
 int ps_overflow_scan_host_chunks(const ps_chunk* host_chunks, int n_chunks, size_t chunk_numel,
-                                 const ps_chunk* staging, int n_slots, ps_step_state* d_state,
-                                 ps_stream_t stream)
+                                 const size_t* used_numel, const ps_chunk* staging, int n_slots,
+                                 ps_step_state* d_state, ps_stream_t stream)
 {
     if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
     ChunkList a;
-    if (int rc = make_chunk_list(a, host_chunks, n_chunks, chunk_numel, kScanTile, true, "host chunk")) return rc;
+    if (int rc = make_chunk_list(a, host_chunks, n_chunks, chunk_numel, used_numel, kScanTile, true, "host chunk")) return rc;
     if (n_chunks == 0 || chunk_numel == 0) return 0;
     std::unique_ptr<bool[]> fp16_in_hbm(new (std::nothrow) bool[n_chunks]);
     if (!fp16_in_hbm) return fail(PS_ERR_BAD_ARG, "no host memory for a list of %d host chunks", n_chunks);
     bool any_on_host = false;
     if (int rc = fp16_payloads_in_hbm(host_chunks, n_chunks, fp16_in_hbm.get(), &any_on_host)) return rc;
     hipStream_t caller = static_cast<hipStream_t>(stream);
-    const size_t b16 = chunk_numel * sizeof(uint16_t);
-    const size_t n_tiles = a.tiles_per_chunk;
+    auto tiles_of = [&](int k) { return (a.numel_of(k) + kScanTile - 1) / kScanTile; };
     // fp16 payloads that live in HBM are probed in place on the caller's stream
     for (int k = 0; k < n_chunks; ++k) {
-        if (!fp16_in_hbm[k]) continue;
-        hipLaunchKernelGGL(scan_f16_kernel, dim3(grid_1d(n_tiles)), dim3(kScanBlock), kScanLdsBytes, caller,
-                           host_chunks[k].param_fp16, chunk_numel, n_tiles, d_state);
+        if (!fp16_in_hbm[k] || a.numel_of(k) == 0) continue;
+        hipLaunchKernelGGL(scan_f16_kernel, dim3(grid_1d(tiles_of(k))), dim3(kScanBlock), kScanLdsBytes, caller,
+                           host_chunks[k].param_fp16, a.numel_of(k), tiles_of(k), d_state);
         PS_HIP(hipGetLastError());
     }
+    any_on_host = false;
+    for (int k = 0; k < n_chunks; ++k) any_on_host = any_on_host || (!fp16_in_hbm[k] && a.numel_of(k) > 0);
     if (!any_on_host) return 0;
     if (int rc = check_slots(staging, n_slots, false, true)) return rc;
     Pipeline* p = nullptr;
@@ -1017,12 +1260,12 @@ int ps_overflow_scan_host_chunks(const ps_chunk* host_chunks, int n_chunks, size
     auto stream_chunk = [&](int k) -> int {
         const int s = streamed++ % n_slots;
         if (p->slot_used[s]) PS_HIP(hipStreamWaitEvent(p->h2d, p->compute_done[s], 0));
-        PS_HIP(hipMemcpyAsync(staging[s].param_fp16, host_chunks[k].param_fp16, b16,
+        PS_HIP(hipMemcpyAsync(staging[s].param_fp16, host_chunks[k].param_fp16, a.numel_of(k) * sizeof(uint16_t),
                               hipMemcpyHostToDevice, p->h2d));
         PS_HIP(hipEventRecord(p->h2d_done[s], p->h2d));
         PS_HIP(hipStreamWaitEvent(p->compute, p->h2d_done[s], 0));
-        hipLaunchKernelGGL(scan_f16_kernel, dim3(grid_1d(n_tiles)), dim3(kScanBlock), kScanLdsBytes, p->compute,
-                           staging[s].param_fp16, chunk_numel, n_tiles, d_state);
+        hipLaunchKernelGGL(scan_f16_kernel, dim3(grid_1d(tiles_of(k))), dim3(kScanBlock), kScanLdsBytes, p->compute,
+                           staging[s].param_fp16, a.numel_of(k), tiles_of(k), d_state);
         PS_HIP(hipGetLastError());
         PS_HIP(hipEventRecord(p->compute_done[s], p->compute));
         p->slot_used[s] = true;
@@ -1030,7 +1273,7 @@ int ps_overflow_scan_host_chunks(const ps_chunk* host_chunks, int n_chunks, size
     };
     int rc = 0;
     for (int k = 0; k < n_chunks && rc == 0; ++k)
-        if (!fp16_in_hbm[k]) rc = stream_chunk(k);
+        if (!fp16_in_hbm[k] && a.numel_of(k) > 0) rc = stream_chunk(k);
     const int joined = p->join(caller);
     return rc ? rc : joined;
 }
@@ -1061,6 +1304,8 @@ int ps_state_init(ps_step_state* d_state, double init_scale, int init_is_int, do
     s.beta2 = (float)beta2;
     // Adam_Optimizer starts with beta^t = 1 and step 0; the first update multiplies once.
     s.operator_step = 0;
+    s.operator_beta1 = s.beta1;
+    s.operator_beta2 = s.beta2;
     s.beta1_t_cur = 1.0f;
     s.beta2_t_cur = 1.0f;
     s.beta1_t_next = 1.0f * s.beta1;
@@ -1141,14 +1386,14 @@ int ps_overflow_scan_f32(const float* d_grads_fp32, size_t numel, ps_step_state*
 }
 
 int ps_overflow_scan_chunks(const ps_chunk* chunks, int n_chunks, size_t chunk_numel,
-                            ps_step_state* d_state, ps_stream_t stream)
+                            const size_t* used_numel, ps_step_state* d_state, ps_stream_t stream)
 {
     if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
     ChunkList a;
-    if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, kScanTile)) return rc;
+    if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, used_numel, kScanTile, true)) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     return for_each_batch(a, [&](const ChunkBatch& b, dim3 grid, int) {
-        hipLaunchKernelGGL(scan_chunks_kernel, grid, dim3(kScanBlock), kScanLdsBytes, s, b, chunk_numel, d_state);
+        hipLaunchKernelGGL(scan_chunks_kernel, grid, dim3(kScanBlock), kScanLdsBytes, s, b, d_state);
     });
 }
 
@@ -1157,26 +1402,27 @@ int ps_overflow_scan_chunks_noalloc(const ps_chunk* chunks, int n_chunks, size_t
 {
     if (!d_flag) return fail(PS_ERR_BAD_ARG, "d_flag is NULL");
     ChunkList a;
-    if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, kPartialTile)) return rc;
-    if (n_chunks == 0 || a.tiles_per_chunk == 0) return 0;
+    if (int rc = make_chunk_list(a, chunks, n_chunks, chunk_numel, nullptr, kPartialTile)) return rc;
+    const size_t tiles_per_chunk = (chunk_numel + kPartialTile - 1) / kPartialTile;
+    if (n_chunks == 0 || tiles_per_chunk == 0) return 0;
     // one scratch word per workgroup of the first kernel
-    const size_t max_chunks = kScratchWords / a.tiles_per_chunk;  // 0 when one chunk alone is too long
+    const size_t max_chunks = kScratchWords / tiles_per_chunk;  // 0 when one chunk alone is too long
     if ((size_t)n_chunks > max_chunks)
         return fail(PS_ERR_BAD_ARG,
                     "%d chunks of %zu elements need %zu scratch words; this entry point holds %zu (at most %zu "
                     "elements per call): split the list or use ps_overflow_scan_chunks",
-                    n_chunks, chunk_numel, (size_t)n_chunks * a.tiles_per_chunk, kScratchWords,
+                    n_chunks, chunk_numel, (size_t)n_chunks * tiles_per_chunk, kScratchWords,
                     kScratchWords * (size_t)kPartialTile);
     uint32_t* scratch = nullptr;
     if (int rc = scratch_address(&scratch)) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     int rc = for_each_batch(a, [&](const ChunkBatch& b, dim3 grid, int first) {
-        hipLaunchKernelGGL(scan_chunks_partial_kernel, grid, dim3(kAuxBlock), 0, s, b, chunk_numel,
-                           scratch + (size_t)first * a.tiles_per_chunk);
+        hipLaunchKernelGGL(scan_chunks_partial_kernel, grid, dim3(kAuxBlock), 0, s, b,
+                           scratch + (size_t)first * tiles_per_chunk);
     });
     if (rc) return rc;
     hipLaunchKernelGGL(scan_reduce_kernel, dim3(1), dim3(kReduceBlock), 0, s, scratch,
-                       (size_t)n_chunks * a.tiles_per_chunk, d_flag);
+                       (size_t)n_chunks * tiles_per_chunk, d_flag);
     PS_HIP(hipGetLastError());
     return 0;
 }

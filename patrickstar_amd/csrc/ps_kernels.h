@@ -14,9 +14,10 @@ namespace {
 constexpr int kBatch = 64;
 struct ChunkBatch {
     ps_chunk c[kBatch];
+    size_t n[kBatch];  // elements of each chunk the launch covers: the chunk's length, or less when only zeros follow
 };
-static_assert(sizeof(ps_chunk) == 32 && sizeof(ps_step_state) == 192 && sizeof(ps_scale_record) == 16 &&
-                  sizeof(ps_call_pattern) == 32,
+static_assert(sizeof(ps_chunk) == 32 && sizeof(ps_step_state) == 256 && sizeof(ps_scale_record) == 16 &&
+                  sizeof(ps_call_pattern) == 32 && sizeof(ps_tensor_call) == 56,
               "layout of the boundary structs");
 
 // Host-decided step: all scalars arrive as kernel arguments and the
@@ -31,11 +32,15 @@ __device__ __forceinline__ void first_call_span(const FirstCall& fc, size_t* lo,
 
 template <int ARITH, int WD, int UNS>
 __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
-    adam_chunks_kernel(ChunkBatch b, size_t chunk_numel, StepConsts c, FirstCall fc)
+    adam_chunks_kernel(ChunkBatch b, StepConsts c, FirstCall fc)
 {
+    // b.n: the host has already decided whether the zeros behind a chunk's last tensor may be left alone
+    const size_t numel = b.n[blockIdx.y];
+    const size_t base = (size_t)blockIdx.x * kTile;
+    if (base >= numel) return;  // the grid is as wide as the longest chunk of the batch
     size_t lo, hi;
     first_call_span(fc, &lo, &hi);
-    adam_tile<ARITH, WD, UNS>(c, b.c[blockIdx.y], (size_t)blockIdx.x * kTile, chunk_numel, lo, hi);
+    adam_tile<ARITH, WD, UNS>(c, b.c[blockIdx.y], base, numel, lo, hi);
 }
 
 struct GatedArgs {
@@ -102,6 +107,16 @@ __device__ __forceinline__ StepConsts gated_consts(const GatedArgs& ga, const St
     return c;
 }
 
+// Zeros in all four lists stay zeros under these constants (so the padding behind a chunk's last tensor need not
+// be touched): the denominator sqrt(0) * bc2inv + eps is a positive number and nothing multiplies a zero by an
+// infinity or a NaN.  With eps == 0 the reference's arithmetic writes 0 / 0 into the padding; then it is computed.
+__host__ __device__ inline bool zeros_are_a_fixed_point(const StepConsts& c)
+{
+    const float s = c.step_size + c.first_step_size + c.bc2inv + c.first_bc2inv + c.wd_term + c.scale + c.beta1 +
+                    c.beta2 + c.b1m + c.b2m + c.eps;
+    return c.eps > 0.0f && (s - s) == 0.0f;  // every term finite (no NaN, and no infinities: inf - inf is NaN)
+}
+
 template <int ARITH, int WD>
 __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
     adam_chunks_gated_kernel(ChunkBatch b, size_t chunk_numel, GatedArgs ga, FirstCall fc,
@@ -109,16 +124,22 @@ __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
 {
     const ps_chunk& ch = b.c[blockIdx.y];
     const size_t base = (size_t)blockIdx.x * kTile;
+    size_t numel = b.n[blockIdx.y];  // what lies behind it is zeros in all four lists
     const StateView sv = view_state(st);
     if (sv.overflow) {
-        restore_tile(ch.param_fp32, ch.param_fp16, base, chunk_numel);
+        restore_tile(ch.param_fp32, ch.param_fp16, base, numel);  // RNE(0) = 0 is already there
         return;
     }
     const bool here = fc.chunk == (int)blockIdx.y;
     size_t lo, hi;
     first_call_span(fc, &lo, &hi);
+    if (base + kTile > numel && numel < chunk_numel) {
+        // a tile that reaches into the padding: leave the zeros alone only if they are a fixed point of this step
+        if (!zeros_are_a_fixed_point(gated_consts<ARITH>(ga, sv, here))) numel = chunk_numel;
+        if (base >= numel) return;
+    }
     adam_tile_late_consts<ARITH, WD, UNSCALE_RUNTIME>([&]() { return gated_consts<ARITH>(ga, sv, here); }, ch, base,
-                                                      chunk_numel, lo, hi);
+                                                      numel, lo, hi);
 }
 
 // ------------------------------------------------------- tensor-list kernels
@@ -219,12 +240,51 @@ __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
                                                       numel, 0, first ? numel : 0);
 }
 
+// Step constants of one distinct call of a device-decided step whose tensors carry their own step numbers and
+// hyper-parameters, formed on the device by plan_consts_kernel (below) before the update kernels run.
+struct PlannedConsts {
+    StepConsts c;
+    float beta1_t, beta2_t;  // the operator object's beta^t after this call (unused by the torch formula)
+};
+static_assert(sizeof(PlannedConsts) == 64, "one 64-byte record per class in the caller's workspace");
+
+// The tensor-list step with the constants of the launch's tensors read from device memory: every tensor of the
+// launch belongs to one class of calls.  No tensor is "the first call" here: a first call that differs is a class
+// of its own.
+template <int ARITH, int WD>
 __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
-    restore_chunks_kernel(ChunkBatch b, size_t chunk_numel, const ps_step_state* __restrict__ st)
+    adam_tensors_planned_kernel(TensorBatch b, const PlannedConsts* __restrict__ consts,
+                                const ps_step_state* __restrict__ st)
+{
+    const int k = blockIdx.y;
+    const uint64_t nh = b.numel_head[k];
+    const size_t numel = (size_t)(nh & kNumelMask);
+    const int head = (int)(nh >> 56);
+    const ptrdiff_t tile = (ptrdiff_t)blockIdx.x - (head ? 1 : 0);
+    const size_t base = tile < 0 ? 0 : (size_t)tile * kTile;
+    if (tile >= 0 && base >= numel) return;
+    if (st->overflow) {
+        if (tile < 0) {
+            for (int j = threadIdx.x; j < head; j += kBlock)
+                b.t[k].param_fp16[(ptrdiff_t)j - head] = (uint16_t)float_to_half_bits(b.t[k].param_fp32[(ptrdiff_t)j - head]);
+        } else {
+            restore_tile(b.t[k].param_fp32, b.t[k].param_fp16, base, numel);
+        }
+        return;
+    }
+    if (tile < 0) {
+        adam_head<ARITH, WD, UNSCALE_RUNTIME>(consts->c, b.t[k], head, false);
+        return;
+    }
+    adam_tile_late_consts<ARITH, WD, UNSCALE_RUNTIME>([&]() { return consts->c; }, b.t[k], base, numel, 0, 0);
+}
+
+__global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
+    restore_chunks_kernel(ChunkBatch b, const ps_step_state* __restrict__ st)
 {
     if (st != nullptr && !st->overflow) return;
     const ps_chunk& ch = b.c[blockIdx.y];
-    restore_tile(ch.param_fp32, ch.param_fp16, (size_t)blockIdx.x * kTile, chunk_numel);
+    restore_tile(ch.param_fp32, ch.param_fp16, (size_t)blockIdx.x * kTile, b.n[blockIdx.y]);
 }
 
 __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
@@ -430,19 +490,19 @@ __global__ void __launch_bounds__(kAuxBlock)
 }
 
 __global__ void __launch_bounds__(kScanBlock)
-    scan_chunks_kernel(ChunkBatch b, size_t chunk_numel, ps_step_state* st)
+    scan_chunks_kernel(ChunkBatch b, ps_step_state* st)
 {
-    uint32_t hit = scan_tile_f16<kScanBlock, kScanUnroll>(b.c[blockIdx.y].param_fp16, chunk_numel, blockIdx.x);
+    uint32_t hit = scan_tile_f16<kScanBlock, kScanUnroll>(b.c[blockIdx.y].param_fp16, b.n[blockIdx.y], blockIdx.x);
     block_flag_commit<kScanBlock>(hit, &st->overflow);
 }
 
 // The same probe without atomics and without a caller-side state: every workgroup leaves the OR over its tile in
 // its own word of a partial-result array; a second, single-workgroup kernel ORs those words into the caller's flag.
 __global__ void __launch_bounds__(kAuxBlock)
-    scan_chunks_partial_kernel(ChunkBatch b, size_t chunk_numel, uint32_t* __restrict__ partial)
+    scan_chunks_partial_kernel(ChunkBatch b, uint32_t* __restrict__ partial)
 {
     __shared__ uint32_t wave_hit[kAuxBlock / 64];
-    uint32_t hit = scan_tile_f16<kAuxBlock, kPartialUnroll>(b.c[blockIdx.y].param_fp16, chunk_numel, blockIdx.x);
+    uint32_t hit = scan_tile_f16<kAuxBlock, kPartialUnroll>(b.c[blockIdx.y].param_fp16, b.n[blockIdx.y], blockIdx.x);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) hit |= (uint32_t)__shfl_xor((int)hit, off, 64);
     if ((threadIdx.x & 63) == 0) wave_hit[threadIdx.x >> 6] = hit;
@@ -592,14 +652,16 @@ __global__ void state_seed_kernel(ps_step_state* st, SeedArgs a)
     if (threadIdx.x == 0 && blockIdx.x == 0) {
         // IncrementStep (cpu_adam.h:143-162) for the first call of step adam_step + 1: changed betas restart from
         // pow; else the running product continues only if the object's own step is adam_step
-        const bool same_betas = st->beta1 == a.beta1 && st->beta2 == a.beta2;
         if (a.fresh_operator) {
-            // a new native object (cpu_adam.h:68-86): step 0, beta^t = 1
+            // a new native object (cpu_adam.h:68-86), created with these betas: step 0, beta^t = 1
             st->operator_step = 0;
             st->beta1_t_cur = 1.0f;
             st->beta2_t_cur = 1.0f;
+            st->operator_beta1 = a.beta1;
+            st->operator_beta2 = a.beta2;
         }
-        const bool follows = (a.fresh_operator || same_betas) && st->operator_step == a.adam_step;
+        const bool same_betas = st->operator_beta1 == a.beta1 && st->operator_beta2 == a.beta2;
+        const bool follows = same_betas && st->operator_step == a.adam_step;
         st->adam_step = a.adam_step;
         st->beta1 = a.beta1;
         st->beta2 = a.beta2;
@@ -638,6 +700,99 @@ __device__ inline double pow_int(double base, int64_t n)
         if (n) x = two_double_mul(x, x);
     }
     return r.hi;
+}
+
+// ------------------------------------- per-tensor step numbers: constants of a device-decided step
+//
+// One distinct call of the step (ps_adam_step_tensors_each): its hyper-parameters, its distance d from the device's
+// step counter, and how Adam_Optimizer::IncrementStep (cpu_adam.h:143-162) treats it, which the host can tell from
+// the call before it:
+//   PLAN_FIRST  the step's first operator call: continues the object's running product if the object, as the last
+//               clean step left it, stands at this call's step minus one with the same betas; else pow
+//   PLAN_MUL    its step number is the previous call's plus one, same betas: the previous call's beta^t times beta
+//   PLAN_POW    anything else: (float)pow((double)beta, step)
+//   PLAN_TORCH  the torch formula: 1 - beta ** step in binary64, no operator call
+enum { PLAN_POW = 0, PLAN_FIRST = 1, PLAN_MUL = 2, PLAN_TORCH = 3 };
+struct PlanClass {
+    double lr, beta1, beta2, eps, wd;
+    int64_t d;     // the call's step number is adam_step + 1 + d
+    int32_t mode;
+    int32_t prev;  // PLAN_MUL: the class (index in the table) of the call before it
+};
+constexpr int kPlanBatch = 32;
+struct PlanBatch {
+    PlanClass k[kPlanBatch];
+};
+struct PlanArgs {
+    double grad_clamp;
+    int64_t last_d;             // of the step's last operator call
+    int adamw, bias_correction;
+    int first_class, n;         // this launch covers classes [first_class, first_class + n) of the table
+    int is_last_launch;         // the launch that leaves the pending record
+    int last_operator_class;    // class of the step's last operator call; -1: the step calls the operator for nothing
+    float last_beta1, last_beta2;
+};
+
+__global__ void __launch_bounds__(64)
+    plan_consts_kernel(PlanBatch pb, PlanArgs a, ps_step_state* st, PlannedConsts* table)
+{
+    __shared__ float b1t_of[kPlanBatch], b2t_of[kPlanBatch];
+    const int j = threadIdx.x;
+    const int64_t adam_step = st->adam_step;
+    const double cur_scale = st->cur_scale;
+    const float clip = clamp_bound(a.grad_clamp, cur_scale);
+    const bool bias = a.bias_correction != 0;
+    if (j < a.n && pb.k[j].mode != PLAN_MUL) {
+        const PlanClass& k = pb.k[j];
+        const int64_t t = adam_step + 1 + k.d;
+        PlannedConsts out;
+        if (k.mode == PLAN_TORCH) {
+            torch_consts(out.c, k.lr, k.beta1, k.beta2, k.eps, k.wd, a.adamw != 0, bias ? 1.0 - pow_int(k.beta1, t) : 1.0,
+                         bias ? 1.0 - pow_int(k.beta2, t) : 1.0, cur_scale, clip);
+            out.beta1_t = out.beta2_t = 0.0f;
+        } else {
+            const float b1 = (float)k.beta1, b2 = (float)k.beta2;
+            const bool follows = k.mode == PLAN_FIRST && st->operator_beta1 == b1 && st->operator_beta2 == b2 &&
+                                 st->operator_step + 1 == t;
+            out.beta1_t = follows ? st->beta1_t_cur * b1 : (float)pow_int((double)b1, t);
+            out.beta2_t = follows ? st->beta2_t_cur * b2 : (float)pow_int((double)b2, t);
+            finish_consts(out.c, (float)k.lr, b1, b2, (float)k.eps, (float)k.wd, a.adamw != 0, out.beta1_t, out.beta2_t,
+                          bias, (float)cur_scale, clip);
+        }
+        b1t_of[j] = out.beta1_t;
+        b2t_of[j] = out.beta2_t;
+        table[a.first_class + j] = out;
+    }
+    __syncthreads();
+    if (j != 0) return;
+    // a call that multiplies needs the call before it: in order, by one lane
+    for (int i = 0; i < a.n; ++i) {
+        const PlanClass& k = pb.k[i];
+        if (k.mode != PLAN_MUL) continue;
+        const int q = k.prev - a.first_class;  // an earlier class: of this launch, or of a launch before it
+        const float p1 = q >= 0 ? b1t_of[q] : table[k.prev].beta1_t;
+        const float p2 = q >= 0 ? b2t_of[q] : table[k.prev].beta2_t;
+        PlannedConsts out;
+        const float b1 = (float)k.beta1, b2 = (float)k.beta2;
+        out.beta1_t = p1 * b1;
+        out.beta2_t = p2 * b2;
+        finish_consts(out.c, (float)k.lr, b1, b2, (float)k.eps, (float)k.wd, a.adamw != 0, out.beta1_t, out.beta2_t, bias,
+                      (float)cur_scale, clip);
+        b1t_of[i] = out.beta1_t;
+        b2t_of[i] = out.beta2_t;
+        table[a.first_class + i] = out;
+    }
+    if (!a.is_last_launch) return;
+    if (a.last_operator_class < 0) {
+        st->pending_operator_step = 0;
+        return;
+    }
+    const int q = a.last_operator_class - a.first_class;
+    st->pending_beta1_t = q >= 0 ? b1t_of[q] : table[a.last_operator_class].beta1_t;
+    st->pending_beta2_t = q >= 0 ? b2t_of[q] : table[a.last_operator_class].beta2_t;
+    st->pending_beta1 = a.last_beta1;
+    st->pending_beta2 = a.last_beta2;
+    st->pending_operator_step = adam_step + 1 + a.last_d;
 }
 
 __global__ void state_set_scaler_kernel(ps_step_state* st, double cur_scale, int scale_is_int,
@@ -690,18 +845,27 @@ __global__ void scaler_update_kernel(ps_step_state* st, int flag_mode, ps_scale_
         // the step ran: state["step"] += 1
         const int64_t t = s.adam_step + 1;
         s.adam_step = t;
-        if (operator_calls >= 1) {
+        if (s.pending_operator_step != 0) {
+            // a step whose tensors carried their own step numbers and betas: what its last call left
+            s.operator_step = s.pending_operator_step;
+            s.beta1_t_cur = s.pending_beta1_t;
+            s.beta2_t_cur = s.pending_beta2_t;
+            s.operator_beta1 = s.pending_beta1;
+            s.operator_beta2 = s.pending_beta2;
+        } else if (operator_calls >= 1) {
             // what the operator object holds after its last call of step t: the first call's beta^t if it
             // was the only one, else pow(beta, t) from the second call on
             s.beta1_t_cur = operator_calls == 1 ? s.beta1_t_next : s.beta1_t_rest;
             s.beta2_t_cur = operator_calls == 1 ? s.beta2_t_next : s.beta2_t_rest;
             s.operator_step = t;
+            s.operator_beta1 = s.beta1;
+            s.operator_beta2 = s.beta2;
         }
         // step t + 1: every call after the first evaluates (float)pow((double)beta, t + 1); the first call
         // multiplies the held value by beta if the object's step is t, else it evaluates pow as well
         s.beta1_t_rest = (float)pow_int((double)s.beta1, t + 1);
         s.beta2_t_rest = (float)pow_int((double)s.beta2, t + 1);
-        const bool follows = s.operator_step == t;
+        const bool follows = s.operator_step == t && s.operator_beta1 == s.beta1 && s.operator_beta2 == s.beta2;
         s.beta1_t_next = follows ? s.beta1_t_cur * s.beta1 : s.beta1_t_rest;
         s.beta2_t_next = follows ? s.beta2_t_cur * s.beta2 : s.beta2_t_rest;
         // fp16_cpu_adam.py:412-413 for the next step
@@ -718,6 +882,7 @@ __global__ void scaler_update_kernel(ps_step_state* st, int flag_mode, ps_scale_
     s.cur_iter += 1;
     s.last_skipped = overflow ? 1u : 0u;
     s.overflow = 0;
+    s.pending_operator_step = 0;
     *st = s;
 }
 

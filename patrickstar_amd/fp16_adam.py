@@ -26,6 +26,7 @@ kernels, on chunks resident in HBM and keeps the operator's for host-resident
 chunks -- bit for bit what the reference computes under the same placement.
 """
 import ctypes
+import logging
 import weakref
 from copy import deepcopy
 
@@ -34,6 +35,9 @@ import torch
 from . import _lib, adam_op
 from .chunk_layout import AccessType, ChunkType, ParamType, register_param
 from .loss_scaler import DynamicLossScaler
+
+
+logger = logging.getLogger("patrickstar_amd")
 
 
 def _empty_fp32_param():
@@ -58,11 +62,13 @@ class _ParamState(dict):
         return super().__getitem__(key)
 
     def __setitem__(self, key, value):
+        if key == "step":
+            self._sync()  # settle every parameter's entry before one of them is overwritten
         super().__setitem__(key, value)
-        if key in ("lr", "betas", "eps", "weight_decay"):
+        if key in ("lr", "betas", "eps", "weight_decay", "step"):
             owner = self._owner()
             if owner is not None:
-                owner._hyper_checked = False  # the next step() looks at every parameter's entries again
+                owner._plan = None  # the next step() looks at every parameter's entries again
 
     def items(self):
         self._sync()
@@ -120,9 +126,15 @@ class FP16Adam(torch.optim.Optimizer):
         self._dynamic = isinstance(loss_scaler, DynamicLossScaler)
         self._host_overflow = False
         self._steps_dirty = False
-        self._hyper_checked = False  # every trainable parameter's state entries hold the same hyper-parameters
-        self._host_step = None  # shared step counter of the host-decided path; taken from state[p]["step"] at first use
-        self.staging_slots = 2  # HBM staging slots for host-resident chunks (double buffering)
+        # What one step does, derived from requires_grad and the state[p] entries of every parameter (_make_plan);
+        # None: look again.  The reference reads all of it per parameter on every step (fp16_cpu_adam.py:569-606).
+        self._plan = None
+        # The common step counter: every trainable parameter's state[p]["step"] is this number plus the parameter's
+        # own distance (0 for all of them in the ordinary case).  Host-decided steps count here; device-decided steps
+        # count in the loss scaler's device state (adam_step) and this is what it was seeded with.
+        self._common_step = 0
+        self._offsets = {}  # parameter -> its distance from the common counter (only parameters that have one)
+        self.staging_slots = 3  # HBM staging slots for host-resident chunks (one being filled, one computed on, one drained)
 
         assert len(self.param_groups) == 1, "Only support one param group at the moment."
         # Eager state initialisation: m and v are chunk tensors shadowing the fp16 parameter chunks.
@@ -169,10 +181,13 @@ class FP16Adam(torch.optim.Optimizer):
         self._tensor_table = None  # (ps_chunk rows, numels, count) when the step has to go tensor by tensor
         self._calls = None  # ps_call_pattern of one step (None: no operator call at all)
         self._stages = None  # the entry-point calls of a step that cannot be made as one (see _plan_stages)
-        self._trainable_seen = None  # requires_grad of every parameter when the tables were built
+        self._trainable_seen = None  # requires_grad of every parameter when the plan was made
         self._operator_calls = 0
+        self._overflow_log_read = 0  # loss-scaler iterations whose outcome has been looked at for the overflow warning
         if self._dynamic and torch.cuda.is_available():
             self.loss_scaler.materialize(self.client.device, betas=betas)
+            self.loss_scaler.enable_log(self.OVERFLOW_LOG_CAPACITY)
+            self.loss_scaler.on_read = weakref.WeakMethod(self._warn_about_overflows)
 
     def __del__(self):
         # the native object is per id and process-global: drop it with the optimizer
@@ -226,14 +241,19 @@ class FP16Adam(torch.optim.Optimizer):
             info.tensor_id not in live_ids for cid in live_chunks for info in index.generate_tensor_info_in_order(cid)
         )
         dev_rows, host_positions, where = [], [], {}
+        dev_used, host_used = [], []
         for pos in self.client.positions():
             if pos.fp16 not in live_chunks or pos.exp_avg is None or pos.exp_avg_sq is None:
                 continue  # a chunk position without trainable parameters
+            # elements in front of the chunk's zero padding: where its last tensor ends
+            used = max((info.start_offset + info.numel for info in index.generate_tensor_info_in_order(pos.fp16)), default=0)
             if pos.on_host:
                 where[pos.fp16] = ("host", len(host_positions))
                 host_positions.append(pos)
+                host_used.append(used)
             else:
                 where[pos.fp16] = ("hbm", len(dev_rows))
+                dev_used.append(used)
                 dev_rows.append(
                     [
                         cl[pos.fp32].payload.data_ptr(),
@@ -262,14 +282,18 @@ class FP16Adam(torch.optim.Optimizer):
             )
         table = _lib.chunk_array(dev_rows) if dev_rows else None
         self._tables = (table, len(dev_rows), host_positions)
+        # the padding behind a chunk's last tensor is zeros in all four lists and stays zeros: the kernels skip it
+        full = self.client.default_chunk_size
+        self._used = _lib.size_array(dev_used) if any(u != full for u in dev_used) else None
+        self._used_all = _lib.size_array(dev_used + host_used) if any(u != full for u in dev_used + host_used) else None
         self._stages = None
         if host_positions:
             from .hybrid import HostChunkStreamer
 
             if partly_frozen:
-                self._plan_stages(trainable, chunk_of, where, host_positions, called, live_ids)
+                self._plan_stages(trainable, chunk_of, where, host_positions, called, live_ids, host_used)
             else:
-                self._streamer = HostChunkStreamer(self.client, host_positions, n_slots=self.staging_slots)
+                self._streamer = HostChunkStreamer(self.client, host_positions, n_slots=self.staging_slots, used=host_used)
         return self._tables
 
     def _tensor_rows(self, params, slot=None):
@@ -295,7 +319,7 @@ class FP16Adam(torch.optim.Optimizer):
             numels.append(p.ps_attr.numel)
         return _lib.chunk_array(rows), (ctypes.c_size_t * len(numels))(*numels), len(numels)
 
-    def _plan_stages(self, trainable, chunk_of, where, host_positions, called, live_ids):
+    def _plan_stages(self, trainable, chunk_of, where, host_positions, called, live_ids, host_used):
         """Chunks that mix trainable and frozen tensors TOGETHER WITH host-resident positions: the step is spread over
         several entry-point calls, all under one call pattern (the stage that holds the step's first operator call
         goes first and names it):
@@ -311,7 +335,8 @@ class FP16Adam(torch.optim.Optimizer):
         for k, pos in enumerate(host_positions):
             frozen_here = any(info.tensor_id not in live_ids for info in index.generate_tensor_info_in_order(pos.fp16))
             (part if frozen_here else whole).append(k)
-        self._streamer = HostChunkStreamer(self.client, host_positions, n_slots=self.staging_slots, step_indices=whole)
+        self._streamer = HostChunkStreamer(self.client, host_positions, n_slots=self.staging_slots, step_indices=whole,
+                                           used=host_used)
         n_calls = len(called)
         first = called[0] if called else None
         first_info = index.get_tensor_info(first.ps_attr.data_id()) if first is not None else None
@@ -370,7 +395,7 @@ class FP16Adam(torch.optim.Optimizer):
                 tensors(stage[1], stage[2])
             elif stage[0] == "stream":
                 self._streamer.step(self.opt_id, step_no, lr, beta1, beta2, eps, weight_decay, loss_scale, None, 0,
-                                    stage[1], scaler)
+                                    stage[1], scaler, self._streamer.host_used_of_step)
             else:
                 _, payloads, staging, table, pat = stage
                 moved = [(s, h) for s, h in zip(staging, payloads) if h.device.type == "cpu"]
@@ -391,6 +416,8 @@ class FP16Adam(torch.optim.Optimizer):
     def invalidate_tables(self):
         """Call after re-allocating chunk payloads."""
         self._tables = None
+        if self._plan is not None and self._plan["kind"] == "each":
+            self._plan["table"] = None
 
     # -- overflow flag ------------------------------------------------------------
     @property
@@ -448,7 +475,7 @@ class FP16Adam(torch.optim.Optimizer):
         if n_dev:
             _lib.check(
                 self._lib.ps_overflow_scan_chunks(
-                    table, n_dev, self.client.default_chunk_size, self.loss_scaler.state_ptr, stream
+                    table, n_dev, self.client.default_chunk_size, self._used, self.loss_scaler.state_ptr, stream
                 ),
                 "ps_overflow_scan_chunks",
             )
@@ -456,75 +483,129 @@ class FP16Adam(torch.optim.Optimizer):
             self._streamer.scan_gradients(self.loss_scaler)
 
     # -- the step -----------------------------------------------------------------
+    def _entries(self, p):
+        """(lr, betas, eps, weight_decay, step) of one parameter as its ``state[p]`` holds them."""
+        g, st = dict.__getitem__, self.state[p]
+        return g(st, "lr"), tuple(g(st, "betas")), g(st, "eps"), g(st, "weight_decay"), g(st, "step")
+
     def _hyper(self):
-        """(lr, betas, eps, weight_decay) of the step: the entries of ``state[p]``, as the reference reads them per
-        tensor (``fp16_cpu_adam.py:593-598``).  The fused step applies ONE set to every tensor, so entries that differ
-        between parameters (somebody wrote ``state[p]["lr"]`` for some parameters only) are refused, not ignored."""
-        g = dict.__getitem__
-        first = None
-        for group in self.param_groups:
-            for p in group["params"]:
-                if not p.requires_grad:
-                    continue
-                st = self.state[p]
-                mine = (g(st, "lr"), g(st, "betas"), g(st, "eps"), g(st, "weight_decay"))
-                if first is None:
-                    first = mine
-                    if self._hyper_checked:
-                        return first
-                elif (mine[0], tuple(mine[1]), mine[2], mine[3]) != (first[0], tuple(first[1]), first[2], first[3]):
-                    raise ValueError(
-                        "optimizer.state holds different hyper-parameters for different parameters "
-                        f"({first} and {mine}); this step applies one lr / betas / eps / weight_decay to all of them"
-                    )
-        self._hyper_checked = True
-        return first
+        """(lr, betas, eps, weight_decay) of the step when every trainable parameter's ``state[p]`` holds the same
+        (None when nothing is trainable, ``"each"`` when they differ)."""
+        plan = self._plan or self._make_plan()
+        return plan["hyper"] if plan["kind"] == "uniform" else (None if plan["kind"] == "empty" else "each")
+
+    def _make_plan(self):
+        """What one step does, from ``requires_grad`` and the ``state[p]`` entries of every parameter.
+
+        The reference counts ``state[p]["step"]`` per parameter and reads lr / betas / eps / weight_decay per
+        parameter, on every step (``fp16_cpu_adam.py:569-606``), and hands each operator call its tensor's own
+        numbers (``:403-428``).  Ordinarily all trainable parameters agree: then ONE counter (on the host, or in the
+        device-resident state of a dynamic loss scaler) stands for all of them and the whole chunk list goes to one
+        fused call ("uniform").  If they do not (a parameter that was frozen for some steps stands behind; somebody
+        wrote ``state[p]["lr"]`` for some parameters; a checkpoint said so) the step goes tensor by tensor through
+        ``ps_adam_step_tensors_each``, every tensor with its own numbers ("each"): its step number is kept as a
+        distance from the common counter, which is all a device-decided step needs to know on the host.
+        Made again whenever ``requires_grad`` of some parameter or a ``state[p]`` entry has changed.
+        """
+        self._sync_steps()  # every state[p]["step"] is now what the steps so far made it
+        params = self.param_groups[0]["params"]
+        self._trainable_seen = tuple(p.requires_grad for p in params)
+        self._tables = None
+        trainable = self._trainable()
+        if not trainable:
+            self._offsets = {}
+            self._plan = {"kind": "empty"}
+            return self._plan
+        entries = [self._entries(p) for p in trainable]
+        common = entries[0][4]
+        self._offsets = {p: e[4] - common for p, e in zip(trainable, entries) if e[4] != common}
+        if all(e == entries[0] for e in entries):
+            self._plan = {"kind": "uniform", "hyper": entries[0][:4]}
+        else:
+            self._plan = {"kind": "each", "trainable": trainable, "entries": entries, "table": None}
+        # the common counter moves to the first trainable parameter's step number (a checkpoint was loaded, or the
+        # parameters that defined it were frozen); for a device-decided step also the betas of the whole-list kernels
+        betas = entries[0][1]
+        if self._dynamic:
+            if self.loss_scaler._state is not None and (
+                common != self._common_step or (float(betas[0]), float(betas[1])) != self.loss_scaler._betas
+            ):
+                # the operator object behind this optimizer stays the one it was (the reference's load_state_dict,
+                # fp16_cpu_adam.py:660-694, does not touch it): whether its running beta^t product continues is
+                # decided on the device, as Adam_Optimizer::IncrementStep would (cpu_adam.h:143-162)
+                self.loss_scaler._seed_step(common, fresh_operator=False, betas=betas)
+        self._common_step = common
+        return self._plan
 
     def _stepped_params(self):
-        """The parameters the steps so far have updated: those that were trainable when the tables were last built
+        """The parameters the steps so far have updated: those that were trainable when the plan was last made
         (before the first step: those that are trainable now)."""
         params = self.param_groups[0]["params"]
         flags = self._trainable_seen if self._trainable_seen is not None else [p.requires_grad for p in params]
         return [p for p, on in zip(params, flags) if on]
 
-    def _first_step_entry(self):
-        for p in self._stepped_params():
-            return dict.__getitem__(self.state[p], "step")
-        return 0
-
     def _sync_steps(self):
-        """Write the shared step counter (device-resident or host-side) into state[p]["step"] of every parameter that
-        the steps so far have updated."""
+        """Write the step counter (device-resident or host-side) into state[p]["step"] of every parameter that
+        the steps so far have updated: the common count plus the parameter's own distance from it."""
         if not self._steps_dirty:
             return
         self._steps_dirty = False
-        step = self.loss_scaler.adam_step if self._dynamic else self._host_step
+        if self._dynamic:
+            self._common_step = self.loss_scaler.adam_step
         for p in self._stepped_params():
-            dict.__setitem__(self.state[p], "step", step)
+            dict.__setitem__(self.state[p], "step", self._common_step + self._offsets.get(p, 0))
 
-    def _trainable_changed(self, now):
-        """requires_grad of some parameter changed since the last step.  The reference counts ``state[p]["step"]`` per
-        parameter and hands each tensor's own count to the operator (fp16_cpu_adam.py:571-574,603); the fused step has
-        ONE counter.  Freezing a parameter is therefore fine at any time; a parameter that becomes trainable must
-        stand at the common count (true before the first step, or if it was trainable for every step so far)."""
-        before = self._trainable_seen
-        if before is not None:
-            self._sync_steps()
+    def _each_table(self, plan):
+        """Tensor rows and per-tensor call records of a step whose tensors carry their own numbers."""
+        if plan["table"] is None:
+            trainable = plan["trainable"]
+            rows, numels, n = self._tensor_rows(trainable)
+            each = (_lib.ps_tensor_call * n)()
+            on_host = {pos.fp16 for pos in self.client.positions() if pos.on_host}
+            index = self.client.chunk_tensor_index
+            operator_calls = 0
+            for i, (p, (lr, (beta1, beta2), eps, weight_decay, _)) in enumerate(zip(trainable, plan["entries"])):
+                e = each[i]
+                e.lr, e.beta1, e.beta2, e.eps, e.weight_decay = lr, beta1, beta2, eps, weight_decay
+                # optimizer state in host memory is updated by the operator whatever the optimizer's arithmetic
+                # (fp16_cpu_adam.py:415-443); the kernel reads and writes such pinned payloads over the link
+                host = index.get_tensor_info(p.ps_attr.data_id()).chunk_id in on_host
+                e.arithmetic = _lib.PS_ARITH_OPERATOR if (host or self.arithmetic == "operator") else _lib.PS_ARITH_TORCH
+                operator_calls += e.arithmetic == _lib.PS_ARITH_OPERATOR
+            workspace = None
             if self._dynamic:
-                common = self.loss_scaler.adam_step
-            else:
-                common = self._host_step if self._host_step is not None else self._first_step_entry()
-            for p, was, on in zip(self.param_groups[0]["params"], before, now):
-                own = dict.__getitem__(self.state[p], "step")
-                if on and not was and own != common:
-                    raise NotImplementedError(
-                        f"parameter {p.ps_attr.name} became trainable after {own} steps of its own while the others "
-                        f"have made {common}: the reference would hand the operator a different step number for it, "
-                        "which one fused step cannot do"
-                    )
-        self._trainable_seen = now
-        self._tables = None
-        self._hyper_checked = False
+                nbytes = self._lib.ps_tensors_each_workspace_bytes(n)
+                workspace = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=self.client.device)
+            plan["table"] = (rows, numels, n, each, workspace, operator_calls)
+        return plan["table"]
+
+    def _step_each(self, plan, stream):
+        """One step through ``ps_adam_step_tensors_each``."""
+        rows, numels, n, each, workspace, operator_calls = self._each_table(plan)
+        offsets = [self._offsets.get(p, 0) for p in plan["trainable"]]
+        if self._dynamic:
+            scaler = self.loss_scaler
+            for i, d in enumerate(offsets):
+                each[i].step = d  # distance from the device's counter
+            _lib.check(
+                self._lib.ps_adam_step_tensors_each(
+                    self.opt_id, 1, rows, numels, each, n, -1.0, scaler.state_ptr, workspace.data_ptr(),
+                    workspace.numel(), stream,
+                ),
+                "ps_adam_step_tensors_each",
+            )
+            scaler.update_scale(None, operator_calls=operator_calls)
+            return
+        self._common_step += 1
+        for i, d in enumerate(offsets):
+            each[i].step = self._common_step + d
+        loss_scale = self.loss_scaler.loss_scale if self.loss_scaler is not None else -1
+        _lib.check(
+            self._lib.ps_adam_step_tensors_each(self.opt_id, 1, rows, numels, each, n, float(loss_scale), None, None, 0, stream),
+            "ps_adam_step_tensors_each",
+        )
+        if self.loss_scaler:
+            self.loss_scaler.update_scale(False)
 
     @torch.no_grad()
     def step(self, closure=None):
@@ -534,21 +615,28 @@ class FP16Adam(torch.optim.Optimizer):
             with torch.enable_grad():
                 loss = closure()
         # which parameters are trainable is looked at every step, as the reference does (fp16_cpu_adam.py:569-571):
-        # freezing or unfreezing a parameter between steps rebuilds the descriptor tables and the call pattern
-        trainable_now = tuple(p.requires_grad for p in self.param_groups[0]["params"])
-        if trainable_now != self._trainable_seen:
-            self._trainable_changed(trainable_now)
-        hyper = self._hyper()
-        if hyper is None:
+        # freezing or unfreezing a parameter between steps makes a new plan (descriptor tables, call pattern, and
+        # whether every tensor can still share one step number)
+        if self._plan is None or tuple(p.requires_grad for p in self.param_groups[0]["params"]) != self._trainable_seen:
+            self._make_plan()
+        plan = self._plan
+        if plan["kind"] == "empty":
             # nothing is trainable: the reference still runs its scale update (fp16_cpu_adam.py:549-558,624-625)
             if self._dynamic:
                 self.loss_scaler.update_scale(None, operator_calls=0)
             return loss
-        lr, (beta1, beta2), eps, weight_decay = hyper
-        table, n_dev, host_positions = self._tables or self._build_tables()
-        chunk_numel = self.client.default_chunk_size
         with torch.cuda.device(self.client.device):
             stream = _lib.current_stream_handle()
+            if plan["kind"] == "each":
+                if self._dynamic and self.scan_in_step:
+                    self.check_overflow_chunks()
+                self._step_each(plan, stream)
+                self._steps_dirty = True
+                return loss
+            hyper = plan["hyper"]
+            lr, (beta1, beta2), eps, weight_decay = hyper
+            table, n_dev, host_positions = self._tables or self._build_tables()
+            chunk_numel = self.client.default_chunk_size
             if self._dynamic:
                 scaler = self.loss_scaler
                 if self.scan_in_step:
@@ -566,11 +654,11 @@ class FP16Adam(torch.optim.Optimizer):
                     )
                 elif host_positions:
                     self._streamer.step(self.opt_id, 0, lr, beta1, beta2, eps, weight_decay, -1.0, table, n_dev,
-                                        self._calls, scaler)
+                                        self._calls, scaler, self._used_all)
                 elif n_dev:
                     _lib.check(
                         self._lib.ps_adam_step_chunks_gated(
-                            self.opt_id, lr, eps, weight_decay, 1, table, n_dev, chunk_numel, self._calls,
+                            self.opt_id, lr, eps, weight_decay, 1, table, n_dev, chunk_numel, self._used, self._calls,
                             scaler.state_ptr, stream,
                         ),
                         "ps_adam_step_chunks_gated",
@@ -584,11 +672,9 @@ class FP16Adam(torch.optim.Optimizer):
             # Static or absent scaler: the host knows every scalar (the static scaler never reports overflow).
             # every parameter's "step" advances together: one host counter, written back to the per-parameter
             # entries only when somebody reads them
-            if self._host_step is None:
-                self._host_step = self._first_step_entry()
-            self._host_step += 1
+            self._common_step += 1
             self._steps_dirty = True
-            step_no = self._host_step
+            step_no = self._common_step
             loss_scale = self.loss_scaler.loss_scale if self.loss_scaler is not None else -1
             if self._stages is not None:
                 self._run_stages(step_no, hyper, loss_scale, None, stream)
@@ -603,18 +689,35 @@ class FP16Adam(torch.optim.Optimizer):
                 )
             elif host_positions:
                 self._streamer.step(self.opt_id, step_no, lr, beta1, beta2, eps, weight_decay, loss_scale, table, n_dev,
-                                    self._calls)
+                                    self._calls, None, self._used_all)
             elif n_dev:
                 _lib.check(
                     self._lib.ps_adam_step_chunks(
                         self.opt_id, step_no, lr, beta1, beta2, eps, weight_decay, 1, table, n_dev,
-                        chunk_numel, self._calls, float(loss_scale), stream,
+                        chunk_numel, self._used, self._calls, float(loss_scale), stream,
                     ),
                     "ps_adam_step_chunks",
                 )
             if self.loss_scaler:
                 self.loss_scaler.update_scale(False)
         return loss
+
+    # -- the reference's overflow warning ----------------------------------------------
+    OVERFLOW_LOG_CAPACITY = 1024
+
+    def _warn_about_overflows(self, records, lost):
+        """``fp16_cpu_adam.py:551-556`` logs every skipped step as it happens.  Here a step is skipped on the device
+        and the host does not wait to learn of it; the loss scaler's device log keeps (flag, scale after) of every
+        iteration, and the lines are written when the scaler's state is next read back (``loss_scale``,
+        ``has_overflow``, ``state[p]["step"]``, ``state_dict()``), one per skipped step, with the reference's text."""
+        if lost:
+            logger.warning(
+                f"Gradient overflow! {lost} loss-scale updates were not read back in time to be reported one by one "
+                f"(the device log holds {self.OVERFLOW_LOG_CAPACITY})."
+            )
+        for _, overflow, before, after in records:
+            if overflow:
+                logger.warning(f"Gradient overflow! Update loss scale from {before} to {after}.")
 
     # -- checkpointing --------------------------------------------------------------
     def state_dict(self):
@@ -637,6 +740,9 @@ class FP16Adam(torch.optim.Optimizer):
         return out
 
     def load_state_dict(self, state_dict):
+        """``fp16_cpu_adam.py:660-694``: every parameter gets its saved ``step``, hyper-parameters and moments back.
+        The next ``step()`` derives the common counter from the parameters that are trainable then (a frozen
+        parameter's own count plays no part) and hands loaded betas to the device-resident state."""
         state_dict = deepcopy(state_dict)
         saved_groups = state_dict["param_groups"]
         saved_state = state_dict["state"]
@@ -644,7 +750,6 @@ class FP16Adam(torch.optim.Optimizer):
         assert len(saved_groups[0]["params"]) == len(self.param_groups[0]["params"])
         assert len(saved_state) == len(self.state)
         self._sync_steps()
-        step_seen = None
         for old_id, p in zip(saved_groups[0]["params"], self.param_groups[0]["params"]):
             saved = saved_state[old_id]
             mine = self.state[p]
@@ -654,15 +759,8 @@ class FP16Adam(torch.optim.Optimizer):
                     self.client.access_data(v).copy_(saved[k])
                 else:
                     dict.__setitem__(mine, k, saved[k])
-                    if k == "step":
-                        step_seen = saved[k]
-        self._hyper_checked = False
-        self._host_step = step_seen
+        self._plan = None
         if self._dynamic:
             self.loss_scaler.materialize(self.client.device)
-            if step_seen is not None:
-                # the operator object behind this optimizer stays the one it was (fp16_cpu_adam.py:660-694 does not
-                # touch it); a new optimizer got a new one when it was constructed
-                self.loss_scaler._seed_step(step_seen, fresh_operator=False)
             if "loss_scaler" in state_dict:
                 self.loss_scaler.load_state_dict(state_dict["loss_scaler"])

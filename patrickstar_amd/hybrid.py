@@ -16,9 +16,10 @@ from . import _lib
 
 
 class HostChunkStreamer:
-    def __init__(self, client, host_positions, n_slots=2, step_indices=None):
+    def __init__(self, client, host_positions, n_slots=3, step_indices=None, used=None):
         """``step_indices``: which of ``host_positions`` ``step()`` streams (default: all of them); the gradient probe
-        always covers every position."""
+        always covers every position.  ``used``: per position, the elements in front of its zero padding (only those
+        cross the link); default: whole chunks."""
         self.client = client
         self.n_slots = n_slots
         self.chunk_numel = client.default_chunk_size
@@ -38,11 +39,16 @@ class HostChunkStreamer:
             rows.append([t.data_ptr() for t in payloads])
         self.host_table = _lib.chunk_array(rows)
         self.n_host = len(rows)
+        used = list(used) if used is not None else [self.chunk_numel] * len(rows)
+        self.host_used = _lib.size_array(used) if any(u != self.chunk_numel for u in used) else None
         if step_indices is None:
-            self.step_table, self.n_step = self.host_table, self.n_host
+            self.step_table, self.n_step, self.step_used = self.host_table, self.n_host, used
         else:
             picked = [rows[k] for k in step_indices]
             self.step_table, self.n_step = (_lib.chunk_array(picked) if picked else None), len(picked)
+            self.step_used = [used[k] for k in step_indices]
+        # for a step() that streams these positions and updates no resident chunk beside them
+        self.host_used_of_step = _lib.size_array(self.step_used) if any(u != self.chunk_numel for u in self.step_used) else None
         dev = client.device
         n = self.chunk_numel
         # staging lives for the life of the optimizer: allocating it per step (as the reference does with
@@ -62,14 +68,15 @@ class HostChunkStreamer:
         self._lib = _lib.load()
 
     def step(self, opt_id, step_no, lr, beta1, beta2, eps, weight_decay, loss_scale, resident, n_resident, calls=None,
-             scaler=None):
+             scaler=None, used=None):
         """One optimizer step over the resident chunk array AND the host-resident chunks.
         ``calls``: the step's ps_call_pattern over both lists (resident positions counted first).
-        ``scaler`` (a device-resident DynamicLossScaler) selects the device-gated form."""
+        ``scaler`` (a device-resident DynamicLossScaler) selects the device-gated form.
+        ``used``: size_t array over the resident positions followed by the streamed ones (None: whole chunks)."""
         _lib.check(
             self._lib.ps_adam_step_hybrid(
                 opt_id, step_no, lr, beta1, beta2, eps, weight_decay, 1, resident, n_resident, self.step_table,
-                self.n_step, self.chunk_numel, self.staging, self.n_slots, calls, float(loss_scale),
+                self.n_step, self.chunk_numel, used, self.staging, self.n_slots, calls, float(loss_scale),
                 scaler.state_ptr if scaler is not None else None, _lib.current_stream_handle(),
             ),
             "ps_adam_step_hybrid",
@@ -78,7 +85,7 @@ class HostChunkStreamer:
     def scan_gradients(self, scaler):
         _lib.check(
             self._lib.ps_overflow_scan_host_chunks(
-                self.host_table, self.n_host, self.chunk_numel, self.staging, self.n_slots, scaler.state_ptr,
+                self.host_table, self.n_host, self.chunk_numel, self.host_used, self.staging, self.n_slots, scaler.state_ptr,
                 _lib.current_stream_handle(),
             ),
             "ps_overflow_scan_host_chunks",

@@ -10,6 +10,7 @@ whether gradients overflowed.  Reading a field from Python
 synchronisation point.
 """
 import ctypes
+import weakref
 
 import torch
 
@@ -90,6 +91,13 @@ class DynamicLossScaler:
         self._state = None  # device tensor holding one ps_step_state
         self._log = None  # optional device tensor of ps_scale_record
         self._log_capacity = 0
+        self._log_start = 0  # the iteration the ring has been recording from
+        self._log_seen = 0  # iterations below this one have been handed to on_read
+        self._scale_seen = init_scale  # loss scale after iteration _log_seen - 1
+        # Called with (records, lost) whenever a field is read back from the device and update_scale calls have
+        # completed since the last time: records = [(iteration, overflow, scale before, scale after)], lost = how
+        # many iterations fell out of the ring unseen.  A callable, or a weak reference to one.  Needs enable_log.
+        self.on_read = None
         self._betas = (0.9, 0.999)
 
     # -- device state ---------------------------------------------------------
@@ -130,9 +138,13 @@ class DynamicLossScaler:
             )
         return self
 
-    def _seed_step(self, adam_step, fresh_operator=True):
-        """Set the Adam step counter.  ``fresh_operator``: a newly created operator object stands behind it (a new
-        optimizer); False keeps the running one, as the reference's ``load_state_dict`` does."""
+    def _seed_step(self, adam_step, fresh_operator=True, betas=None):
+        """Set the Adam step counter and, if given, the betas of the steps to come.  ``fresh_operator``: a newly
+        created operator object stands behind it (a new optimizer); False keeps the running one, as the reference's
+        ``load_state_dict`` does: its first call then continues the running beta^t product only if the object stands
+        at ``adam_step`` with the same betas (``cpu_adam.h:143-162``)."""
+        if betas is not None:
+            self._betas = (float(betas[0]), float(betas[1]))
         _lib.check(
             _lib.load().ps_state_seed_step(
                 self._state.data_ptr(), int(adam_step), self._betas[0], self._betas[1], int(bool(fresh_operator)),
@@ -142,31 +154,61 @@ class DynamicLossScaler:
         )
 
     def enable_log(self, capacity):
-        """Record (overflow flag, scale after) of every ``update_scale`` in a device ring of ``capacity`` entries."""
+        """Record (overflow flag, scale after) of every ``update_scale`` in a device ring of ``capacity`` entries,
+        from the present iteration on."""
+        fresh = self._state is None
         self.materialize()
+        if not fresh:
+            s = self._read()  # settle what the old ring (if any) still holds
+            self._log_start = self._log_seen = int(s.cur_iter)
+            self._scale_seen = int(s.cur_scale) if s.scale_is_int else float(s.cur_scale)
         self._log = torch.zeros(capacity * ctypes.sizeof(_lib.ps_scale_record), dtype=torch.uint8, device=self._state.device)
         self._log_capacity = capacity
 
-    def read_log(self):
-        """[(overflow: bool, loss_scale)] for the iterations recorded so far (synchronises)."""
-        n = min(self.cur_iter, self._log_capacity)
+    def _records(self, first, last):
+        """Ring entries of iterations [first, last) as (overflow, typed scale after); the ring must still hold them."""
         raw = self._log.cpu().numpy().tobytes()
         recs = (_lib.ps_scale_record * self._log_capacity).from_buffer_copy(raw)
-        start = self.cur_iter - n
         out = []
-        for it in range(start, start + n):
+        for it in range(first, last):
             r = recs[it % self._log_capacity]
             out.append((bool(r.overflow), int(r.scale_after) if r.scale_is_int else float(r.scale_after)))
         return out
 
-    def _read(self):
+    def read_log(self):
+        """[(overflow: bool, loss_scale)] for the iterations the ring still holds (synchronises)."""
+        cur = int(self._read(notify=False).cur_iter)
+        return self._records(max(self._log_start, cur - self._log_capacity), cur)
+
+    def _read(self, notify=True):
         host = _lib.ps_step_state()
         with torch.cuda.device(self._state.device):
             _lib.check(
                 _lib.load().ps_state_read(self._state.data_ptr(), ctypes.byref(host), _lib.current_stream_handle()),
                 "ps_state_read",
             )
+        if notify and self._log is not None and self.on_read is not None and host.cur_iter > self._log_seen:
+            self._notify(int(host.cur_iter))
         return host
+
+    def _notify(self, cur_iter):
+        """Hand the outcomes of the iterations completed since the last read-back to ``on_read``."""
+        hook = self.on_read
+        if isinstance(hook, weakref.ReferenceType):
+            hook = hook()
+        first = max(self._log_seen, self._log_start, cur_iter - self._log_capacity)
+        lost = first - max(self._log_seen, self._log_start)
+        got = self._records(first, cur_iter)
+        records, before = [], self._scale_seen
+        for k, (overflow, after) in enumerate(got):
+            # (the scale in front of an iteration that fell out of the ring is not known)
+            records.append((first + k, overflow, None if (lost and k == 0) else before, after))
+            before = after
+        self._log_seen = cur_iter
+        if got:
+            self._scale_seen = got[-1][1]
+        if hook is not None and (records or lost):
+            hook(records, lost)
 
     @property
     def state_ptr(self):
@@ -302,6 +344,10 @@ class DynamicLossScaler:
 
     def load_state_dict(self, sd):
         self.materialize()
+        if self._log is not None:
+            self._read()  # outcomes recorded so far belong to the run that is being replaced: hand them on now
+            self._log_start = self._log_seen = int(sd["cur_iter"])
+            self._scale_seen = sd["cur_scale"]
         with torch.cuda.device(self._state.device):
             _lib.check(
                 _lib.load().ps_state_set_scaler(

@@ -157,7 +157,7 @@ int main()
             new_gradients(rng, host[c], scale);
             if (upload(host[c], dev[c], n)) return 2;
         }
-        PS_OK(ps_adam_step_chunks(31, step, lr, b1, b2, eps, wd, 1, table, C, n, &calls, scale, stream));
+        PS_OK(ps_adam_step_chunks(31, step, lr, b1, b2, eps, wd, 1, table, C, n, nullptr, &calls, scale, stream));
         HIP_OK(hipStreamSynchronize(stream));
         for (int c = 0; c < C; ++c) {
             oracle_adam_advance(&native, step, b1, b2);  // one adam_update per tensor, same step number
@@ -185,8 +185,8 @@ int main()
             if (poison && c == it % C) host[c].h[n - 1] = 0x7C00;  // +inf in the last element
             if (upload(host[c], dev[c], n)) return 2;
         }
-        PS_OK(ps_overflow_scan_chunks(table, C, n, d_state, stream));
-        PS_OK(ps_adam_step_chunks_gated(32, lr, eps, wd, 1, table, C, n, &calls, d_state, stream));
+        PS_OK(ps_overflow_scan_chunks(table, C, n, nullptr, d_state, stream));
+        PS_OK(ps_adam_step_chunks_gated(32, lr, eps, wd, 1, table, C, n, nullptr, &calls, d_state, stream));
         PS_OK(ps_scaler_update(d_state, PS_FLAG_FROM_DEVICE, NULL, 0, calls.n_calls, stream));
         HIP_OK(hipStreamSynchronize(stream));
         if (poison) {
@@ -262,7 +262,7 @@ int main()
                     HIP_OK(hipMemcpy(dev[c].h, host[c].h.data(), n * 2, hipMemcpyHostToDevice));
             }
         }
-        PS_OK(ps_adam_step_hybrid(33, step, lr, b1, b2, eps, wd, 1, table, 1, host_table, 2, n, staging, 2, &calls, scale,
+        PS_OK(ps_adam_step_hybrid(33, step, lr, b1, b2, eps, wd, 1, table, 1, host_table, 2, n, nullptr, staging, 2, &calls, scale,
                                   NULL, stream));
         HIP_OK(hipStreamSynchronize(stream));
         for (int c = 0; c < C; ++c) {
@@ -294,7 +294,7 @@ int main()
     // the probe over host-resident positions: an inf in the pinned fp16 payload must reach the device flag
     PS_OK(ps_state_init(d_state, 1024.0, 1, 2.0, 1, 1000, 1.0, 1, 1, 0, b1, b2, stream));
     pinned[2].h[n / 2] = 0xFC00;  // -inf
-    PS_OK(ps_overflow_scan_host_chunks(host_table, 2, n, staging, 2, d_state, stream));
+    PS_OK(ps_overflow_scan_host_chunks(host_table, 2, n, nullptr, staging, 2, d_state, stream));
     PS_OK(ps_state_read(d_state, &st, stream));
     if (st.overflow != 1) {
         fprintf(stderr, "the probe of host-resident chunks missed an inf\n");

@@ -21,15 +21,15 @@ int main(void)
     ps_chunk bad;
     ps_step_state st;
     int rc;
-    if (sizeof(ps_chunk) != 32 || sizeof(ps_step_state) != 192 || sizeof(ps_call_pattern) != 32 || sizeof(ps_scale_record) != 16) return 10;
+    if (sizeof(ps_chunk) != 32 || sizeof(ps_step_state) != 256 || sizeof(ps_call_pattern) != 32 || sizeof(ps_scale_record) != 16) return 10;
     if (ps_abi_version() != PS_ABI_VERSION) return 11;
     if (ps_adam_create(4242, 1e-3f, 0.9f, 0.999f, 1e-8f, 0.01f, 1, 0) != 0) return 12;
     if (ps_adam_set_arithmetic(4242, PS_ARITH_TORCH) != 0) return 13;
     if (ps_adam_set_arithmetic(4242, 5) != PS_ERR_BAD_ARG) return 14;
     memset(&bad, 0, sizeof bad);
-    rc = ps_adam_step_chunks(4242, 1, 1e-3, 0.9, 0.999, 1e-8, 0.01, 1, &bad, 1, 1024, NULL, 4096.0, NULL);
+    rc = ps_adam_step_chunks(4242, 1, 1e-3, 0.9, 0.999, 1e-8, 0.01, 1, &bad, 1, 1024, NULL, NULL, 4096.0, NULL);
     if (rc != PS_ERR_BAD_ARG || strstr(ps_last_error(), "NULL payload") == NULL) return 15;
-    if (ps_adam_step_chunks(4243, 1, 1e-3, 0.9, 0.999, 1e-8, 0.01, 1, &bad, 0, 1024, NULL, 4096.0, NULL) != PS_ERR_UNKNOWN_ID) return 16;
+    if (ps_adam_step_chunks(4243, 1, 1e-3, 0.9, 0.999, 1e-8, 0.01, 1, &bad, 0, 1024, NULL, NULL, 4096.0, NULL) != PS_ERR_UNKNOWN_ID) return 16;
     if (ps_state_read(NULL, &st, NULL) != PS_ERR_BAD_ARG) return 17;
     if (ps_adam_destroy(4242) != 0) return 18;
     puts("c abi ok");

@@ -140,7 +140,7 @@ def test_hip_torch_arithmetic_reproduces_torch_gpu_kernels_bitwise(case):
         h = torch.from_numpy(TVEC[f"{name}/g{k}"].copy()).cuda()  # gradients in, fp16 parameters out
         rows = _lib.chunk_array([[dp.data_ptr(), dm.data_ptr(), dv.data_ptr(), h.data_ptr()]])
         _lib.check(
-            lib.ps_adam_step_chunks(oid, t0 + k, lr, b1, b2, eps, wd, 1, rows, 1, n, None,
+            lib.ps_adam_step_chunks(oid, t0 + k, lr, b1, b2, eps, wd, 1, rows, 1, n, None, None,
                                     float(scale) if scale is not None else -1.0, _lib.current_stream_handle()),
             "ps_adam_step_chunks",
         )

@@ -220,14 +220,14 @@ def test_empty_and_zero_sized_chunk_lists():
     lib = _lib.load()
     s = _lib.current_stream_handle()
     lib.ps_adam_create(902, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, 0)
-    assert lib.ps_adam_step_chunks(902, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, 1024, None, -1.0, s) == 0
+    assert lib.ps_adam_step_chunks(902, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, 1024, None, None, -1.0, s) == 0
     buf = torch.zeros(64, dtype=torch.float, device="cuda")
     one = _lib.chunk_array([[buf.data_ptr()] * 4])
-    assert lib.ps_adam_step_chunks(902, 2, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, one, 1, 0, None, -1.0, s) == 0
-    assert lib.ps_adam_step_chunks(902, 3, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 2, 16, None, -1.0, s) == _lib.PS_ERR_BAD_ARG
-    assert lib.ps_adam_step_chunks(902, 3, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, one, -1, 16, None, -1.0, s) == _lib.PS_ERR_BAD_ARG
+    assert lib.ps_adam_step_chunks(902, 2, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, one, 1, 0, None, None, -1.0, s) == 0
+    assert lib.ps_adam_step_chunks(902, 3, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 2, 16, None, None, -1.0, s) == _lib.PS_ERR_BAD_ARG
+    assert lib.ps_adam_step_chunks(902, 3, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, one, -1, 16, None, None, -1.0, s) == _lib.PS_ERR_BAD_ARG
     null_payload = _lib.chunk_array([[buf.data_ptr(), 0, buf.data_ptr(), buf.data_ptr()]])
-    assert lib.ps_adam_step_chunks(902, 3, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, null_payload, 1, 16, None, -1.0, s) == _lib.PS_ERR_BAD_ARG
+    assert lib.ps_adam_step_chunks(902, 3, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, null_payload, 1, 16, None, None, -1.0, s) == _lib.PS_ERR_BAD_ARG
     assert b"NULL payload" in lib.ps_last_error()
     assert lib.ps_cast_fp32_to_fp16(None, None, 0, s) == 0
     lib.ps_adam_destroy(902)
@@ -523,7 +523,7 @@ def test_randomised_call_sequences_match_the_oracle_state_machine():
             dg = _dev(g.copy())
             if use_chunks:
                 table = _lib.chunk_array([[dp.data_ptr(), dm.data_ptr(), dv.data_ptr(), dg.data_ptr()]])
-                rc = lib.ps_adam_step_chunks(oid, step, lr, betas[0], betas[1], eps, wd, bias_correction, table, 1, n, None, scale, stream)
+                rc = lib.ps_adam_step_chunks(oid, step, lr, betas[0], betas[1], eps, wd, bias_correction, table, 1, n, None, None, scale, stream)
             else:
                 rc = lib.ps_adam_update(oid, step, lr, betas[0], betas[1], eps, wd, bias_correction, dp.data_ptr(), dg.data_ptr(), 1,
                                         dm.data_ptr(), dv.data_ptr(), n, scale, None, stream)
@@ -561,7 +561,7 @@ def test_chunk_step_with_unaligned_payload_bases(offsets):
         rows.append([d[0][op:].data_ptr(), d[1][om:].data_ptr(), d[2][ov:].data_ptr(), d[3][oh:].data_ptr()])
     oid = 905
     lib.ps_adam_create(oid, 1e-3, 0.9, 0.999, 1e-8, 0.01, 1, 0)
-    assert lib.ps_adam_step_chunks(oid, 3, 1e-3, 0.9, 0.999, 1e-8, 0.01, 1, _lib.chunk_array(rows), C, n, None, 16.0,
+    assert lib.ps_adam_step_chunks(oid, 3, 1e-3, 0.9, 0.999, 1e-8, 0.01, 1, _lib.chunk_array(rows), C, n, None, None, 16.0,
                                    _lib.current_stream_handle()) == 0
     torch.cuda.synchronize()
     lib.ps_adam_destroy(oid)
@@ -615,7 +615,7 @@ def test_randomised_shapes_hyperparameters_and_arithmetics():
         if torch_arith:
             _lib.check(lib.ps_adam_set_arithmetic(oid, _lib.PS_ARITH_TORCH), "set_arithmetic")
         _lib.check(
-            lib.ps_adam_step_chunks(oid, step, lr, b1, b2, eps, wd, 1, _lib.chunk_array(rows), C, n, None,
+            lib.ps_adam_step_chunks(oid, step, lr, b1, b2, eps, wd, 1, _lib.chunk_array(rows), C, n, None, None,
                                     float(scale) if scale is not None else -1.0, _lib.current_stream_handle()),
             what,
         )
@@ -662,7 +662,7 @@ def test_two_host_threads_step_their_own_optimizers_concurrently():
                 for s in range(steps):
                     for c in range(C):
                         dev[c][3].copy_(torch.from_numpy(grads[s][c]), non_blocking=False)
-                    assert lib.ps_adam_step_chunks(oid, s + 1, lr, 0.9, 0.999, 1e-8, wd, 1, rows, C, n, None, 8.0, handle) == 0
+                    assert lib.ps_adam_step_chunks(oid, s + 1, lr, 0.9, 0.999, 1e-8, wd, 1, rows, C, n, None, None, 8.0, handle) == 0
                 stream.synchronize()
                 lib.ps_adam_destroy(oid)
             o = oracle.AdamOracle(lr, 0.9, 0.999, 1e-8, wd, bool(tid))

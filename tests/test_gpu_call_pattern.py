@@ -78,7 +78,7 @@ def test_host_decided_steps_follow_the_per_tensor_pattern(adamw, wd, scale, offs
         R.new_grads(rng, scale)
         oopt.step_count = step - 1
         _lib.check(
-            lib.ps_adam_step_chunks(oid, step, lr, b1, b2, eps, wd, 1, R.table, 3, N, calls, scale,
+            lib.ps_adam_step_chunks(oid, step, lr, b1, b2, eps, wd, 1, R.table, 3, N, None, calls, scale,
                                     _lib.current_stream_handle()),
             "ps_adam_step_chunks",
         )
@@ -106,7 +106,7 @@ def test_the_pattern_changes_bits_and_a_missing_pattern_means_one_call():
             R.new_grads(rng, 1.0)
             calls = _lib.call_pattern(len(tensors), *tensors[0]) if tensors else None
             _lib.check(
-                lib.ps_adam_step_chunks(oid, step, lr, b1, b2, eps, 0.0, 1, R.table, 3, N, calls, -1.0,
+                lib.ps_adam_step_chunks(oid, step, lr, b1, b2, eps, 0.0, 1, R.table, 3, N, None, calls, -1.0,
                                         _lib.current_stream_handle()),
                 "ps_adam_step_chunks",
             )
@@ -144,8 +144,8 @@ def test_device_gated_steps_follow_the_per_tensor_pattern():
     for it in range(9):
         R.new_grads(rng, float(oscaler.loss_scale), poison=(2, N - 1) if it in (2, 6) else None)
         s = _lib.current_stream_handle()
-        _lib.check(lib.ps_overflow_scan_chunks(R.table, 3, N, scaler.state_ptr, s), "scan")
-        _lib.check(lib.ps_adam_step_chunks_gated(oid, lr, eps, wd, 1, R.table, 3, N, calls, scaler.state_ptr, s), "gated")
+        _lib.check(lib.ps_overflow_scan_chunks(R.table, 3, N, None, scaler.state_ptr, s), "scan")
+        _lib.check(lib.ps_adam_step_chunks_gated(oid, lr, eps, wd, 1, R.table, 3, N, None, calls, scaler.state_ptr, s), "gated")
         scaler.update_scale(None, operator_calls=len(TENSORS))
         oopt.check_overflow()
         skipped.append(oopt.step())
@@ -161,7 +161,7 @@ def test_device_gated_steps_follow_the_per_tensor_pattern():
     for it in range(2):
         R.new_grads(rng, float(oscaler.loss_scale))
         s = _lib.current_stream_handle()
-        _lib.check(lib.ps_adam_step_chunks_gated(oid, lr, eps, wd, 1, R.table, 3, N, calls, scaler.state_ptr, s), "gated")
+        _lib.check(lib.ps_adam_step_chunks_gated(oid, lr, eps, wd, 1, R.table, 3, N, None, calls, scaler.state_ptr, s), "gated")
         scaler.update_scale(None, operator_calls=len(TENSORS))
         oopt2.step()
         R.compare(f"after reload, iteration {it}")
@@ -222,14 +222,14 @@ def test_call_pattern_argument_checks():
     E = _lib.PS_ERR_BAD_ARG
 
     def step(calls):
-        return lib.ps_adam_step_chunks(843, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, rows, 2, 512, calls, -1.0, s)
+        return lib.ps_adam_step_chunks(843, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, rows, 2, 512, None, calls, -1.0, s)
 
     assert step(_lib.call_pattern(0)) == E and b"n_calls" in lib.ps_last_error()
     assert step(_lib.call_pattern(2, 2, 0, 8)) == E and b"first_chunk" in lib.ps_last_error()
     assert step(_lib.call_pattern(2, -1, 0, 8)) == E
     assert step(_lib.call_pattern(2, 0, 500, 13)) == E and b"does not fit" in lib.ps_last_error()
     assert step(_lib.call_pattern(2, 0, 513, 0)) == 0  # a first call without elements: nothing to place
-    assert lib.ps_adam_step_chunks_gated(843, 1e-3, 1e-8, 0.0, 1, rows, 2, 512, _lib.call_pattern(3, 5, 0, 1),
+    assert lib.ps_adam_step_chunks_gated(843, 1e-3, 1e-8, 0.0, 1, rows, 2, 512, None, _lib.call_pattern(3, 5, 0, 1),
                                          ctypes.c_void_p(buf.data_ptr()), s) == E
     torch.cuda.synchronize()
     lib.ps_adam_destroy(843)

@@ -642,7 +642,7 @@ def test_frozen_parameters_together_with_host_resident_positions(host, loss_scal
 def test_freezing_and_unfreezing_parameters_between_steps():
     """requires_grad is looked at every step (fp16_cpu_adam.py:569-571).  Unfreezing before the first step and freezing
     later both follow the reference (oracle with the matching tensor list); a parameter that comes back after it missed
-    steps would need its own step number, which is refused loudly instead of being updated with the common one."""
+    steps is updated with its own step number, as the reference counts it (fp16_cpu_adam.py:571-574,603)."""
     torch.manual_seed(0)
     config = {
         "optimizer": {"type": "AdamW", "params": {"lr": 1e-2, "betas": (0.9, 0.999), "eps": 1e-8, "weight_decay": 0.1}},
@@ -687,7 +687,8 @@ def test_freezing_and_unfreezing_parameters_between_steps():
     assert torch.equal(client.access_data(module.gain), gain_before)
     assert optimizer.state[module.gain]["step"] == 2 and optimizer.state[module.fc2.weight]["step"] == 4
     module.gain.requires_grad_(True)  # stands at 2 steps, the others at 4
-    loss = engine(x)
-    engine.backward(loss)
-    with pytest.raises(NotImplementedError, match="became trainable after 2 steps"):
-        optimizer.step()
+    oopt.tensors = tensor_spans(client, optimizer)
+    iterate("gain back: its step 3 beside the others' step 5")
+    iterate("step 4 beside step 6")
+    assert optimizer.state[module.gain]["step"] == 4 and optimizer.state[module.fc2.weight]["step"] == 6
+    assert optimizer.state[module.fc2.bias]["step"] == 2

@@ -70,8 +70,8 @@ def test_chunk_lists_under_random_call_patterns(seed):
             for it in range(int(rng.integers(2, 6))):
                 poison = (int(rng.integers(0, C)), int(rng.integers(0, n))) if rng.random() < 0.25 else None
                 R.new_grads(rng, float(oscaler.loss_scale), poison=poison)
-                _lib.check(lib.ps_overflow_scan_chunks(R.table, C, n, scaler.state_ptr, stream), "scan")
-                _lib.check(lib.ps_adam_step_chunks_gated(oid, lr, eps, wd, 1, R.table, C, n, calls, scaler.state_ptr, stream), "gated")
+                _lib.check(lib.ps_overflow_scan_chunks(R.table, C, n, None, scaler.state_ptr, stream), "scan")
+                _lib.check(lib.ps_adam_step_chunks_gated(oid, lr, eps, wd, 1, R.table, C, n, None, calls, scaler.state_ptr, stream), "gated")
                 scaler.update_scale(None, operator_calls=len(tensors))
                 oopt.check_overflow()
                 assert oopt.step() == (poison is not None), what
@@ -86,7 +86,7 @@ def test_chunk_lists_under_random_call_patterns(seed):
                 step = step + 1 if rng.random() < 0.7 else int(rng.integers(1, 3000))
                 R.new_grads(rng, scale or 1.0)
                 oopt.step_count = step - 1
-                _lib.check(lib.ps_adam_step_chunks(oid, step, lr, b1, b2, eps, wd, 1, R.table, C, n, calls, scale if scale else -1.0, stream),
+                _lib.check(lib.ps_adam_step_chunks(oid, step, lr, b1, b2, eps, wd, 1, R.table, C, n, None, calls, scale if scale else -1.0, stream),
                            "chunks")
                 oopt.step()
                 R.compare(f"{what} step {step}")

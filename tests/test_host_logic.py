@@ -185,14 +185,14 @@ def test_library_loads_and_exports_every_declared_symbol():
     lib = _lib.load()
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.ps_abi_version() == _lib.PS_ABI_VERSION == 4
+    assert lib.ps_abi_version() == _lib.PS_ABI_VERSION == 5
     # host-only entry points: registry and argument checks work without a GPU
     assert lib.ps_adam_create(77, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, 0) == 0
     assert lib.ps_adam_destroy(77) == 0
     assert lib.ps_scaler_update(None, 0, None, 0, 1, None) == _lib.PS_ERR_BAD_ARG
     assert b"d_state" in lib.ps_last_error()
     assert lib.ps_state_init(None, 1.0, 1, 2.0, 1, 10, 1.0, 1, 1, 0, 0.9, 0.999, None) == _lib.PS_ERR_BAD_ARG
-    assert ctypes.sizeof(_lib.ps_step_state) == 192 and ctypes.sizeof(_lib.ps_chunk) == 32
+    assert ctypes.sizeof(_lib.ps_step_state) == 256 and ctypes.sizeof(_lib.ps_chunk) == 32
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
@@ -278,16 +278,16 @@ def test_argument_checks_happen_before_any_gpu_work():
     fake = _lib.chunk_array([[16, 32, 48, 64]])  # never dereferenced: every call below fails validation first
     bad_slot = _lib.chunk_array([[16, 0, 48, 64]])
     E = _lib.PS_ERR_BAD_ARG
-    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, None, 2, None, 1.0, None, None) == E
+    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, None, None, 2, None, 1.0, None, None) == E
     assert b"staging" in lib.ps_last_error()
-    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, fake, 0, None, 1.0, None, None) == E
-    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, fake, 9, None, 1.0, None, None) == E
-    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, bad_slot, 1, None, 1.0, None, None) == E
-    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, bad_slot, 1, 1024, fake, 1, None, 1.0, None, None) == E
+    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, None, fake, 0, None, 1.0, None, None) == E
+    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, None, fake, 9, None, 1.0, None, None) == E
+    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, None, bad_slot, 1, None, 1.0, None, None) == E
+    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, bad_slot, 1, 1024, None, fake, 1, None, 1.0, None, None) == E
     assert b"host chunk 0" in lib.ps_last_error()
-    assert lib.ps_adam_step_hybrid(4711, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, fake, 1, None, 1.0, None, None) == _lib.PS_ERR_UNKNOWN_ID
-    assert lib.ps_adam_step_chunks_gated(88, 1e-3, 1e-8, 0.0, 1, fake, 1, 1024, None, None, None) == E
-    assert lib.ps_overflow_scan_host_chunks(fake, 1, 1024, fake, 1, None, None) == E
+    assert lib.ps_adam_step_hybrid(4711, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, None, 0, fake, 1, 1024, None, fake, 1, None, 1.0, None, None) == _lib.PS_ERR_UNKNOWN_ID
+    assert lib.ps_adam_step_chunks_gated(88, 1e-3, 1e-8, 0.0, 1, fake, 1, 1024, None, None, None, None) == E
+    assert lib.ps_overflow_scan_host_chunks(fake, 1, 1024, None, fake, 1, None, None) == E
     assert lib.ps_overflow_scan(None, 10, None, None) == E
     assert lib.ps_adam_set_grad_clamp(4711, 1.0) == _lib.PS_ERR_UNKNOWN_ID
     assert lib.ps_adam_set_grad_clamp(88, 1.0) == 0
@@ -296,7 +296,7 @@ def test_argument_checks_happen_before_any_gpu_work():
     assert lib.ps_adam_set_arithmetic(88, _lib.PS_ARITH_OPERATOR) == 0
     assert lib.ps_adam_set_arithmetic(4711, _lib.PS_ARITH_TORCH) == _lib.PS_ERR_UNKNOWN_ID
     # descriptors are validated before the operator's step scalars advance or anything is enqueued
-    assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, bad_slot, 1, 1024, None, 1.0, None) == E
+    assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, bad_slot, 1, 1024, None, None, 1.0, None) == E
     assert b"chunk 0 has a NULL payload" in lib.ps_last_error()
     assert lib.ps_state_init(ctypes.c_void_p(16), 1.0, 1, 2.0, 1, 0, 1.0, 1, 1, 0, 0.9, 0.999, None) == E  # window 0
     assert b"scale_window" in lib.ps_last_error()
@@ -307,21 +307,21 @@ def test_argument_checks_happen_before_any_gpu_work():
     # 2^62 elements is beyond the limit of each of them, whatever its tile size
     huge = 2**62
     flag = ctypes.c_void_p(16)
-    assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, 1, huge, None, 1.0, None) == E
+    assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, 1, huge, None, None, 1.0, None) == E
     assert b"beyond the launch grid" in lib.ps_last_error()
-    assert lib.ps_adam_step_chunks_gated(88, 1e-3, 1e-8, 0.0, 1, fake, 1, huge, None, flag, None) == E
-    assert lib.ps_overflow_scan_chunks(fake, 1, huge, flag, None) == E
+    assert lib.ps_adam_step_chunks_gated(88, 1e-3, 1e-8, 0.0, 1, fake, 1, huge, None, None, flag, None) == E
+    assert lib.ps_overflow_scan_chunks(fake, 1, huge, None, flag, None) == E
     assert lib.ps_overflow_scan_chunks_noalloc(fake, 1, huge, flag, None) == E
     assert lib.ps_restore_fp16_chunks(fake, 1, huge, None, None) == E
-    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, 1, None, 0, huge, None, 0, None, 1.0, None, None) == E
+    assert lib.ps_adam_step_hybrid(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, 1, None, 0, huge, None, None, 0, None, 1.0, None, None) == E
     one = (ctypes.c_size_t * 1)(huge)
     assert lib.ps_adam_step_tensors(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, one, 1, None, 1.0, None, None) == E
     assert b"beyond the launch grid" in lib.ps_last_error()
     # negative counts and a call pattern that does not fit the list
-    assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, -1, 1024, None, 1.0, None) == E
-    assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, 1, 1024, _lib.call_pattern(2, 1, 0, 10), 1.0, None) == E
+    assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, -1, 1024, None, None, 1.0, None) == E
+    assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, 1, 1024, None, _lib.call_pattern(2, 1, 0, 10), 1.0, None) == E
     assert b"first_chunk" in lib.ps_last_error()
-    assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, 1, 1024, _lib.call_pattern(2, 0, 1000, 25), 1.0, None) == E
+    assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, 1, 1024, None, _lib.call_pattern(2, 0, 1000, 25), 1.0, None) == E
     assert b"does not fit a chunk" in lib.ps_last_error()
     lib.ps_adam_destroy(88)
 
@@ -442,10 +442,11 @@ def test_step_tables_follow_the_reference_call_order_and_skip_frozen_parameters(
 
 
 @pytest.mark.skipif(not os.path.exists(_lib.LIB_PATH), reason="HIP library not built")
-def test_hyper_parameters_are_read_from_the_state_entries_and_must_agree():
+def test_hyper_parameters_are_read_from_the_state_entries_per_parameter():
     """The reference reads lr / betas / eps / weight_decay from state[p] per tensor (fp16_cpu_adam.py:593-598), not
-    from param_groups.  The fused step applies one set: rewriting every parameter's entry takes effect at the next
-    step, entries that differ between trainable parameters are refused, frozen parameters are not looked at."""
+    from param_groups, and hands each operator call its own (:403-428).  While every trainable parameter agrees the
+    whole chunk list goes to one fused call; entries that differ send the step tensor by tensor, each with its own
+    numbers; frozen parameters are not looked at."""
     client = ps.PatrickStarClient(0, 32, device="cpu")
     model = _Tiny()
     model.a.bias.requires_grad_(False)
@@ -453,16 +454,81 @@ def test_hyper_parameters_are_read_from_the_state_entries_and_must_agree():
     opt = ps.FP16Adam(client, model.parameters(), lr=1e-3, betas=(0.9, 0.99), eps=1e-6, weight_decay=0.1)
     assert opt._hyper() == (1e-3, (0.9, 0.99), 1e-6, 0.1)
     opt.param_groups[0]["lr"] = 7.0  # ignored, as in the reference
-    assert opt._hyper()[0] == 1e-3
+    assert opt._plan is not None and opt._hyper()[0] == 1e-3
     opt.state[model.b.weight]["lr"] = 5e-4
-    with pytest.raises(ValueError, match="different hyper-parameters"):
-        opt._hyper()
+    assert opt._plan is None and opt._hyper() == "each"
+    rows, numels, n, each, workspace, operator_calls = opt._each_table(opt._plan)
+    trainable = [model.scale, model.a.weight, model.b.weight, model.b.bias]  # parameters() order without a.bias
+    assert n == 4 == operator_calls and workspace is None and list(numels) == [p.numel() for p in trainable]
+    assert [each[i].lr for i in range(4)] == [1e-3, 1e-3, 5e-4, 1e-3]
+    assert all((each[i].beta1, each[i].beta2, each[i].eps, each[i].weight_decay) == (0.9, 0.99, 1e-6, 0.1) for i in range(4))
+    assert all(each[i].arithmetic == _lib.PS_ARITH_OPERATOR for i in range(4))
+    assert [rows[i].param_fp16 for i in range(4)] == [client.access_data(p).data_ptr() for p in trainable]
     for p in model.parameters():
         if p.requires_grad:
             opt.state[p]["lr"] = 5e-4
     assert opt._hyper()[0] == 5e-4
     opt.state[model.a.bias]["weight_decay"] = 0.5  # frozen: never handed to the operator
     assert opt._hyper() == (5e-4, (0.9, 0.99), 1e-6, 0.1)
+
+
+def _tiny_optimizer(freeze=(), **kw):
+    client = ps.PatrickStarClient(0, 32, device="cpu")
+    model = _Tiny()
+    for name in freeze:
+        dict(model.named_parameters())[name].requires_grad_(False)
+    client.register_model(model)
+    return client, model, ps.FP16Adam(client, model.parameters(), lr=1e-3, **kw)
+
+
+@pytest.mark.skipif(not os.path.exists(_lib.LIB_PATH), reason="HIP library not built")
+def test_a_checkpoint_with_a_frozen_last_parameter_resumes_at_its_step_count():
+    """load_state_dict restores `step` per parameter (fp16_cpu_adam.py:660-694).  The counter the next step continues
+    from is that of the TRAINABLE parameters: the last parameter in parameters() order is frozen here and stands at 0
+    steps while the others have made 7; a resumed optimizer must go on with step 8, not with step 1."""
+    _, model, opt = _tiny_optimizer(freeze=("b.bias",))
+    opt._make_plan()
+    opt._common_step, opt._steps_dirty = 7, True  # as seven host-decided steps leave it
+    sd = opt.state_dict()
+    assert [sd["state"][i]["step"] for i in range(5)] == [7, 7, 7, 7, 0]
+    _, model2, opt2 = _tiny_optimizer(freeze=("b.bias",))
+    opt2.load_state_dict(sd)
+    assert [dict.__getitem__(opt2.state[p], "step") for p in model2.parameters()] == [7, 7, 7, 7, 0]
+    opt2._make_plan()
+    assert opt2._plan["kind"] == "uniform" and opt2._common_step == 7 and opt2._offsets == {}
+    assert opt2.state[model2.scale]["step"] == 7 and opt2.state[model2.b.bias]["step"] == 0
+    # betas and the other entries come from the checkpoint too
+    sd["state"][0]["betas"] = sd["state"][1]["betas"] = sd["state"][2]["betas"] = sd["state"][3]["betas"] = (0.8, 0.9)
+    opt2.load_state_dict(sd)
+    assert opt2._hyper()[1] == (0.8, 0.9)
+
+
+@pytest.mark.skipif(not os.path.exists(_lib.LIB_PATH), reason="HIP library not built")
+def test_a_parameter_that_missed_steps_keeps_its_own_step_number():
+    """The reference counts state[p]["step"] per parameter (fp16_cpu_adam.py:571-574): a parameter that was frozen for
+    some steps stands behind the others when it becomes trainable again, and each operator call gets its tensor's own
+    step number (:406,603).  The plan keeps such a parameter's distance from the common counter."""
+    _, model, opt = _tiny_optimizer()
+    opt._make_plan()
+    opt._common_step, opt._steps_dirty = 2, True  # two steps with everything trainable
+    model.b.weight.requires_grad_(False)
+    opt._make_plan()
+    assert opt._plan["kind"] == "uniform" and opt.state[model.b.weight]["step"] == 2
+    opt._common_step, opt._steps_dirty = 5, True  # three more without b.weight
+    assert opt.state[model.scale]["step"] == 5 and opt.state[model.b.weight]["step"] == 2
+    model.b.weight.requires_grad_(True)
+    opt._make_plan()
+    assert opt._plan["kind"] == "each" and opt._common_step == 5 and opt._offsets == {model.b.weight: -3}
+    opt._common_step, opt._steps_dirty = 6, True  # one step together: both advance
+    assert opt.state[model.scale]["step"] == 6 and opt.state[model.b.weight]["step"] == 3
+    # the first trainable parameter defines the common counter: freeze it and the counter moves to the next one's
+    model.scale.requires_grad_(False)
+    opt._make_plan()
+    assert opt._common_step == 6 and opt._offsets == {model.b.weight: -3} and opt.state[model.scale]["step"] == 6
+    # writing an entry by hand is picked up like any other change
+    opt.state[model.b.weight]["step"] = 6
+    opt._make_plan()
+    assert opt._plan["kind"] == "uniform" and opt._offsets == {}
 
 
 def test_placement_is_decided_from_the_free_hbm_when_the_model_is_registered():

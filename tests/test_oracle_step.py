@@ -262,3 +262,125 @@ def test_frozen_tensors_are_not_listed_and_not_touched():
         assert np.array_equal(cs[0][key][100:300], before[0][key][100:300])
         assert not np.array_equal(cs[0][key][:100], before[0][key][:100])
     assert np.array_equal(cs[0]["p16"][100:300].view(np.uint16), before[0]["p32"][100:300].astype(np.float16).view(np.uint16))
+
+
+def _pow32(b, t):
+    return np.float32(math.pow(float(b), t))
+
+
+def test_every_tensor_carries_its_own_step_number():
+    """state[p]["step"] is counted per parameter and every operator call gets its tensor's own
+    (fp16_cpu_adam.py:571-574,603,406).  Tensor 1 is frozen during steps 3..5 and comes back standing at 2 while the
+    others stand at 5.  Which branch of IncrementStep (cpu_adam.h:143-162) each call then takes follows from the
+    step numbers of consecutive calls alone, and is worked out by hand here:
+      6th step  T0(6): the object stands at 5 (T2's call of the 5th step, a pow) -> pow(b,5)*b
+                T1(3): the object stands at 6 -> pow(b,3);   T2(6): the object stands at 3 -> pow(b,6)
+      7th step  T0(7): the object stands at 6 -> pow(b,6)*b; T1(4): pow(b,4); T2(7): pow(b,7)
+    Probe elements (parameter and moments zero) are compared with the float64 textbook value for that beta^t."""
+    lr, eps = 1e-3, 1e-8
+    tensors = _three_tensor_layout()
+    cs = _chunks(n_chunks=2, n=600, seed=61)
+    opt = oracle.OptimizerStepOracle(cs, None, lr=lr, betas=(0.9, 0.999), eps=eps, tensors=tensors)
+    rng = np.random.default_rng(62)
+
+    def one_step(active, expect):
+        opt.tensors = [tensors[k] for k in active]
+        for k in active:
+            ci, off, numel = tensors[k]
+            g = rng.normal(0, 1e-2, numel).astype(np.float16)
+            g[0] = np.float16(0.0123)
+            cs[ci]["p16"][off : off + numel] = g
+            cs[ci]["p32"][off] = cs[ci]["m"][off] = cs[ci]["v"][off] = 0.0
+        frozen_before = {k: cs[tensors[k][0]]["p32"][tensors[k][1] : tensors[k][1] + tensors[k][2]].copy()
+                         for k in range(len(tensors)) if k not in active}
+        assert opt.step() is False
+        for k, (b1t, b2t) in expect.items():
+            ci, off, _ = tensors[k]
+            right = _probe_update_f64(float(np.float16(0.0123)), 0.0, 0.0, lr, eps, b1t, b2t)
+            got = float(cs[ci]["p32"][off])
+            assert abs(got - right) <= 4e-7 * abs(right), (k, got, right)
+        for k, before in frozen_before.items():
+            ci, off, numel = tensors[k]
+            assert np.array_equal(cs[ci]["p32"][off : off + numel], before)
+
+    both = lambda f: (f(B1), f(B2))
+    one_step([0, 1, 2], {})
+    one_step([0, 1, 2], {1: both(lambda b: _pow32(b, 2)), 2: both(lambda b: _pow32(b, 2))})
+    for t in (3, 4, 5):
+        one_step([0, 2], {0: both(lambda b: np.float32(_pow32(b, t - 1) * b)), 2: both(lambda b: _pow32(b, t))})
+    assert [opt.state(s)["step"] for s in tensors] == [5, 2, 5]
+    one_step([0, 1, 2], {0: both(lambda b: np.float32(_pow32(b, 5) * b)), 1: both(lambda b: _pow32(b, 3)),
+                         2: both(lambda b: _pow32(b, 6))})
+    one_step([0, 1, 2], {0: both(lambda b: np.float32(_pow32(b, 6) * b)), 1: both(lambda b: _pow32(b, 4)),
+                         2: both(lambda b: _pow32(b, 7))})
+    assert [opt.state(s)["step"] for s in tensors] == [7, 4, 7]
+    # the branches are different numbers: tensor 1 updated with the others' step number would be off by far more
+    wrong = _probe_update_f64(0.0123, 0.0, 0.0, lr, eps, _pow32(B1, 7), _pow32(B2, 7))
+    right = _probe_update_f64(0.0123, 0.0, 0.0, lr, eps, _pow32(B1, 4), _pow32(B2, 4))
+    assert abs(wrong - right) > 1e-3 * abs(right)
+
+    # a call whose step number is the previous call's plus one continues the product in the MIDDLE of a step:
+    # T0 sits out one step and then stands one behind T1, which is called right after it
+    cs = _chunks(n_chunks=2, n=600, seed=63)
+    opt = oracle.OptimizerStepOracle(cs, None, lr=lr, betas=(0.9, 0.999), eps=eps, tensors=tensors[:2])
+    two = tensors[:2]
+
+    def step_two(active, expect):
+        nonlocal tensors
+        saved, tensors = tensors, two
+        try:
+            one_step(active, expect)
+        finally:
+            tensors = saved
+
+    step_two([0, 1], {})
+    step_two([1], {1: both(lambda b: np.float32(_pow32(b, 1) * b))})  # the object stood at 1 (T1's pow of step 1)
+    # T0(2): the object stands at 2 -> 3 != 2 -> pow(b,2);  T1(3): the object stands at 2 -> multiplies T0's value
+    step_two([0, 1], {0: both(lambda b: _pow32(b, 2)), 1: both(lambda b: np.float32(_pow32(b, 2) * b))})
+
+
+def test_every_tensor_carries_its_own_hyper_parameters():
+    """lr / betas / eps / weight_decay are read from state[p] per parameter (fp16_cpu_adam.py:596-601) and handed to
+    the tensor's own call (:407-410,416-428).  Bit for bit against fresh operator objects driven by hand; betas that
+    differ from the object's restart beta^t from pow on that call AND, because the object keeps them, on the next."""
+    tensors = _three_tensor_layout()
+    cs = _chunks(n_chunks=2, n=600, seed=71)
+    s = oracle.StaticScalerOracle(32)
+    opt = oracle.OptimizerStepOracle(cs, s, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True,
+                                     tensors=tensors)
+    opt.state(tensors[1])["lr"] = 5e-4
+    opt.state(tensors[1])["weight_decay"] = 0.0
+    opt.state(tensors[2])["betas"] = (0.8, 0.99)
+    opt.state(tensors[2])["eps"] = 1e-6
+    hyper = [(1e-3, 0.9, 0.999, 1e-8, 0.01), (5e-4, 0.9, 0.999, 1e-8, 0.0), (1e-3, 0.8, 0.99, 1e-6, 0.01)]
+    rng = np.random.default_rng(72)
+    for t in range(1, 6):
+        for c in cs:
+            c["p16"][...] = (rng.normal(0, 1e-3, c["p16"].size) * 32).astype(np.float16)
+        ref = _copy(cs)
+        opt.step()
+        for k, ((ci, off, numel), (lr, b1, b2, eps, wd)) in enumerate(zip(tensors, hyper)):
+            o = oracle.AdamOracle(1e-3, 0.9, 0.999, 1e-8, 0.01, True)
+            # by hand: T0 follows T2's call of the step before, whose betas were others -> pow; T1 follows T0 in the
+            # same step -> pow; T2's betas differ from T1's -> pow.  A fresh object at step 0 takes pow for t > 1 and
+            # multiplies 1 * beta for t == 1, which is the same float as pow(beta, 1).
+            sl = slice(off, off + numel)
+            o.update(t, lr, b1, b2, eps, wd, True, ref[ci]["p32"][sl], ref[ci]["p16"][sl], ref[ci]["m"][sl],
+                     ref[ci]["v"][sl], 32.0)
+        for c, r in zip(cs, ref):
+            for key in ("p32", "m", "v"):
+                assert np.array_equal(c[key].view(np.uint32), r[key].view(np.uint32)), (t, key)
+    # decoupled decay really was off for tensor 1 and on for the others: with zero gradient and moments only the
+    # decay moves a parameter
+    cs2 = _chunks(n_chunks=2, n=600, seed=73)
+    for c in cs2:
+        c["p16"][...] = 0
+        c["m"][...] = 0
+        c["v"][...] = 0
+    before = _copy(cs2)
+    opt2 = oracle.OptimizerStepOracle(cs2, None, lr=1e-2, weight_decay=0.1, use_adamw=True, tensors=tensors)
+    opt2.state(tensors[1])["weight_decay"] = 0.0
+    opt2.step()
+    assert np.array_equal(cs2[0]["p32"][250:550], before[0]["p32"][250:550])
+    want = before[0]["p32"][:250].astype(np.float64) * (1 - 1e-2 * 0.1)
+    assert np.allclose(cs2[0]["p32"][:250], want, rtol=1e-6, atol=0)

@@ -25,7 +25,7 @@ def _chunks(n_chunks, n, seed):
 def _existing(table, n_chunks, n):
     s = ps.DynamicLossScaler(init_scale=2)
     s.materialize("cuda:0")
-    _lib.check(_lib.load().ps_overflow_scan_chunks(table, n_chunks, n, s.state_ptr, _lib.current_stream_handle()), "scan")
+    _lib.check(_lib.load().ps_overflow_scan_chunks(table, n_chunks, n, None, s.state_ptr, _lib.current_stream_handle()), "scan")
     return int(s.overflow_flag)
 
 
