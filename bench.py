@@ -16,8 +16,11 @@ same run:
   tensor_list    ps_adam_step_tensors over a GPT-2-XL-shaped list of 580 tensors whose m / v tensors are packed in
                  other orders than the parameters (the reference's own packing);
   hybrid         the 12 B-parameter hybrid placement: 180 chunks, 60 of them in pinned host memory, streamed through
-                 double-buffered HBM staging; effective params/s, overlap efficiency, link rate and a CPU baseline for
-                 the host-resident share (the reference updates such chunks with its CPU operator);
+                 HBM staging slots; effective params/s, overlap efficiency, link rate and a CPU baseline for the
+                 host-resident share (the reference updates such chunks with its CPU operator); `fp16_in_hbm`: the same
+                 with the host positions' fp16 payloads kept in HBM, the form initialize_engine produces;
+  padded         the GPT-2-small-sized configuration: 124,439,808 parameters in 2 chunks of 64 Mi elements, the tail of
+                 the second chunk zero padding, which the step leaves alone: real parameters/s beside chunk slots/s;
   unfused_gpu_baseline   the reference's GPU branch restated with torch kernels;
   cpu_baseline   the CPU oracle (a port of the reference's AVX/OpenMP Adam) on this host: reported baseline only.
 `--mode ceiling` measures the memory system itself (pure read, pure write, 1:1 copy, the step's access pattern without
@@ -57,14 +60,16 @@ def parse_args():
     ap.add_argument("--hybrid-chunks", type=int, default=180, help="hybrid leg: chunk positions in all")
     ap.add_argument("--host-chunks", type=int, default=60, help="hybrid leg: how many of them live in pinned host memory (the LAST ones)")
     ap.add_argument("--hybrid-steps", type=int, default=3)
-    ap.add_argument("--slots", type=int, default=2, help="hybrid leg: HBM staging slots")
+    ap.add_argument("--slots", type=int, default=3, help="hybrid leg: HBM staging slots")
     ap.add_argument("--host-fp16", choices=["host", "hbm"], default="host",
                     help="hybrid leg: where a host-resident position keeps its fp16 payload (host: the whole "
                     "position is streamed, 14 B/element each way; hbm: only fp32 param / m / v are, 12 B/element)")
-    ap.add_argument("--mode", choices=["static", "dynamic", "hybrid", "ceiling"], default="static",
+    ap.add_argument("--mode", choices=["static", "dynamic", "hybrid", "ceiling", "operator"], default="static",
                     help="static: the 1.5 B-parameter configuration as specified (static loss scale, one fused kernel per step) "
                     "plus the extra legs. dynamic: the headline numbers are those of the dynamic step. hybrid: only the "
-                    "hybrid-placement leg, as its own JSON line. ceiling: streaming-kernel ceilings of the memory system")
+                    "hybrid-placement leg, as its own JSON line. ceiling: streaming-kernel ceilings of the memory system. "
+                    "operator: the per-tensor operator (ps_adam_update, what an unchanged FP16Adam loop calls) and the "
+                    "chunk-list step on ONE 64 Mi-element tensor / chunk")
     ap.add_argument("--arithmetic", choices=["operator", "torch"], default="operator",
                     help="operator: the native operator's order of operations (default, the headline line); "
                     "torch: the formula of the reference's GPU branch")
@@ -193,15 +198,39 @@ def cpu_baseline(reps, seconds):
 
 # ------------------------------------------------------------------------------------------------ hybrid leg
 
-def run_hybrid(args, with_cpu_baseline=True):
-    """The streamed hybrid configuration, then (its memory released) the same chunk list with everything resident."""
+def release_memory():
+    """Give freed device AND pinned host memory back to the system.  A later leg then pins fresh host memory, as an
+    optimizer does once when it is built: pinned blocks handed out again by torch's caching host allocator (in another
+    order than they were first allocated) measured 49 -> 32-39 GB/s each way on the streamed step."""
     import gc
 
     import torch
 
-    out = run_streamed(args, with_cpu_baseline)
     gc.collect()
     torch.cuda.empty_cache()
+    empty_host = getattr(torch._C, "_host_emptyCache", None)
+    if empty_host is not None:
+        empty_host()
+
+
+def run_hybrid(args, with_cpu_baseline=True):
+    """The streamed hybrid configuration, then (its memory released) the same chunk list with everything resident."""
+    out = run_streamed(args, with_cpu_baseline)
+    release_memory()
+    if "skipped" not in out and args.host_chunks and args.host_fp16 == "host":
+        # the form initialize_engine produces: a module's parameters are views of the fp16 payloads, which therefore stay
+        # in HBM; only fp32 param / m / v of a host position cross the link (12 instead of 14 B/element each way)
+        import copy
+
+        hbm_args = copy.copy(args)
+        hbm_args.host_fp16 = "hbm"
+        try:
+            leg = run_streamed(hbm_args, with_cpu_baseline=False, with_link_probe=False)
+        except Exception as e:
+            leg = {"skipped": f"{type(e).__name__}: {str(e)[:200]}"}
+        out["fp16_in_hbm"] = {k: v for k, v in leg.items() if k not in ("link_duplex_GBps_each_way", "link_duplex_floor_s",
+                                                                        "wall_over_link_duplex_floor")}
+        release_memory()
     if "skipped" not in out and args.host_chunks:
         # BASELINE's split (a third of the positions on the host) is given; this GPU's 288 GB hold the whole list, which is
         # what the placement rule of the engine (PatrickStarClient.plan_placement) decides when nobody forces a policy
@@ -209,12 +238,11 @@ def run_hybrid(args, with_cpu_baseline=True):
             out["all_resident"] = run_all_resident(args)
         except Exception as e:
             out["all_resident"] = {"skipped": f"{type(e).__name__}: {str(e)[:200]}"}
-        gc.collect()
-        torch.cuda.empty_cache()
+        release_memory()
     return out
 
 
-def run_streamed(args, with_cpu_baseline=True):
+def run_streamed(args, with_cpu_baseline=True, with_link_probe=True):
     """The hybrid-placement configuration: C chunks, the last H of them in pinned host memory, streamed through HBM staging.
     Reports effective params/s over the whole list and the overlap efficiency
     max(kernel total, H2D total, D2H total) / wall.  Returns a dict; {"skipped": reason} if the memory is not there."""
@@ -327,7 +355,7 @@ def run_streamed(args, with_cpu_baseline=True):
     # What the link gives when both directions are busy: plain copies of the pipeline's piece sizes, downward on one
     # stream and upward on another, nothing else running.  A perfectly overlapped pipeline cannot beat link bytes / this.
     duplex_rate = None
-    if len(host_pos) >= 2:
+    if len(host_pos) >= 2 and with_link_probe:
         slot_up = [torch.empty_like(t) for t in slot]
         side = [torch.cuda.Stream(), torch.cuda.Stream()]
         reps = 6
@@ -577,6 +605,63 @@ def dynamic_leg(cfg, steps, warmup):
     }
 
 
+def padded_leg(args, steps, warmup):
+    """The GPT-2-small-sized configuration: 124,439,808 parameters packed into 2 chunks of 64 Mi elements, the last
+    9,777,920 slots of the second chunk zero padding.  The step leaves the padding alone (zeros are a fixed point of
+    the update); timed beside the same step made over every slot."""
+    import torch
+
+    import patrickstar_amd as ps
+    from patrickstar_amd import _lib
+
+    N, real = N_CHUNK, 124_439_808
+    dev = torch.device("cuda:0")
+    client = ps.PatrickStarClient(0, N)
+    params = client.append_flat_chunks(2, used_numel_last=real - N)
+    opt = ps.FP16Adam(client, params, loss_scaler=ps.LossScaler(2**16), use_adamw=True, **HYPER)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(0)
+    cl = client.chunk_list
+    for pos, p in zip(client.positions(), params):
+        n = p.ps_attr.numel
+        cl[pos.fp32].payload[:n].normal_(0, 0.02, generator=gen)
+        cl[pos.exp_avg].payload[:n].normal_(0, 1e-4, generator=gen)
+        cl[pos.exp_avg_sq].payload[:n].normal_(0, 1e-6, generator=gen).abs_()
+        cl[pos.fp16].payload[:n].copy_(torch.empty(n, device=dev).normal_(0, 1e-3, generator=gen).mul_(2.0**16))
+    for p in params:
+        dict.__setitem__(opt.state[p], "step", 99 - warmup)
+    ms, kernel_ms = time_steps(torch, opt.step, steps, warmup)
+    avg = sum(kernel_ms) / len(kernel_ms)
+    # the same two chunks with every slot updated (no used lengths), through the C ABI
+    table, n_dev, _ = opt._tables
+    lib = _lib.load()
+    lib.ps_adam_create(994, HYPER["lr"], 0.9, 0.999, HYPER["eps"], HYPER["weight_decay"], 1, 0)
+    t = [200]
+
+    def every_slot():
+        t[0] += 1
+        _lib.check(lib.ps_adam_step_chunks(994, t[0], HYPER["lr"], 0.9, 0.999, HYPER["eps"], HYPER["weight_decay"], 1, table, n_dev, N,
+                                           None, None, 65536.0, _lib.current_stream_handle()), "ps_adam_step_chunks")
+
+    _, all_ms = time_steps(torch, every_slot, steps, warmup)
+    lib.ps_adam_destroy(994)
+    tail_zero = bool((cl[client.positions()[1].fp32].payload[real - N:] == 0).all()) and bool(
+        (cl[client.positions()[1].fp16].payload[real - N:] == 0).all())
+    all_avg = sum(all_ms) / len(all_ms)
+    del opt, client, params
+    torch.cuda.empty_cache()
+    return {
+        "workload": f"GPT-2-small-sized: {real} parameters in 2 chunks x {N} elements ({2 * N} slots, {2 * N - real} of them zero "
+        "padding behind the last tensor), AdamW wd 0.01 lr 1e-4, static loss scale 2^16, first timed step t=100",
+        "real_params": real, "slots": 2 * N,
+        "real_params_per_s": real / (ms * 1e-3), "slots_per_s": 2 * N / (ms * 1e-3), "ms_per_step": ms, "avg_device_ms": avg,
+        "achieved_GBps": 28 * real / (avg * 1e-3) / 1e9, "frac": 28 * real / (avg * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "every_slot_updated": {"avg_device_ms": all_avg, "real_params_per_s": real / (all_avg * 1e-3),
+                               "achieved_GBps": 28 * 2 * N / (all_avg * 1e-3) / 1e9},
+        "padding_still_zero": tail_zero,
+    }
+
+
 def gpt2_xl_tensor_sizes():
     d, layers = 1600, 48
     sizes = [50257 * d, 1024 * d]
@@ -626,7 +711,8 @@ def tensor_list_leg(cfg, steps, warmup):
 
         ms, kernel_ms = time_steps(torch, step, steps, warmup)
         avg = sum(kernel_ms) / len(kernel_ms)
-        return {"value": total / (ms * 1e-3), "unit": "params/s", "ms_per_step": ms, "avg_device_ms": avg,
+        return {"value": total / (ms * 1e-3), "unit": "params/s", "real_params_per_s": total / (ms * 1e-3), "ms_per_step": ms,
+                "avg_device_ms": avg,
                 "achieved_GBps": 28 * total / (avg * 1e-3) / 1e9, "frac": 28 * total / (avg * 1e-3) / 1e9 / HBM_PEAK_GBS}
 
     # the unfavourable case of the reference's packing first (momentum and variance at other offsets than their parameters:
@@ -640,6 +726,89 @@ def tensor_list_leg(cfg, steps, warmup):
     })
     lib.ps_adam_destroy(993)
     return out
+
+
+def calibration_copy(torch, dev):
+    """One plain device-to-device copy of 1 Gi floats (4 GiB read, 4 GiB written): a kernel of known traffic for a
+    rocprofv3 --pmc run to scale FETCH_SIZE / WRITE_SIZE by."""
+    src = torch.empty(1 << 30, dtype=torch.float32, device=dev).normal_()
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+
+
+def operator_mode(args):
+    """ps_adam_update (the reference's adam_update on one flat tensor, the form its unchanged per-tensor loop calls,
+    patrickstar/ops/fp16_cpu_adam.py:415-428) on ONE tensor of `--chunk-size` elements, beside the chunk-list step on one
+    chunk of the same buffers.  One JSON line; every entry is over `--steps` launches, each timed with its own pair of
+    events on the launch stream."""
+    import torch
+
+    import patrickstar_amd as ps
+    from patrickstar_amd import _lib
+
+    dev = torch.device("cuda:0")
+    N = args.chunk_size
+    client = ps.PatrickStarClient(0, N)
+    params = client.append_flat_chunks(4)  # four positions out of one slab per list; position 1 is the tensor
+    opt = ps.FP16Adam(client, params, loss_scaler=ps.LossScaler(2**12), use_adamw=True, **HYPER)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(0)
+    cl = client.chunk_list
+    for pos in client.positions():
+        cl[pos.fp32].payload.normal_(0, 0.02, generator=gen)
+        cl[pos.exp_avg].payload.normal_(0, 1e-4, generator=gen)
+        cl[pos.exp_avg_sq].payload.normal_(0, 1e-6, generator=gen).abs_()
+        cl[pos.fp16].payload.copy_(torch.empty(N, device=dev).normal_(0, 1e-3, generator=gen).mul_(2.0**12))
+    if args.calibration_copy:
+        calibration_copy(torch, dev)
+    q = client.positions()[1]
+    p, m, v, h = (cl[c].payload for c in (q.fp32, q.exp_avg, q.exp_avg_sq, q.fp16))
+    lib = _lib.load()
+    lib.ps_adam_create(995, HYPER["lr"], 0.9, 0.999, HYPER["eps"], HYPER["weight_decay"], 1, 0)
+    t = [100]
+
+    def update(p, g, m, v, out, n, half=True):
+        t[0] += 1
+        _lib.check(lib.ps_adam_update(995, t[0], HYPER["lr"], 0.9, 0.999, HYPER["eps"], HYPER["weight_decay"], 1, p.data_ptr(), g.data_ptr(),
+                                      int(half), m.data_ptr(), v.data_ptr(), n, 4096.0, out.data_ptr() if out is not None else None,
+                                      _lib.current_stream_handle()), "ps_adam_update")
+
+    one = _lib.chunk_array([[p.data_ptr(), m.data_ptr(), v.data_ptr(), h.data_ptr()]])
+
+    def chunk_step():
+        t[0] += 1
+        _lib.check(lib.ps_adam_step_chunks(995, t[0], HYPER["lr"], 0.9, 0.999, HYPER["eps"], HYPER["weight_decay"], 1, one, 1, N, None,
+                                           None, 4096.0, _lib.current_stream_handle()), "ps_adam_step_chunks")
+
+    def entry(fn, bytes_per_element, n, what):
+        _, ms = time_steps(torch, fn, args.steps, args.warmup)
+        avg, med = sum(ms) / len(ms), sorted(ms)[len(ms) // 2]
+        gbps = bytes_per_element * n / (avg * 1e-3) / 1e9
+        return {"what": what, "bytes_per_element": bytes_per_element, "avg_device_ms": avg, "median_device_ms": med,
+                "min_device_ms": min(ms), "achieved_GBps": gbps, "frac": gbps / HBM_PEAK_GBS, "params_per_s": n / (avg * 1e-3)}
+
+    g32 = torch.empty(N, device=dev).normal_(0, 4.0, generator=gen)
+    out = {
+        "metric": "Adam params/sec + achieved HBM GB/s, the per-tensor operator on one tensor, 1 GPU",
+        "config": {"workload": f"one tensor of {N} elements inside a four-chunk slab, AdamW hyper-parameters of the 1.5 B configuration, "
+                   "static loss scale 2^12", "chunk_numel": N},
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "unit": "params/s", "dtype": "f32", "data": "synthetic",
+        "update_fp16_out": entry(lambda: update(p, h, m, v, h, N), 28, N,
+                                 "ps_adam_update, fp16 gradients overwritten by the fp16 parameters (28 B/element)"),
+        "update_no_fp16_out": entry(lambda: update(p, h, m, v, None, N), 26, N,
+                                    "ps_adam_update as the reference's operator is called: no fp16 output (26 B/element)"),
+        "update_offset_1": entry(lambda: update(p[1:], h[1:], m[1:], v[1:], h[1:], N - 1), 28, N - 1,
+                                 "the same tensor one element into its chunk (28 B/element)"),
+        "update_fp32_grads": entry(lambda: update(p, g32, m, v, h, N, half=False), 30, N,
+                                   "fp32 gradients, fp16 output (30 B/element)"),
+        "chunk_step_one_chunk": entry(chunk_step, 28, N, "ps_adam_step_chunks over one chunk (28 B/element)"),
+    }
+    out["value"] = out["update_fp16_out"]["params_per_s"]
+    out["ms_per_step"] = out["update_fp16_out"]["avg_device_ms"]
+    lib.ps_adam_destroy(995)
+    print(json.dumps(out))
 
 
 PROBE_SOURCE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "bench_kernels", "ps_stream_probe.hip")
@@ -797,6 +966,8 @@ def main():
     torch.cuda.set_device(0)
     if args.mode == "ceiling":
         return ceiling(args)
+    if args.mode == "operator":
+        return operator_mode(args)
     if args.mode == "hybrid":
         leg = run_hybrid(args, with_cpu_baseline=not args.no_cpu_baseline)
         if "skipped" in leg:
@@ -823,11 +994,7 @@ def main():
     for p in cfg.params:
         dict.__setitem__(cfg.opt.state[p], "step", 99 - args.warmup)
     if args.calibration_copy:
-        src = torch.empty(1 << 30, dtype=torch.float32, device=cfg.dev).normal_()
-        dst = torch.empty_like(src)
-        dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
+        calibration_copy(torch, cfg.dev)
     elements = C * N
     static_ms, static_kernel_ms = time_steps(torch, cfg.opt.step, args.steps, args.warmup)
     extras = {}
@@ -835,6 +1002,10 @@ def main():
         extras["dynamic"] = dynamic_leg(cfg, args.steps, args.warmup)
     if not args.no_extras:
         extras["tensor_list"] = tensor_list_leg(cfg, max(5, args.steps // 2), 2)
+        try:
+            extras["padded"] = padded_leg(args, args.steps, args.warmup)
+        except Exception as e:
+            extras["padded"] = {"skipped": f"{type(e).__name__}: {str(e)[:200]}"}
 
     if args.mode == "dynamic":
         d = extras.pop("dynamic")
@@ -871,6 +1042,9 @@ def main():
             "mode": args.mode,
             "arithmetic": args.arithmetic,
         },
+        # every slot of the 24 chunks is updated: the workload is the full chunk list (GPT-2 XL's own 1,557,611,200
+        # parameters would leave 3.3 % of the slots as padding; `padded` and `tensor_list` report real-parameter rates)
+        "slots_per_s": elements / (ms_per_step * 1e-3),
         "roofline": {
             "bound": "hbm",
             "achieved": achieved,

@@ -664,11 +664,11 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
 #undef PS_FLAT
     };
 
-    // Tensors handed to the operator are views at one element offset into the four chunk
-    // payloads, so their addresses normally share a phase relative to 16-byte (4-element)
-    // boundaries: whole 256-element tiles with vector accesses from the first aligned element on;
-    // the up to 3 elements before it and the remainder behind the last tile go element-wise, in
-    // the same launch.
+    // Tensors handed to the operator are views at one element offset into the four chunk payloads, so their
+    // addresses normally share a phase relative to 16-byte (4-element) boundaries: whole 256-element tiles with
+    // vector accesses from the fp32 parameter's first 1 KiB boundary on (every wave access then covers one aligned
+    // KiB); the up to 255 elements before it and the remainder behind the last whole tile go element-wise, in the
+    // same launch.
     auto elem_phase = [](const void* a, size_t elem_size) -> int {
         uintptr_t u = reinterpret_cast<uintptr_t>(a);
         if (u % elem_size) return -1;
@@ -683,35 +683,68 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
     const bool state_aligned = elem_phase(d_exp_avg, 4) == ph && elem_phase(d_exp_avg_sq, 4) == ph;
     if (!vec_ok) {
         scalar_span(0, numel);
-    } else {
-        const size_t head = (size_t)((4 - ph) & 3);
-        const size_t n_tiles = (numel - head) / 256;
-        const int tail = (int)(numel - head - n_tiles * 256);
-        dim3 grid(grid_1d(n_tiles + 1)), block(64);  // + 1: the workgroup that does head and tail
-        uint16_t* out = d_param_fp16_out ? d_param_fp16_out + head : nullptr;
-#define PS_FLAT_VEC_AS(WD, HALF, DWORD)                                                           \
-    hipLaunchKernelGGL((adam_flat_vec_kernel<WD, HALF, DWORD>), grid, block, kLdsBytes, s, c,     \
-                       d_params + head, static_cast<const void*>(gbytes + head * gsz),            \
-                       d_exp_avg + head, d_exp_avg_sq + head, out, n_tiles, (int)head, tail)
-#define PS_FLAT_VEC(WD, HALF)                       \
-    do {                                            \
-        if (state_aligned)                          \
-            PS_FLAT_VEC_AS(WD, HALF, false);        \
-        else                                        \
-            PS_FLAT_VEC_AS(WD, HALF, true);         \
-    } while (0)
-        if (grads_are_half) {
-            if (c.wd_mode == WD_DECOUPLED) PS_FLAT_VEC(WD_DECOUPLED, true);
-            else if (c.wd_mode == WD_L2) PS_FLAT_VEC(WD_L2, true);
-            else PS_FLAT_VEC(WD_NONE, true);
-        } else {
-            if (c.wd_mode == WD_DECOUPLED) PS_FLAT_VEC(WD_DECOUPLED, false);
-            else if (c.wd_mode == WD_L2) PS_FLAT_VEC(WD_L2, false);
-            else PS_FLAT_VEC(WD_NONE, false);
-        }
-#undef PS_FLAT_VEC
-#undef PS_FLAT_VEC_AS
+        PS_HIP(hipGetLastError());
+        return 0;
     }
+    const size_t head = (size_t)((kTile - (reinterpret_cast<uintptr_t>(d_params) / sizeof(float)) % kTile) % kTile);
+    // one tile per workgroup: a tensor beyond the launch grid (2^39 elements) goes in several launches
+    const size_t max_tiles = kMaxGridX - 1;
+    size_t done = 0;  // elements behind the head that earlier launches of this call have covered
+    const size_t body = numel - head;
+    do {
+        const size_t left = body - done;
+        const bool last = left / kTile <= max_tiles;
+        const size_t n_tiles = last ? left / kTile : max_tiles;
+        const int tail = last ? (int)(left - n_tiles * kTile) : 0;
+        const int this_head = done == 0 ? (int)head : 0;
+        const size_t at = head + done;
+        dim3 grid((unsigned)(n_tiles + 1)), block(kBlock);  // + 1: the workgroup that does head and tail
+        uint16_t* out = d_param_fp16_out ? d_param_fp16_out + at : nullptr;
+#define PS_FLAT_VEC_5(WD, UNS, HALF, OUT, DWORD)                                                              \
+    hipLaunchKernelGGL((adam_flat_vec_kernel<WD, UNS, HALF, OUT, DWORD>), grid, block, kLdsBytes, s, c,       \
+                       d_params + at, static_cast<const void*>(gbytes + at * gsz), d_exp_avg + at,            \
+                       d_exp_avg_sq + at, out, n_tiles, this_head, tail)
+#define PS_FLAT_VEC_4(WD, UNS, HALF, OUT)                  \
+    do {                                                   \
+        if (state_aligned)                                 \
+            PS_FLAT_VEC_5(WD, UNS, HALF, OUT, false);      \
+        else                                               \
+            PS_FLAT_VEC_5(WD, UNS, HALF, OUT, true);       \
+    } while (0)
+#define PS_FLAT_VEC_3(WD, UNS, HALF)                       \
+    do {                                                   \
+        if (out != nullptr)                                \
+            PS_FLAT_VEC_4(WD, UNS, HALF, true);            \
+        else                                               \
+            PS_FLAT_VEC_4(WD, UNS, HALF, false);           \
+    } while (0)
+#define PS_FLAT_VEC_2(WD, UNS)                             \
+    do {                                                   \
+        if (grads_are_half)                                \
+            PS_FLAT_VEC_3(WD, UNS, true);                  \
+        else                                               \
+            PS_FLAT_VEC_3(WD, UNS, false);                 \
+    } while (0)
+#define PS_FLAT_VEC_1(WD)                                  \
+    do {                                                   \
+        if (c.unscale == UNSCALE_MUL)                      \
+            PS_FLAT_VEC_2(WD, UNSCALE_MUL);                \
+        else if (c.unscale == UNSCALE_DIV)                 \
+            PS_FLAT_VEC_2(WD, UNSCALE_DIV);                \
+        else                                               \
+            PS_FLAT_VEC_2(WD, UNSCALE_NONE);               \
+    } while (0)
+        if (c.wd_mode == WD_DECOUPLED) PS_FLAT_VEC_1(WD_DECOUPLED);
+        else if (c.wd_mode == WD_L2) PS_FLAT_VEC_1(WD_L2);
+        else PS_FLAT_VEC_1(WD_NONE);
+#undef PS_FLAT_VEC_1
+#undef PS_FLAT_VEC_2
+#undef PS_FLAT_VEC_3
+#undef PS_FLAT_VEC_4
+#undef PS_FLAT_VEC_5
+        PS_HIP(hipGetLastError());
+        done += n_tiles * kTile + tail;
+    } while (done < body);
     PS_HIP(hipGetLastError());
     return 0;
 }
