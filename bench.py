@@ -920,6 +920,20 @@ def ceiling(args):
         e["plain_copy_GBps"] = 8 * k * n_win / (measure(plain_copies) * 1e-3) / 1e9
         e["read_then_copy_GBps"] = 8 * k * n_win / (measure(read_then_copy) * 1e-3) / 1e9
         windows[f"{mib}MiB"] = {key: round(val, 1) for key, val in e.items()}
+    # Does it matter where in a KiB a wave's 1 KiB access starts?  The same kernels with the base address moved by a
+    # part of a KiB (every access still covers whole 128-byte lines).  The tensor-list step meets this when momentum and
+    # variance tensors are packed at other offsets than their parameters (the reference's own packing).
+    phases = {}
+    n_ph = n - 256 * 8 * 4  # room behind the shifted base
+    for shift in ((0, 256) if args.no_sweep else (0, 128, 256, 512, 768, 1024)):
+        phases[f"{shift}B"] = {
+            "read": round(4 * n_ph / (measure(lambda: probe.ps_probe_read(p.data_ptr() + shift, n_ph, sink.data_ptr(), 8, 26, s())) * 1e-3) / 1e9, 1),
+            "write": round(4 * n_ph / (measure(lambda: probe.ps_probe_write(m.data_ptr() + shift, n_ph, 0.0, 4, 40, s())) * 1e-3) / 1e9, 1),
+            "copy_source_shifted": round(8 * n_ph / (measure(lambda: probe.ps_probe_copy(p.data_ptr() + shift, m.data_ptr(), n_ph, 1, 0, s())) * 1e-3) / 1e9, 1),
+            "copy_destination_shifted": round(8 * n_ph / (measure(lambda: probe.ps_probe_copy(p.data_ptr(), m.data_ptr() + shift, n_ph, 1, 0, s())) * 1e-3) / 1e9, 1),
+            "update4_two_of_four_arrays_shifted": round(28 * n_ph / (measure(lambda: probe.ps_probe_update4(
+                p.data_ptr(), m.data_ptr() + shift, v.data_ptr() + shift, h.data_ptr(), n_ph, 1, 26, s())) * 1e-3) / 1e9, 1),
+        }
     # the probe kernels have rewritten the lists: refill what the optimizer kernels need to stay finite
     m.normal_(0, 1e-4)
     v.normal_(0, 1e-6).abs_()
@@ -944,11 +958,13 @@ def ceiling(args):
         "time_sliced_bound_GBps": 28.0 / (14.0 / r + 14.0 / w),
         "sweeps_GBps": sweeps,
         "windows": windows,
+        "phase_of_a_KiB_GBps": phases,
         "note": "probe_*: best launch shape of the sweep (sweeps_GBps holds every shape); time_sliced_bound: 14 B/element read at the "
         "pure-read rate plus 14 B/element written at the pure-write rate, as if reads and writes never met on the memory bus; "
         "probe_update4 is the step's access pattern without its arithmetic; windows: reread = the pure-read kernel launched repeatedly "
         "over one window of that size (a window of up to 256 MiB fits the memory-side cache), plain_copy / read_then_copy = 4 GiB "
-        "copied window by window, without and with a pure-read pass over each window just before its copy (GB/s of the copy's bytes)",
+        "copied window by window, without and with a pure-read pass over each window just before its copy (GB/s of the copy's bytes); "
+        "phase_of_a_KiB_GBps: the read / write / copy / update4 kernels with a base address moved by part of a KiB",
     }
     print(json.dumps(out))
 
