@@ -137,11 +137,16 @@ std::shared_ptr<HostAdam> find_opt(int id)
 
 // ------------------------------------------------------------ launch helpers
 
-constexpr size_t kMaxGridX = 0x7FFFFFFFull;
+// The runtime refuses a launch whose grid times block size reaches 2^32 threads in a dimension.  Kernels that take one
+// tile per single-wave workgroup are checked against kMaxGridX before anything is queued (2^26 - 1 tiles: chunks and
+// tensors of up to 17 G elements); kernels that loop over their tiles are simply capped (grid_1d).
+constexpr size_t kMaxGridX = 0xFFFFFFFFull / 64;
+static_assert(kBlock == 64 && kScanBlock == 64, "kMaxGridX is for 64-thread workgroups");
 
-unsigned grid_1d(size_t n_blocks)
+unsigned grid_1d(size_t n_blocks, size_t block_threads)
 {
-    size_t g = n_blocks < kMaxGridX ? n_blocks : kMaxGridX;
+    const size_t most = 0xFFFFFFFFull / block_threads;
+    size_t g = n_blocks < most ? n_blocks : most;
     return (unsigned)(g ? g : 1);
 }
 
@@ -646,7 +651,7 @@ int ps_adam_update(int optimizer_id, size_t step, float lr, float beta1, float b
     auto scalar_span = [&](size_t lo, size_t hi) {
         if (hi <= lo) return;
         const size_t n = hi - lo;
-        dim3 grid(grid_1d((n + kAuxBlock - 1) / kAuxBlock)), block(kAuxBlock);
+        dim3 grid(grid_1d((n + kAuxBlock - 1) / kAuxBlock, kAuxBlock)), block(kAuxBlock);
         uint16_t* out = d_param_fp16_out ? d_param_fp16_out + lo : nullptr;
 #define PS_FLAT(WD, HALF)                                                                      \
     hipLaunchKernelGGL((adam_flat_kernel<WD, HALF>), grid, block, 0, s, c, d_params + lo,      \
@@ -1131,7 +1136,7 @@ int ps_cast_fp32_to_fp16(const float* d_src, uint16_t* d_dst, size_t numel, ps_s
     if (numel == 0) return 0;
     if (!d_src || !d_dst) return fail(PS_ERR_BAD_ARG, "ps_cast_fp32_to_fp16: NULL pointer");
     size_t n_tiles = (numel + kTile - 1) / kTile;
-    hipLaunchKernelGGL(cast_kernel, dim3(grid_1d(n_tiles)), dim3(kBlock), 0,
+    hipLaunchKernelGGL(cast_kernel, dim3(grid_1d(n_tiles, kBlock)), dim3(kBlock), 0,
                        static_cast<hipStream_t>(stream), d_src, d_dst, numel, n_tiles);
     PS_HIP(hipGetLastError());
     return 0;
@@ -1277,7 +1282,7 @@ int ps_overflow_scan_host_chunks(const ps_chunk* host_chunks, int n_chunks, size
     // fp16 payloads that live in HBM are probed in place on the caller's stream
     for (int k = 0; k < n_chunks; ++k) {
         if (!fp16_in_hbm[k] || a.numel_of(k) == 0) continue;
-        hipLaunchKernelGGL(scan_f16_kernel, dim3(grid_1d(tiles_of(k))), dim3(kScanBlock), kScanLdsBytes, caller,
+        hipLaunchKernelGGL(scan_f16_kernel, dim3(grid_1d(tiles_of(k), kScanBlock)), dim3(kScanBlock), kScanLdsBytes, caller,
                            host_chunks[k].param_fp16, a.numel_of(k), tiles_of(k), d_state);
         PS_HIP(hipGetLastError());
     }
@@ -1297,7 +1302,7 @@ int ps_overflow_scan_host_chunks(const ps_chunk* host_chunks, int n_chunks, size
                               hipMemcpyHostToDevice, p->h2d));
         PS_HIP(hipEventRecord(p->h2d_done[s], p->h2d));
         PS_HIP(hipStreamWaitEvent(p->compute, p->h2d_done[s], 0));
-        hipLaunchKernelGGL(scan_f16_kernel, dim3(grid_1d(tiles_of(k))), dim3(kScanBlock), kScanLdsBytes, p->compute,
+        hipLaunchKernelGGL(scan_f16_kernel, dim3(grid_1d(tiles_of(k), kScanBlock)), dim3(kScanBlock), kScanLdsBytes, p->compute,
                            staging[s].param_fp16, a.numel_of(k), tiles_of(k), d_state);
         PS_HIP(hipGetLastError());
         PS_HIP(hipEventRecord(p->compute_done[s], p->compute));
@@ -1399,7 +1404,7 @@ int ps_overflow_scan(const uint16_t* d_grads_fp16, size_t numel, ps_step_state* 
     if (numel == 0) return 0;
     if (!d_grads_fp16) return fail(PS_ERR_BAD_ARG, "d_grads_fp16 is NULL");
     size_t n_tiles = (numel + kScanTile - 1) / kScanTile;
-    hipLaunchKernelGGL(scan_f16_kernel, dim3(grid_1d(n_tiles)), dim3(kScanBlock), kScanLdsBytes,
+    hipLaunchKernelGGL(scan_f16_kernel, dim3(grid_1d(n_tiles, kScanBlock)), dim3(kScanBlock), kScanLdsBytes,
                        static_cast<hipStream_t>(stream), d_grads_fp16, numel, n_tiles, d_state);
     PS_HIP(hipGetLastError());
     return 0;
@@ -1412,7 +1417,7 @@ int ps_overflow_scan_f32(const float* d_grads_fp32, size_t numel, ps_step_state*
     if (numel == 0) return 0;
     if (!d_grads_fp32) return fail(PS_ERR_BAD_ARG, "d_grads_fp32 is NULL");
     size_t blocks = (numel + (size_t)kAuxBlock * 16 - 1) / ((size_t)kAuxBlock * 16);
-    hipLaunchKernelGGL(scan_f32_kernel, dim3(grid_1d(blocks)), dim3(kAuxBlock), 0,
+    hipLaunchKernelGGL(scan_f32_kernel, dim3(grid_1d(blocks, kAuxBlock)), dim3(kAuxBlock), 0,
                        static_cast<hipStream_t>(stream), d_grads_fp32, numel, d_state);
     PS_HIP(hipGetLastError());
     return 0;
@@ -1473,7 +1478,7 @@ int ps_grad_to_chunk(const void* d_grad, int grad_is_half, uint16_t* d_slot_fp16
         if (hi <= lo) return;
         const size_t n = hi - lo;
         size_t blocks = (n + (size_t)kAuxBlock * 4 - 1) / ((size_t)kAuxBlock * 4);
-        dim3 grid(grid_1d(blocks)), block(kAuxBlock);
+        dim3 grid(grid_1d(blocks, kAuxBlock)), block(kAuxBlock);
         const void* src = gbytes + lo * esz;
         if (grad_is_half)
             hipLaunchKernelGGL(grad_to_chunk_kernel<true>, grid, block, 0, s, src, d_slot_fp16 + lo, n, d_state);
@@ -1493,7 +1498,7 @@ int ps_grad_to_chunk(const void* d_grad, int grad_is_half, uint16_t* d_slot_fp16
         const size_t body_end = head + n_vec * 8;
         scalar_span(0, head);
         size_t blocks = (n_vec + kAuxBlock - 1) / kAuxBlock;
-        dim3 grid(grid_1d(blocks)), block(kAuxBlock);
+        dim3 grid(grid_1d(blocks, kAuxBlock)), block(kAuxBlock);
         uint16_t* dst_al = d_slot_fp16 + head;
         if (grad_is_half) {
             const uintptr_t first = src + head * 2;

@@ -303,8 +303,11 @@ def test_argument_checks_happen_before_any_gpu_work():
     assert lib.ps_scaler_update(ctypes.c_void_p(16), 3, None, 0, 1, None) == E
     assert lib.ps_scaler_update(ctypes.c_void_p(16), 0, None, 0, -1, None) == E
     assert lib.ps_state_seed_step(ctypes.c_void_p(16), -1, 0.9, 0.999, 1, None) == E
-    # sizes beyond what one launch grid can cover (2^31 - 1 tiles per chunk) are refused by every chunk-list entry point;
-    # 2^62 elements is beyond the limit of each of them, whatever its tile size
+    # sizes beyond what one launch grid can cover (the runtime refuses 2^32 threads in a dimension: 2^26 - 1 tiles of 256
+    # elements per chunk) are refused by every chunk-list entry point; 2^62 elements is beyond the limit of each of them,
+    # whatever its tile size
+    assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, 1, 2**34, None, None, 1.0, None) == E
+    assert b"beyond the launch grid" in lib.ps_last_error()
     huge = 2**62
     flag = ctypes.c_void_p(16)
     assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, 1, huge, None, None, 1.0, None) == E
@@ -317,6 +320,33 @@ def test_argument_checks_happen_before_any_gpu_work():
     one = (ctypes.c_size_t * 1)(huge)
     assert lib.ps_adam_step_tensors(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, one, 1, None, 1.0, None, None) == E
     assert b"beyond the launch grid" in lib.ps_last_error()
+    # the per-tensor form: every record is looked at before the operator object moves or anything is queued
+    numels = (ctypes.c_size_t * 2)(100, 200)
+    two = _lib.chunk_array([[16, 16, 16, 16], [16, 16, 16, 16]])
+    each = (_lib.ps_tensor_call * 2)()
+    for e in each:
+        e.lr, e.beta1, e.beta2, e.eps, e.weight_decay, e.step, e.arithmetic = 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, -1
+    assert lib.ps_adam_step_tensors_each(4711, 1, two, numels, each, 2, 1.0, None, None, 0, None) == _lib.PS_ERR_UNKNOWN_ID
+    assert lib.ps_adam_step_tensors_each(88, 1, two, numels, None, 2, 1.0, None, None, 0, None) == E
+    each[1].arithmetic = 7
+    assert lib.ps_adam_step_tensors_each(88, 1, two, numels, each, 2, 1.0, None, None, 0, None) == E
+    assert b"each[1].arithmetic" in lib.ps_last_error()
+    each[1].arithmetic, each[1].step = _lib.PS_ARITH_TORCH, 0
+    assert lib.ps_adam_step_tensors_each(88, 1, two, numels, each, 2, 1.0, None, None, 0, None) == E
+    assert b"at least 1" in lib.ps_last_error()
+    # device-decided: a distance of 0 or less is fine, a workspace that is missing, short or misaligned is not
+    assert lib.ps_tensors_each_workspace_bytes(2) == 128 and lib.ps_tensors_each_workspace_bytes(0) == 0
+    assert lib.ps_adam_step_tensors_each(88, 1, two, numels, each, 2, 1.0, flag, None, 0, None) == E
+    assert lib.ps_adam_step_tensors_each(88, 1, two, numels, each, 2, 1.0, flag, ctypes.c_void_p(4096), 127, None) == E
+    assert b"needs 128" in lib.ps_last_error()
+    assert lib.ps_adam_step_tensors_each(88, 1, two, numels, each, 2, 1.0, flag, ctypes.c_void_p(4104), 128, None) == E
+    assert b"16-byte aligned" in lib.ps_last_error()
+    numels[1] = huge
+    assert lib.ps_adam_step_tensors_each(88, 1, two, numels, each, 2, 1.0, flag, ctypes.c_void_p(4096), 128, None) == E
+    # used lengths beyond the chunk
+    used = (ctypes.c_size_t * 1)(1025)
+    assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, 1, 1024, used, None, 1.0, None) == E
+    assert b"used_numel" in lib.ps_last_error()
     # negative counts and a call pattern that does not fit the list
     assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, -1, 1024, None, None, 1.0, None) == E
     assert lib.ps_adam_step_chunks(88, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, fake, 1, 1024, None, _lib.call_pattern(2, 1, 0, 10), 1.0, None) == E
