@@ -34,7 +34,7 @@ class ChunkPosition:
         self.fp16, self.fp32, self.exp_avg, self.exp_avg_sq, self.on_host = fp16, fp32, exp_avg, exp_avg_sq, on_host
 
 
-def plan_host_positions(n_positions, chunk_size, free_bytes, staging_slots=2, margin_use_ratio=0.8,
+def plan_host_positions(n_positions, chunk_size, free_bytes, staging_slots=3, margin_use_ratio=0.8,
                         host_keeps_fp16=True):
     """Which chunk positions to keep in pinned host memory when ``free_bytes`` of HBM are available.
 
@@ -84,7 +84,7 @@ class PatrickStarClient:
         self.use_hybrid_adam = True  # the optimizer's switch (fp16_cpu_adam.py:523-528); initialize_engine sets it
         self.hbm_budget_bytes = None  # None: ask the device (torch.cuda.mem_get_info)
         self.margin_use_ratio = 0.8  # the reference's default share of the margin (memtracer.py:190-214)
-        self.staging_slots = 2
+        self.staging_slots = 3  # what the optimizer streams host-resident positions through (FP16Adam.staging_slots)
         self.placement = None  # what plan_placement decided, for inspection
         if config is not None:
             self.opt_config.update(config.get("opts", {}))

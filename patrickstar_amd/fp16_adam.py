@@ -134,7 +134,9 @@ class FP16Adam(torch.optim.Optimizer):
         # count in the loss scaler's device state (adam_step) and this is what it was seeded with.
         self._common_step = 0
         self._offsets = {}  # parameter -> its distance from the common counter (only parameters that have one)
-        self.staging_slots = 3  # HBM staging slots for host-resident chunks (one being filled, one computed on, one drained)
+        # HBM staging slots for host-resident chunks (one being filled, one computed on, one drained); the client has
+        # budgeted that many when it placed the payloads
+        self.staging_slots = getattr(client, "staging_slots", 3)
 
         assert len(self.param_groups) == 1, "Only support one param group at the moment."
         # Eager state initialisation: m and v are chunk tensors shadowing the fp16 parameter chunks.

@@ -461,7 +461,7 @@ def test_engine_places_optimizer_state_by_the_hbm_budget(arithmetic):
                                                   "use_hybrid_adam": True, "arithmetic": arithmetic}},
         "fp16": {"enabled": True, "loss_scale": 0, "initial_scale_power": 7, "loss_scale_window": 3, "hysteresis": 2, "min_loss_scale": 1},
         "default_chunk_size": 300,
-        "client": {"hbm_budget_bytes": 25000},
+        "client": {"hbm_budget_bytes": 28000},
     }
     engine, optimizer = ps.initialize_engine(model_func=_Deep, local_rank=0, config=config)
     client = engine.client
@@ -499,7 +499,7 @@ def test_engine_refuses_host_placement_without_hybrid_adam():
     config = {
         "optimizer": {"type": "Adam", "params": {"lr": 1e-3, "use_hybrid_adam": False}},
         "default_chunk_size": 300,
-        "client": {"hbm_budget_bytes": 25000},
+        "client": {"hbm_budget_bytes": 28000},
     }
     with pytest.raises(RuntimeError, match="use_hybrid_adam is False"):
         ps.initialize_engine(model_func=_Deep, local_rank=0, config=config)

@@ -575,12 +575,12 @@ def test_placement_is_decided_from_the_free_hbm_when_the_model_is_registered():
     c = client_with()
     c.plan_placement(free_bytes=6 * per / 0.8)
     assert c.host_chunk_policy is None and c.placement["host_positions"] == []
-    # 20,000 usable bytes: 6 fp16 payloads (3,600) + 2 staging slots (7,200) leave room for 2 resident states (3,600 each)
-    c = client_with(hbm_budget_bytes=25000)
+    # 22,400 usable bytes: 6 fp16 payloads (3,600) + 3 staging slots (10,800) leave room for 2 resident states (3,600 each)
+    c = client_with(hbm_budget_bytes=28000)
     c.plan_placement()
-    assert c.placement["host_positions"] == [2, 3, 4, 5] and c.placement["free_bytes"] == 25000
+    assert c.placement["host_positions"] == [2, 3, 4, 5] and c.placement["free_bytes"] == 28000
     assert [c.host_chunk_policy(i) for i in range(6)] == [False, False, True, True, True, True]
-    c = client_with(hbm_budget_bytes=25000)
+    c = client_with(hbm_budget_bytes=28000)
     c.use_hybrid_adam = False
     with pytest.raises(RuntimeError, match="use_hybrid_adam is False"):
         c.plan_placement()
