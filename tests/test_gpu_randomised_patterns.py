@@ -233,3 +233,118 @@ def test_engine_with_random_frozen_sets_and_host_placements(seed):
                     ["one tensor list" if optimizer._tensor_table else "whole chunks"])
     # the draw covers every way a step can be put together
     assert {"tensors", "stream", "staged", "one tensor list", "whole chunks"} <= seen, seen
+
+
+@pytest.mark.parametrize("seed", [6, 7, 8])
+def test_per_tensor_step_numbers_and_hyper_parameters_under_random_sequences(seed):
+    """ps_adam_step_tensors_each through the C ABI: tensors cut at random places out of two chunks (momentum and variance
+    at other element phases than the parameters in half of the cases), visited in a random order, every tensor with its
+    own step number (drawn so that "the previous call's plus one" happens often), betas / lr / eps / weight decay from
+    small pools, some tensors sitting out some steps; operator arithmetic everywhere, or the torch formula for the
+    tensors of chunk 0 and the operator for those of chunk 1; host-decided and device-decided (with poisoned steps).
+    Bar: bit-exact against the oracle, whose operator object walks through the same calls."""
+    lib = _lib.load()
+    rng = np.random.default_rng(seed)
+    for case in range(24):
+        n = int(rng.choice([700, 1500, 4099, 6000]))
+        offs = tuple(int(x) for x in rng.integers(0, 4, 4)) if rng.random() < 0.5 else (0, 0, 0, 0)
+        R = RawChunks(2, n, seed=int(rng.integers(1 << 30)), offs=offs)
+        spans = []
+        for ci in range(2):
+            cuts = sorted(set([0, n] + [int(x) for x in rng.integers(0, n + 1, int(rng.integers(1, 5)))]))
+            spans += [(ci, a, b - a) for a, b in zip(cuts[:-1], cuts[1:])]
+            if rng.random() < 0.3:
+                spans.append((ci, int(rng.integers(0, n)), 0))  # the reference calls the operator for empty tensors too
+        spans = [spans[i] for i in rng.permutation(len(spans))]
+        torch_arith = rng.random() < 0.4
+        gated = bool(rng.integers(0, 2))
+        adamw = bool(rng.integers(0, 2))
+        clip = float(rng.choice([-1, -1, 0.5]))
+        betas0 = (0.9, 0.999)
+        beta_pool = [(0.9, 0.999), (0.9, 0.999), (0.8, 0.99), (0.0, 0.9)]
+        base = int(rng.integers(0, 50))
+        oid = 9000 + case
+        _lib.check(lib.ps_adam_create(oid, 1e-3, betas0[0], betas0[1], 1e-8, 0.0, int(adamw), 0), "create")
+        if clip > 0:
+            _lib.check(lib.ps_adam_set_grad_clamp(oid, clip), "clamp")
+        if torch_arith:
+            _lib.check(lib.ps_adam_set_arithmetic(oid, _lib.PS_ARITH_TORCH), "arithmetic")
+        if gated:
+            kw = dict(init_scale=float(rng.choice([2.0**10, 1000.0])), scale_factor=2, scale_window=int(rng.integers(1, 4)), min_scale=1)
+            scaler = ps.DynamicLossScaler(**kw)
+            scaler.materialize("cuda:0", betas=betas0)
+            scaler._seed_step(base)
+            oscaler = oracle.ScalerOracle(**kw)
+        else:
+            scale = [None, 8.0, 2.0**12, 1000.0][int(rng.integers(0, 4))]
+            oscaler = oracle.StaticScalerOracle(scale) if scale else None
+        oopt = oracle.OptimizerStepOracle(R.host, oscaler, lr=1e-3, betas=betas0, eps=1e-8, weight_decay=0.0, use_adamw=adamw,
+                                          tensors=spans, gradient_clipping=clip, arithmetic="torch" if torch_arith else "operator",
+                                          operator_chunks=(1,))
+        for span in spans:
+            st = oopt.state(span)
+            st["step"] = base + int(rng.integers(0, 4))  # steps made so far: neighbours often differ by exactly one
+            st["betas"] = beta_pool[int(rng.integers(0, len(beta_pool)))]
+            st["lr"] = float(rng.choice([1e-3, 1e-3, 5e-4]))
+            st["eps"] = float(rng.choice([1e-8, 1e-8, 1e-6]))
+            st["weight_decay"] = float(rng.choice([0.0, 0.01, 0.01]))
+        device_step = base  # adam_step of the device-resident state
+        what = (f"seed {seed} case {case}: n={n} offs={offs} tensors={len(spans)} torch={torch_arith} gated={gated} adamw={adamw} "
+                f"clip={clip} base={base}")
+        workspace = torch.empty(64 * len(spans), dtype=torch.uint8, device="cuda")
+        stream = _lib.current_stream_handle()
+        for it in range(int(rng.integers(3, 6))):
+            active = [s for s in spans if rng.random() < 0.8] or spans[:1]
+            oopt.tensors = active
+            rows, numels = [], []
+            each = (_lib.ps_tensor_call * len(active))()
+            n_operator = 0
+            for k, (ci, off, numel) in enumerate(active):
+                rows.append([t[o + off:].data_ptr() for t, o in zip(R.dev[ci], R.offs)])
+                numels.append(numel)
+                st = oopt.state((ci, off, numel))
+                e = each[k]
+                e.lr, (e.beta1, e.beta2), e.eps, e.weight_decay = st["lr"], st["betas"], st["eps"], st["weight_decay"]
+                e.step = st["step"] + 1 - (device_step + 1) if gated else st["step"] + 1
+                e.arithmetic = _lib.PS_ARITH_OPERATOR if ci == 1 else -1
+                n_operator += not (torch_arith and ci == 0)
+            table, sizes = _lib.chunk_array(rows), (ctypes.c_size_t * len(numels))(*numels)
+
+            def idle_slots_hold_parameters():
+                # the slot of a tensor that sits out a step holds its fp16 parameter (nothing wrote a gradient over
+                # it), which is what the reference's whole-chunk write-back puts there again
+                for ci, off, numel in spans:
+                    if (ci, off, numel) not in active and numel:
+                        R.host[ci]["p16"][off:off + numel] = oracle.cast_fp32_to_fp16(np.ascontiguousarray(R.host[ci]["p32"][off:off + numel]))
+                        o = R.offs[3] + off
+                        R.dev[ci][3][o:o + numel].copy_(torch.from_numpy(R.host[ci]["p16"][off:off + numel]))
+
+            if gated:
+                poison = None
+                filled = [s for s in active if s[2]]
+                if rng.random() < 0.25 and filled:  # an inf in the gradient of a tensor that takes part in the step
+                    ci, off, numel = filled[int(rng.integers(0, len(filled)))]
+                    poison = (ci, off + int(rng.integers(0, numel)))
+                R.new_grads(rng, float(oscaler.loss_scale), poison=None)
+                idle_slots_hold_parameters()
+                if poison is not None:
+                    R.host[poison[0]]["p16"][poison[1]] = np.float16("inf")
+                    R.dev[poison[0]][3][R.offs[3] + poison[1]] = float("inf")
+                _lib.check(lib.ps_overflow_scan_chunks(R.table, 2, n, None, scaler.state_ptr, stream), "scan")
+                _lib.check(lib.ps_adam_step_tensors_each(oid, 1, table, sizes, each, len(active), -1.0, scaler.state_ptr,
+                                                         workspace.data_ptr(), workspace.numel(), stream), "each")
+                scaler.update_scale(None, operator_calls=n_operator)
+                oopt.check_overflow()
+                skipped = oopt.step()
+                assert skipped == (poison is not None), what
+                device_step += not skipped
+                R.compare(f"{what} iteration {it}")
+                assert scaler.loss_scale == oscaler.loss_scale and scaler.adam_step == device_step, what
+            else:
+                R.new_grads(rng, oscaler.loss_scale if oscaler else 1.0)
+                idle_slots_hold_parameters()
+                _lib.check(lib.ps_adam_step_tensors_each(oid, 1, table, sizes, each, len(active),
+                                                         float(oscaler.loss_scale) if oscaler else -1.0, None, None, 0, stream), "each")
+                oopt.step()
+                R.compare(f"{what} iteration {it}")
+        lib.ps_adam_destroy(oid)
