@@ -353,6 +353,129 @@ int main()
         PS_OK(ps_adam_destroy(34));
     }
 
+    // ---- every tensor its own step number and hyper-parameters (ps_adam_step_tensors_each): six tensors, one of
+    //      them standing three steps behind, one with another learning rate and no decay, one with other betas whose
+    //      neighbour in the call order stands exactly one step ahead of it (that call multiplies in mid-step);
+    //      host-decided first, then device-decided with a skipped step in between
+    {
+        const size_t cut = 256 * 4 + 77;
+        struct Span { int chunk; size_t off, len; };
+        const Span order[6] = {{2, cut, n - cut}, {0, 0, cut}, {0, cut, n - cut}, {1, 0, cut}, {1, cut, n - cut}, {2, 0, cut}};
+        uint64_t steps_made[6] = {20, 20, 17, 20, 20, 21};   // state[p]["step"] before the next step
+        const double lrs[6] = {1e-4, 1e-4, 1e-4, 5e-5, 1e-4, 1e-4}, wds[6] = {0.01, 0.01, 0.01, 0.0, 0.01, 0.01};
+        const double be1[6] = {0.9, 0.9, 0.9, 0.9, 0.8, 0.8}, be2[6] = {0.999, 0.999, 0.999, 0.999, 0.99, 0.99};
+        PS_OK(ps_adam_create(35, lr, b1, b2, eps, wd, 1, 0));
+        oracle_adam_init(&native, lr, b1, b2, eps, wd, 1);
+        ps_chunk rows[6];
+        size_t lens[6];
+        for (int k = 0; k < 6; ++k) {
+            const Span& t = order[k];
+            rows[k].param_fp32 = dev[t.chunk].p + t.off;
+            rows[k].exp_avg = dev[t.chunk].m + t.off;
+            rows[k].exp_avg_sq = dev[t.chunk].v + t.off;
+            rows[k].param_fp16 = dev[t.chunk].h + t.off;
+            lens[k] = t.len;
+        }
+        auto oracle_calls = [&](double loss_scale) -> int {
+            for (int k = 0; k < 6; ++k) {
+                const Span& t = order[k];
+                steps_made[k] += 1;
+                oracle_adam_advance(&native, steps_made[k], (float)be1[k], (float)be2[k]);
+                oracle_adam_set(&native, (float)lrs[k], eps, (float)wds[k], 1);
+                HostChunk& hc = host[t.chunk];
+                if (oracle_adam_span(&native, hc.p.data() + t.off, hc.h.data() + t.off, 1, hc.m.data() + t.off,
+                                     hc.v.data() + t.off, t.len, (float)loss_scale, 0) <= 0)
+                    return 5;
+            }
+            for (int c = 0; c < C; ++c) oracle_cast_f32_to_f16(host[c].p.data(), host[c].h.data(), n);
+            return 0;
+        };
+        ps_tensor_call each[6];
+        for (int it = 0; it < 2; ++it) {  // host-decided
+            for (int c = 0; c < C; ++c) {
+                new_gradients(rng, host[c], scale);
+                if (upload(host[c], dev[c], n)) return 2;
+            }
+            for (int k = 0; k < 6; ++k)
+                each[k] = ps_tensor_call{lrs[k], be1[k], be2[k], eps, wds[k], (int64_t)steps_made[k] + 1, -1, 0};
+            PS_OK(ps_adam_step_tensors_each(35, 1, rows, lens, each, 6, scale, NULL, NULL, 0, stream));
+            HIP_OK(hipStreamSynchronize(stream));
+            if (int rc = oracle_calls(scale)) return rc;
+            for (int c = 0; c < C; ++c)
+                if (int rc = compare(host[c], dev[c], n, "per-tensor step, host-decided", c)) return rc;
+        }
+        // device-decided: the device's counter stands at tensor 0's count; every tensor says how far from it it stands
+        void* d_work = nullptr;
+        const size_t work_bytes = ps_tensors_each_workspace_bytes(6);
+        HIP_OK(hipMalloc(&d_work, work_bytes));
+        PS_OK(ps_state_init(d_state, 256.0, 1, 2.0, 1, 1000, 1.0, 1, 1, 0, b1, b2, stream));
+        // the operator object goes on running (fresh_operator = 0 would need the device to hold it; this library object is
+        // the host's, so the device starts from a fresh one and so does the restatement)
+        PS_OK(ps_state_seed_step(d_state, (int64_t)steps_made[0], b1, b2, 1, stream));
+        oracle_adam_init(&native, lr, b1, b2, eps, wd, 1);
+        double dyn_scale = 256.0;
+        for (int it = 0; it < 3; ++it) {
+            const bool poison = it == 1;
+            for (int c = 0; c < C; ++c) {
+                new_gradients(rng, host[c], dyn_scale);
+                if (poison && c == 1) host[c].h[7] = 0x7E00;  // nan
+                if (upload(host[c], dev[c], n)) return 2;
+            }
+            for (int k = 0; k < 6; ++k)
+                each[k] = ps_tensor_call{lrs[k], be1[k], be2[k], eps, wds[k], (int64_t)steps_made[k] - (int64_t)steps_made[0], -1, 0};
+            PS_OK(ps_overflow_scan_chunks(table, C, n, nullptr, d_state, stream));
+            PS_OK(ps_adam_step_tensors_each(35, 1, rows, lens, each, 6, -1.0, d_state, d_work, work_bytes, stream));
+            PS_OK(ps_scaler_update(d_state, PS_FLAG_FROM_DEVICE, NULL, 0, 6, stream));
+            HIP_OK(hipStreamSynchronize(stream));
+            if (poison) {
+                for (int c = 0; c < C; ++c) oracle_cast_f32_to_f16(host[c].p.data(), host[c].h.data(), n);
+                dyn_scale /= 2.0;
+            } else if (int rc = oracle_calls(dyn_scale)) {
+                return rc;
+            }
+            for (int c = 0; c < C; ++c)
+                if (int rc = compare(host[c], dev[c], n, poison ? "per-tensor step, skipped" : "per-tensor step, device-decided", c)) return rc;
+        }
+        PS_OK(ps_state_read(d_state, &st, stream));
+        if (st.adam_step != (int64_t)steps_made[0] || st.cur_scale != dyn_scale || st.pending_operator_step != 0) {
+            fprintf(stderr, "per-tensor steps: device counter %lld (want %llu), scale %g (want %g)\n", (long long)st.adam_step,
+                    (unsigned long long)steps_made[0], st.cur_scale, dyn_scale);
+            return 6;
+        }
+        HIP_OK(hipFree(d_work));
+        PS_OK(ps_adam_destroy(35));
+    }
+
+    // ---- a chunk list whose last chunk ends in zero padding: the step leaves the padding alone, same bits
+    {
+        const size_t used_last = 256 * 6 + 9;
+        HostChunk& last = host[C - 1];
+        for (size_t i = used_last; i < n; ++i) last.p[i] = last.m[i] = last.v[i] = 0.0f, last.h[i] = 0;
+        PS_OK(ps_adam_create(36, lr, b1, b2, eps, wd, 1, 0));
+        oracle_adam_init(&native, lr, b1, b2, eps, wd, 1);
+        const size_t used[C] = {n, n, used_last};
+        for (uint64_t step = 1; step < 3; ++step) {
+            for (int c = 0; c < C; ++c) {
+                new_gradients(rng, host[c], scale);
+                if (c == C - 1)
+                    for (size_t i = used_last; i < n; ++i) host[c].h[i] = 0;
+                if (upload(host[c], dev[c], n)) return 2;
+            }
+            PS_OK(ps_adam_step_chunks(36, step, lr, b1, b2, eps, wd, 1, table, C, n, used, &calls, scale, stream));
+            HIP_OK(hipStreamSynchronize(stream));
+            for (int c = 0; c < C; ++c) {
+                oracle_adam_advance(&native, step, b1, b2);
+                oracle_adam_set(&native, lr, eps, wd, 1);
+                if (oracle_adam_span(&native, host[c].p.data(), host[c].h.data(), 1, host[c].m.data(), host[c].v.data(), n,
+                                     (float)scale, 0) <= 0)  // the restatement updates every slot, padding included
+                    return 5;
+                oracle_cast_f32_to_f16(host[c].p.data(), host[c].h.data(), n);
+                if (int rc = compare(host[c], dev[c], n, "step over a padded chunk list", c)) return rc;
+            }
+        }
+        PS_OK(ps_adam_destroy(36));
+    }
+
     // ---- the probe that allocates nothing: same answer as the probe with a caller-side state
     {
         uint32_t* d_flag = nullptr;
@@ -378,6 +501,7 @@ int main()
         HIP_OK(hipFree(d_flag));
     }
     printf("c abi gpu check ok: 3 host-decided and 8 device-decided steps (2 skipped), 3 steps with host-resident chunks, "
-           "3 tensor-list steps in two calls each, the allocation-free probe, over %d x %zu elements\n", C, n);
+           "3 tensor-list steps in two calls each, 5 steps with per-tensor step numbers and hyper-parameters, 2 over a padded list, "
+           "the allocation-free probe, over %d x %zu elements\n", C, n);
     return 0;
 }
