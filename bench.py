@@ -724,6 +724,50 @@ def tensor_list_leg(cfg, steps, warmup):
         "workload": "GPT-2 XL's 580 parameter tensors (1,557,611,200 elements), m and v packed in other orders than the parameters",
         "same_offsets": dict(measure(offs_p, offs_p), workload="the same tensors with m and v at their parameters' offsets"),
     })
+
+    # every tensor with its own numbers (ps_adam_step_tensors_each): the twelve tensors of one transformer block stand three
+    # steps behind the rest (a layer that was frozen for a while) and the two embeddings have their own learning rate
+    def measure_each(gated):
+        import patrickstar_amd as ps
+
+        rows = [[p.data_ptr() + 4 * offs_p[i], m.data_ptr() + 4 * offs_p[i], v.data_ptr() + 4 * offs_p[i], h.data_ptr() + 2 * offs_p[i]]
+                for i in range(len(sizes))]
+        table = _lib.chunk_array(rows)
+        each = (_lib.ps_tensor_call * len(sizes))()
+        behind = set(range(2 + 12 * 20, 2 + 12 * 21))
+        for i, e in enumerate(each):
+            e.lr, e.beta1, e.beta2, e.eps, e.weight_decay, e.arithmetic = HYPER["lr"] * (0.5 if i < 2 else 1.0), 0.9, 0.999, HYPER["eps"], HYPER["weight_decay"], -1
+        scaler = workspace = None
+        if gated:
+            scaler = ps.DynamicLossScaler(init_scale=2**12, scale_factor=2, scale_window=1000, min_scale=1)
+            scaler.materialize(cfg.dev, betas=HYPER["betas"])
+            scaler._seed_step(200)
+            workspace = torch.empty(lib.ps_tensors_each_workspace_bytes(len(sizes)), dtype=torch.uint8, device=cfg.dev)
+            for i, e in enumerate(each):
+                e.step = -3 if i in behind else 0
+
+        def step():
+            t[0] += 1
+            if gated:
+                _lib.check(lib.ps_adam_step_tensors_each(993, 1, table, numels, each, len(sizes), -1.0, scaler.state_ptr,
+                                                         workspace.data_ptr(), workspace.numel(), _lib.current_stream_handle()), "each")
+                scaler.update_scale(None, operator_calls=len(sizes))
+            else:
+                for i, e in enumerate(each):
+                    e.step = t[0] - (3 if i in behind else 0)
+                _lib.check(lib.ps_adam_step_tensors_each(993, 1, table, numels, each, len(sizes), 4096.0, None, None, 0,
+                                                         _lib.current_stream_handle()), "each")
+
+        ms, kernel_ms = time_steps(torch, step, steps, warmup)
+        avg = sum(kernel_ms) / len(kernel_ms)
+        return {"value": total / (ms * 1e-3), "unit": "params/s", "ms_per_step": ms, "avg_device_ms": avg,
+                "achieved_GBps": 28 * total / (avg * 1e-3) / 1e9, "frac": 28 * total / (avg * 1e-3) / 1e9 / HBM_PEAK_GBS}
+
+    out["per_tensor_numbers"] = dict(
+        measure_each(False), device_decided=measure_each(True),
+        workload="ps_adam_step_tensors_each over the same tensors at their parameters' offsets: one transformer block three steps behind "
+        "the rest, the embeddings at half the learning rate (four distinct calls); device_decided: the same through the device-resident state "
+        "(no probe in this figure)")
     lib.ps_adam_destroy(993)
     return out
 
