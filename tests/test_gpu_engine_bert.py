@@ -170,3 +170,75 @@ def test_checkpoint_reload_reproduces_the_losses_exactly():
     assert loss1 == loss3, f"Optimizer checkpoint error. {loss1} vs {loss3}"
     with pytest.raises(RuntimeError, match="strictly"):
         model.load_state_dict({"no.such.key": torch.zeros(1)}, strict=True)
+
+
+def test_a_fine_tuning_schedule_that_thaws_layers_matches_the_oracle():
+    """Only the classifier head and the last encoder layer train at first; the first encoder layer joins after three
+    steps and the embeddings after five.  The reference counts state[p]["step"] per parameter
+    (fp16_cpu_adam.py:571-574), so from then on every operator call carries its own tensor's step number: the head's
+    stand at 4, 5, 6 ..., layer 0's at 1, 2, 3 ..., the embeddings' at 1, 2.  Dynamic loss scale with a skipped step in
+    the middle; bit for bit against the oracle, which is told the same schedule."""
+    transformers = pytest.importorskip("transformers")
+    import oracle
+    from _harness import assert_bits_equal, tensor_spans
+
+    cfg = transformers.BertConfig(
+        vocab_size=256, hidden_size=64, num_hidden_layers=2, num_attention_heads=4, intermediate_size=128,
+        max_position_embeddings=64, num_labels=2, hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0,
+    )
+    torch.manual_seed(0)
+    config = {
+        "optimizer": {"type": "AdamW", "params": {"lr": 1e-3, "betas": (0.9, 0.999), "eps": 1e-8, "weight_decay": 0.01}},
+        "fp16": {"enabled": True, "loss_scale": 0, "initial_scale_power": 10, "loss_scale_window": 4, "hysteresis": 2, "min_loss_scale": 1},
+        "default_chunk_size": 32 * 1024,
+    }
+
+    def build():
+        model = transformers.BertForSequenceClassification(cfg)
+        for p in list(model.bert.embeddings.parameters()) + list(model.bert.encoder.layer[0].parameters()):
+            p.requires_grad_(False)
+        return model
+
+    engine, optimizer = ps.initialize_engine(model_func=build, local_rank=0, config=config)
+    client, module = engine.client, engine.module
+    cl, pos = client.chunk_list, client.positions()
+
+    def snap(t):
+        return t.detach().to("cpu", copy=True).numpy()
+
+    mirror = [{"p32": snap(cl[q.fp32].payload), "m": snap(cl[q.exp_avg].payload), "v": snap(cl[q.exp_avg_sq].payload),
+               "p16": snap(cl[q.fp16].payload)} for q in pos]
+    oscaler = oracle.scaler_from_config(config["fp16"])
+    oopt = oracle.OptimizerStepOracle(mirror, oscaler, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True,
+                                      tensors=tensor_spans(client, optimizer))
+    n_head = len(oopt.tensors)
+    ids = torch.randint(0, 256, (4, 32), device="cuda")
+    labels = torch.randint(0, 2, (4,), device="cuda")
+    kinds = []
+    for it in range(9):
+        if it == 3:
+            for p in module.bert.encoder.layer[0].parameters():
+                p.requires_grad_(True)
+        if it == 5:
+            for p in module.bert.embeddings.parameters():
+                p.requires_grad_(True)
+        oopt.tensors = tensor_spans(client, optimizer)
+        poison = it == 6
+        emb = module.bert.embeddings.word_embeddings.weight
+        out = engine(input_ids=ids, labels=labels)
+        loss = out.loss * (float("inf") if poison else 1.0)  # an overflowing loss: every gradient comes back inf / nan
+        engine.backward(loss)
+        for q, c in zip(pos, mirror):
+            c["p16"][...] = snap(cl[q.fp16].payload)
+        optimizer.step()
+        kinds.append(optimizer._plan["kind"])
+        oopt.check_overflow()
+        assert oopt.step() == poison
+        for i, (q, c) in enumerate(zip(pos, mirror)):
+            for key, cid in (("p32", q.fp32), ("m", q.exp_avg), ("v", q.exp_avg_sq), ("p16", q.fp16)):
+                assert_bits_equal(snap(cl[cid].payload), c[key], f"iteration {it} position {i} {key}")
+        assert optimizer.loss_scaler.loss_scale == oscaler.loss_scale
+    assert kinds == ["uniform"] * 3 + ["each"] * 6 and len(oopt.tensors) > n_head + 20
+    head = module.classifier.weight
+    layer0 = module.bert.encoder.layer[0].output.dense.weight
+    assert [optimizer.state[p]["step"] for p in (head, layer0, emb)] == [8, 5, 3]

@@ -4,6 +4,7 @@ import ctypes
 import os
 import re
 
+import numpy as np
 import pytest
 import torch
 
@@ -672,3 +673,54 @@ def test_layout_invariants_hold_for_random_models():
     ran = []
     check()
     assert len(ran) >= 20
+
+
+@pytest.mark.skipif(not os.path.exists(_lib.LIB_PATH), reason="HIP library not built")
+def test_per_parameter_step_counts_follow_the_reference_under_random_schedules():
+    """state[p]["step"] under random sequences of steps, freezing, thawing, hand-written entries and checkpoint reloads,
+    against the reference's rule written out plainly (fp16_cpu_adam.py:569-574: every step adds one to the count of every
+    parameter that is trainable at that moment).  No GPU: a host-decided step is stood in for by what it does to the
+    common counter."""
+    rng = np.random.default_rng(0)
+    for case in range(30):
+        client, model, opt = _tiny_optimizer()
+        params = list(model.parameters())
+        want = {p: 0 for p in params}
+
+        def host_decided_step():
+            if opt._plan is None or tuple(p.requires_grad for p in params) != opt._trainable_seen:
+                opt._make_plan()
+            if opt._plan["kind"] != "empty":
+                opt._common_step += 1
+                opt._steps_dirty = True
+            for p in params:
+                if p.requires_grad:
+                    want[p] += 1
+
+        for _ in range(40):
+            op = rng.integers(0, 10)
+            if op < 5:
+                host_decided_step()
+            elif op < 7:
+                params[int(rng.integers(0, len(params)))].requires_grad_(bool(rng.integers(0, 2)))
+            elif op == 7:
+                p = params[int(rng.integers(0, len(params)))]
+                value = int(rng.integers(0, 20))
+                opt.state[p]["step"] = value
+                want[p] = value
+            elif op == 8:
+                sd = opt.state_dict()
+                assert [sd["state"][i]["step"] for i in range(len(params))] == [want[p] for p in params]
+                client, model2, opt2 = _tiny_optimizer()
+                params2 = list(model2.parameters())
+                for p, q in zip(params, params2):
+                    q.requires_grad_(p.requires_grad)
+                opt2.load_state_dict(sd)
+                want = {q: want[p] for p, q in zip(params, params2)}
+                model, opt, params = model2, opt2, params2
+            else:
+                assert [opt.state[p]["step"] for p in params] == [want[p] for p in params], case
+            if opt._plan is not None and opt._plan["kind"] == "uniform":
+                trainable = [p for p in params if p.requires_grad]
+                assert len({want[p] for p in trainable}) <= 1 or tuple(p.requires_grad for p in params) != opt._trainable_seen
+        assert [opt.state[p]["step"] for p in params] == [want[p] for p in params], case
