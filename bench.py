@@ -851,6 +851,34 @@ def operator_mode(args):
     }
     out["value"] = out["update_fp16_out"]["params_per_s"]
     out["ms_per_step"] = out["update_fp16_out"]["avg_device_ms"]
+    # The reference's per-tensor loop left as it is (fp16_cpu_adam.py:336-468 calling the operator once per tensor, no fp16
+    # output, then its whole-chunk write-back): GPT-2 XL's 580 tensors over the four positions' memory, one ps_adam_update
+    # each, followed by one ps_cast_fp32_to_fp16 over the list.  Host time included: the calls are made from Python.
+    sizes = gpt2_xl_tensor_sizes()
+    if sum(sizes) <= 4 * N and N % 512 == 0:
+        first = client.positions()[0]
+        flat = [cl[c].payload.as_strided((4 * N,), (1,)) for c in (first.fp32, first.exp_avg, first.exp_avg_sq, first.fp16)]
+        offs, cur = [], 0
+        for n in sizes:
+            offs.append(cur)
+            cur += n
+        ptrs = [(flat[0].data_ptr() + 4 * o, flat[3].data_ptr() + 2 * o, flat[1].data_ptr() + 4 * o, flat[2].data_ptr() + 4 * o, n)
+                for o, n in zip(offs, sizes)]
+
+        def loop():
+            t[0] += 1
+            s = _lib.current_stream_handle()
+            for pp, gg, mm, vv, n in ptrs:
+                lib.ps_adam_update(995, t[0], HYPER["lr"], 0.9, 0.999, HYPER["eps"], HYPER["weight_decay"], 1, pp, gg, 1, mm, vv, n, 4096.0, None, s)
+            lib.ps_cast_fp32_to_fp16(flat[0].data_ptr(), flat[3].data_ptr(), cur, s)
+
+        wall_ms, ms = time_steps(torch, loop, max(5, args.steps // 2), 2)
+        avg = sum(ms) / len(ms)
+        out["per_tensor_loop_gpt2_xl"] = {
+            "what": "580 ps_adam_update calls (26 B/element) + one ps_cast_fp32_to_fp16 (6 B/element) per step, from Python",
+            "elements": cur, "ms_per_step_wall": wall_ms, "avg_device_ms": avg, "params_per_s": cur / (wall_ms * 1e-3),
+            "achieved_GBps": 32 * cur / (avg * 1e-3) / 1e9,
+        }
     lib.ps_adam_destroy(995)
     print(json.dumps(out))
 

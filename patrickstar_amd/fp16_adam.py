@@ -575,20 +575,20 @@ class FP16Adam(torch.optim.Optimizer):
                 e.arithmetic = _lib.PS_ARITH_OPERATOR if (host or self.arithmetic == "operator") else _lib.PS_ARITH_TORCH
                 operator_calls += e.arithmetic == _lib.PS_ARITH_OPERATOR
             workspace = None
+            offsets = [self._offsets.get(p, 0) for p in trainable]
             if self._dynamic:
                 nbytes = self._lib.ps_tensors_each_workspace_bytes(n)
                 workspace = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=self.client.device)
-            plan["table"] = (rows, numels, n, each, workspace, operator_calls)
+                for i, d in enumerate(offsets):
+                    each[i].step = d  # a device-decided step is told every tensor's distance from the device's counter
+            plan["table"] = (rows, numels, n, each, workspace, operator_calls, offsets)
         return plan["table"]
 
     def _step_each(self, plan, stream):
         """One step through ``ps_adam_step_tensors_each``."""
-        rows, numels, n, each, workspace, operator_calls = self._each_table(plan)
-        offsets = [self._offsets.get(p, 0) for p in plan["trainable"]]
+        rows, numels, n, each, workspace, operator_calls, offsets = self._each_table(plan)
         if self._dynamic:
             scaler = self.loss_scaler
-            for i, d in enumerate(offsets):
-                each[i].step = d  # distance from the device's counter
             _lib.check(
                 self._lib.ps_adam_step_tensors_each(
                     self.opt_id, 1, rows, numels, each, n, -1.0, scaler.state_ptr, workspace.data_ptr(),
