@@ -185,7 +185,6 @@ class FP16Adam(torch.optim.Optimizer):
         self._stages = None  # the entry-point calls of a step that cannot be made as one (see _plan_stages)
         self._trainable_seen = None  # requires_grad of every parameter when the plan was made
         self._operator_calls = 0
-        self._overflow_log_read = 0  # loss-scaler iterations whose outcome has been looked at for the overflow warning
         if self._dynamic and torch.cuda.is_available():
             self.loss_scaler.materialize(self.client.device, betas=betas)
             self.loss_scaler.enable_log(self.OVERFLOW_LOG_CAPACITY)
