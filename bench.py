@@ -727,7 +727,7 @@ def tensor_list_leg(cfg, steps, warmup):
 
     # every tensor with its own numbers (ps_adam_step_tensors_each): the twelve tensors of one transformer block stand three
     # steps behind the rest (a layer that was frozen for a while) and the two embeddings have their own learning rate
-    def measure_each(gated):
+    def measure_each(gated, lr_of=lambda i: HYPER["lr"] * (0.5 if i < 2 else 1.0)):
         import patrickstar_amd as ps
 
         rows = [[p.data_ptr() + 4 * offs_p[i], m.data_ptr() + 4 * offs_p[i], v.data_ptr() + 4 * offs_p[i], h.data_ptr() + 2 * offs_p[i]]
@@ -736,7 +736,7 @@ def tensor_list_leg(cfg, steps, warmup):
         each = (_lib.ps_tensor_call * len(sizes))()
         behind = set(range(2 + 12 * 20, 2 + 12 * 21))
         for i, e in enumerate(each):
-            e.lr, e.beta1, e.beta2, e.eps, e.weight_decay, e.arithmetic = HYPER["lr"] * (0.5 if i < 2 else 1.0), 0.9, 0.999, HYPER["eps"], HYPER["weight_decay"], -1
+            e.lr, e.beta1, e.beta2, e.eps, e.weight_decay, e.arithmetic = lr_of(i), 0.9, 0.999, HYPER["eps"], HYPER["weight_decay"], -1
         scaler = workspace = None
         if gated:
             scaler = ps.DynamicLossScaler(init_scale=2**12, scale_factor=2, scale_window=1000, min_scale=1)
@@ -768,6 +768,16 @@ def tensor_list_leg(cfg, steps, warmup):
         workload="ps_adam_step_tensors_each over the same tensors at their parameters' offsets: one transformer block three steps behind "
         "the rest, the embeddings at half the learning rate (four distinct calls); device_decided: the same through the device-resident state "
         "(no probe in this figure)")
+
+    # the number of distinct calls: a learning rate per transformer block (layer-wise decay: 50 of them, and the block that
+    # stands behind), and every tensor with a learning rate of its own
+    def block_of(i):
+        return 0 if i < 2 else (49 if i >= 2 + 12 * 48 else 1 + (i - 2) // 12)
+
+    per_block = lambda i: HYPER["lr"] * 0.95 ** (49 - block_of(i))
+    per_tensor = lambda i: HYPER["lr"] * (1.0 + 1e-3 * i)
+    out["per_tensor_numbers"]["one_lr_per_block"] = dict(measure_each(False, per_block), device_decided=measure_each(True, per_block))
+    out["per_tensor_numbers"]["every_tensor_its_own_lr"] = dict(measure_each(False, per_tensor), device_decided=measure_each(True, per_tensor))
     lib.ps_adam_destroy(993)
     return out
 

@@ -298,9 +298,10 @@ size_t ps_tensors_each_workspace_bytes(int n_tensors);
  * Adam_Optimizer::IncrementStep (cpu_adam.h:143-162) moves: a call continues the running float product beta^t
  * only if its step number is the previous call's plus one and its betas are the previous call's, and evaluates
  * (float)pow((double)beta, step) otherwise.  Calls with the torch arithmetic form 1 - beta ** step in binary64
- * from their own numbers and leave the object alone.  Tensors whose calls come out with the same constants
- * share launches (sorted by length as in ps_adam_step_tensors), so the common cases (one thawed layer, two
- * learning rates) take two or three launches more than the uniform step.
+ * from their own numbers and leave the object alone.  Launches are cut by the tensors' lengths as in
+ * ps_adam_step_tensors and take tensors of any step number and any lr / betas / eps (every tensor finds its
+ * call's constants through an index), so a list in which every tensor has numbers of its own runs like a
+ * uniform one; only the arithmetic and the weight-decay form (none, L2, decoupled) separate launches.
  *   d_state == NULL  host-decided: each[i].step is the step number; loss_scale as for ps_adam_step_chunks;
  *                    d_workspace is not used
  *   d_state != NULL  device-decided: a flagged step restores the fp16 slots from fp32; else every call's

@@ -46,6 +46,7 @@
 #include <memory>
 #include <mutex>
 #include <new>
+#include <string>
 #include <unordered_map>
 #include <vector>
 
@@ -814,6 +815,7 @@ struct TensorItem {
     int index;  // in the caller's list
     uint32_t head;
     size_t body, tiles;
+    int cls;  // the class of calls it belongs to (steps whose tensors carry their own numbers; 0 otherwise)
 };
 static_assert(kTile <= 256, "TensorBatch::numel_head keeps the head length (up to kTile - 1 elements) in 8 bits");
 
@@ -837,28 +839,52 @@ TensorItem tensor_item(const ps_chunk* tensors, const size_t* numels, int i)
     size_t head = p_addr % sizeof(float) ? 0 : (kTile - (p_addr / sizeof(float)) % kTile) % kTile;
     if (head > numels[i]) head = numels[i];
     const size_t body = numels[i] - head;
-    return TensorItem{i, (uint32_t)head, body, (head ? 1 : 0) + (body + kTile - 1) / kTile};
+    return TensorItem{i, (uint32_t)head, body, (head ? 1 : 0) + (body + kTile - 1) / kTile, 0};
 }
 
-// Calls launch(batch, grid) for groups of the given tensors (all of them non-empty): longest first; one launch
+// Calls launch(batch, grid, classes) for groups of the given tensors (all of them non-empty): longest first; one launch
 // takes tensors of nearly the same length (its grid is as wide as the longest of them: at most a tenth of a
 // launch's workgroups find nothing to do), short tensors all together.  `first_tensor`: the index (in the caller's
 // list) of the tensor that is the step's first operator call, marked in its batch; -1: none.
+//
+// `classes`: which class each tensor of the batch belongs to.  max_classes == 0: the items' own class numbers.
+// max_classes > 0: a launch takes at most that many distinct classes; classes.k[] then numbers them 0, 1, ... in the
+// order of their first tensor in the batch and classes.of[] says which of the items' classes each one is.
+struct BatchClasses {
+    ClassIndex k;
+    int of[kTensorBatch];
+    int n;
+};
+
 template <typename F>
-int for_each_tensor_batch(std::vector<TensorItem>& items, const ps_chunk* tensors, int first_tensor, F launch)
+int for_each_tensor_batch(std::vector<TensorItem>& items, const ps_chunk* tensors, int first_tensor, int max_classes,
+                          F launch)
 {
     std::stable_sort(items.begin(), items.end(), [](const TensorItem& a, const TensorItem& b) { return a.tiles > b.tiles; });
     constexpr size_t kShortTensorTiles = 256;
     TensorBatch b;
+    BatchClasses bc;
     size_t next = 0;
     while (next < items.size()) {
         memset(&b, 0, sizeof(b));
+        memset(&bc, 0, sizeof(bc));
         b.first_call = -1;
         const size_t widest = items[next].tiles;
         int in_batch = 0;
         while (next < items.size() && in_batch < kTensorBatch &&
                (items[next].tiles * 10 >= widest * 9 || widest <= kShortTensorTiles)) {
             const TensorItem& it = items[next];
+            if (max_classes > 0) {
+                int j = 0;
+                while (j < bc.n && bc.of[j] != it.cls) ++j;
+                if (j == bc.n) {
+                    if (bc.n == max_classes) break;  // the next launch starts with this tensor
+                    bc.of[bc.n++] = it.cls;
+                }
+                bc.k.k[in_batch] = (uint16_t)j;
+            } else {
+                bc.k.k[in_batch] = (uint16_t)it.cls;
+            }
             ps_chunk t = tensors[it.index];
             t.param_fp32 += it.head;
             t.exp_avg += it.head;
@@ -870,7 +896,7 @@ int for_each_tensor_batch(std::vector<TensorItem>& items, const ps_chunk* tensor
             in_batch += 1;
             next += 1;
         }
-        launch(b, dim3((unsigned)widest, (unsigned)in_batch));
+        launch(b, dim3((unsigned)widest, (unsigned)in_batch), bc);
         PS_HIP(hipGetLastError());
     }
     return 0;
@@ -885,16 +911,72 @@ int wd_mode_of(int arith, double wd, bool adamw)
 }
 
 template <int ARITH>
-void launch_tensors_planned_arith(const TensorBatch& b, dim3 grid, int wd_mode, const PlannedConsts* d_consts,
-                                  const ps_step_state* d_state, hipStream_t s)
+void launch_tensors_planned_arith(const TensorBatch& b, dim3 grid, const ClassIndex& ci, int wd_mode,
+                                  const PlannedConsts* d_consts, const ps_step_state* d_state, hipStream_t s)
 {
     dim3 block(kBlock);
     if (wd_mode == WD_DECOUPLED)
-        hipLaunchKernelGGL((adam_tensors_planned_kernel<ARITH, WD_DECOUPLED>), grid, block, kLdsBytes, s, b, d_consts, d_state);
+        hipLaunchKernelGGL((adam_tensors_planned_kernel<ARITH, WD_DECOUPLED>), grid, block, kLdsBytes, s, b, ci, d_consts, d_state);
     else if (wd_mode == WD_L2)
-        hipLaunchKernelGGL((adam_tensors_planned_kernel<ARITH, WD_L2>), grid, block, kLdsBytes, s, b, d_consts, d_state);
+        hipLaunchKernelGGL((adam_tensors_planned_kernel<ARITH, WD_L2>), grid, block, kLdsBytes, s, b, ci, d_consts, d_state);
     else
-        hipLaunchKernelGGL((adam_tensors_planned_kernel<ARITH, WD_NONE>), grid, block, kLdsBytes, s, b, d_consts, d_state);
+        hipLaunchKernelGGL((adam_tensors_planned_kernel<ARITH, WD_NONE>), grid, block, kLdsBytes, s, b, ci, d_consts, d_state);
+}
+
+// Numbers the distinct records (classes of calls) of a step by their bytes; records are zero-filled before they are
+// set, so equal records have equal bytes.  Consecutive tensors mostly repeat the previous record.
+template <typename T>
+struct ClassTable {
+    std::vector<T> records;
+    std::vector<int> arith;
+    std::unordered_map<std::string, int> by_bytes;
+    int last = -1;
+
+    int intern(const T& r, int a)
+    {
+        if (last >= 0 && arith[last] == a && memcmp(&records[last], &r, sizeof(T)) == 0) return last;
+        std::string key(reinterpret_cast<const char*>(&r), sizeof(T));
+        key.push_back((char)a);
+        auto found = by_bytes.find(key);
+        if (found == by_bytes.end()) {
+            found = by_bytes.emplace(std::move(key), (int)records.size()).first;
+            records.push_back(r);
+            arith.push_back(a);
+        }
+        return last = found->second;
+    }
+    int size() const { return (int)records.size(); }
+};
+
+// What a launch of the per-tensor-numbers step is compiled for; classes that agree in it share launches.
+struct Flavour {
+    int arith, wd_mode, unscale;
+    bool operator==(const Flavour& o) const { return arith == o.arith && wd_mode == o.wd_mode && unscale == o.unscale; }
+};
+
+template <int ARITH, int WD>
+void launch_tensors_each_wd(const TensorBatch& b, dim3 grid, const ClassIndex& ci, const ConstsBatch& cb, int unscale,
+                            hipStream_t s)
+{
+    dim3 block(kBlock);
+    if (unscale == UNSCALE_MUL)
+        hipLaunchKernelGGL((adam_tensors_each_kernel<ARITH, WD, UNSCALE_MUL>), grid, block, kLdsBytes, s, b, ci, cb);
+    else if (ARITH == PS_ARITH_OPERATOR && unscale == UNSCALE_DIV)  // the torch formula never divides
+        hipLaunchKernelGGL((adam_tensors_each_kernel<ARITH, WD, UNSCALE_DIV>), grid, block, kLdsBytes, s, b, ci, cb);
+    else
+        hipLaunchKernelGGL((adam_tensors_each_kernel<ARITH, WD, UNSCALE_NONE>), grid, block, kLdsBytes, s, b, ci, cb);
+}
+
+template <int ARITH>
+void launch_tensors_each_arith(const TensorBatch& b, dim3 grid, const ClassIndex& ci, const ConstsBatch& cb,
+                               const Flavour& f, hipStream_t s)
+{
+    if (f.wd_mode == WD_DECOUPLED)
+        launch_tensors_each_wd<ARITH, WD_DECOUPLED>(b, grid, ci, cb, f.unscale, s);
+    else if (f.wd_mode == WD_L2)
+        launch_tensors_each_wd<ARITH, WD_L2>(b, grid, ci, cb, f.unscale, s);
+    else
+        launch_tensors_each_wd<ARITH, WD_NONE>(b, grid, ci, cb, f.unscale, s);
 }
 
 }  // namespace
@@ -946,7 +1028,7 @@ int ps_adam_step_tensors(int optimizer_id, size_t step, double lr, double beta1,
     }
     for (int i = 0; i < n_tensors; ++i)
         if (numels[i] != 0) items.push_back(tensor_item(tensors, numels, i));
-    return for_each_tensor_batch(items, tensors, first_tensor, [&](const TensorBatch& b, dim3 grid) {
+    return for_each_tensor_batch(items, tensors, first_tensor, 0, [&](const TensorBatch& b, dim3 grid, const BatchClasses&) {
         if (d_state == nullptr) {
             if (arith == PS_ARITH_TORCH)
                 launch_tensors_arith<PS_ARITH_TORCH>(b, grid, c, s);
@@ -996,10 +1078,9 @@ int ps_adam_step_tensors_each(int optimizer_id, int bias_correction, const ps_ch
     try {
         // Calls that come out with the same constants form a class; class_of[i] says which one tensor i belongs to.
         std::vector<int> class_of((size_t)n_tensors, -1);
-        std::vector<int> class_arith, class_wd;
         if (d_state == nullptr) {
             // ---- host-decided: the operator object goes through the calls, in order
-            std::vector<StepConsts> consts;
+            ClassTable<StepConsts> classes;
             for (int i = 0; i < n_tensors; ++i) {
                 const ps_tensor_call& e = each[i];
                 const int arith = arith_of(i);
@@ -1010,27 +1091,37 @@ int ps_adam_step_tensors_each(int optimizer_id, int bias_correction, const ps_ch
                     c = torch_step_consts(*o, (size_t)e.step, hp);
                 else
                     c = operator_step_consts(*o, (size_t)e.step, hp, 1);
-                int k = 0;
-                for (; k < (int)consts.size(); ++k)
-                    if (class_arith[k] == arith && memcmp(&consts[k], &c, sizeof(c)) == 0) break;
-                if (k == (int)consts.size()) {
-                    consts.push_back(c);
-                    class_arith.push_back(arith);
-                    class_wd.push_back(c.wd_mode);
-                }
-                class_of[i] = k;
+                class_of[i] = classes.intern(c, arith);
+            }
+            const std::vector<StepConsts>& consts = classes.records;
+            // one pass of launches per flavour (what the kernels are compiled for); inside it, tensors of any class
+            std::vector<Flavour> flavours;
+            std::vector<int> flavour_of(consts.size());
+            for (size_t k = 0; k < consts.size(); ++k) {
+                const Flavour f{classes.arith[k], consts[k].wd_mode, consts[k].unscale};
+                size_t j = 0;
+                while (j < flavours.size() && !(flavours[j] == f)) ++j;
+                if (j == flavours.size()) flavours.push_back(f);
+                flavour_of[k] = (int)j;
             }
             std::vector<TensorItem> items;
-            for (int k = 0; k < (int)consts.size(); ++k) {
+            for (size_t j = 0; j < flavours.size(); ++j) {
                 items.clear();
                 for (int i = 0; i < n_tensors; ++i)
-                    if (class_of[i] == k && numels[i] != 0) items.push_back(tensor_item(tensors, numels, i));
-                const StepConsts& c = consts[k];
-                int rc = for_each_tensor_batch(items, tensors, -1, [&](const TensorBatch& b, dim3 grid) {
-                    if (class_arith[k] == PS_ARITH_TORCH)
-                        launch_tensors_arith<PS_ARITH_TORCH>(b, grid, c, s);
+                    if (numels[i] != 0 && flavour_of[class_of[i]] == (int)j) {
+                        items.push_back(tensor_item(tensors, numels, i));
+                        items.back().cls = class_of[i];
+                    }
+                const Flavour& f = flavours[j];
+                int rc = for_each_tensor_batch(items, tensors, -1, kLaunchClasses,
+                                               [&](const TensorBatch& b, dim3 grid, const BatchClasses& bc) {
+                    ConstsBatch cb;
+                    memset(&cb, 0, sizeof(cb));
+                    for (int q = 0; q < bc.n; ++q) cb.c[q] = consts[bc.of[q]];
+                    if (f.arith == PS_ARITH_TORCH)
+                        launch_tensors_each_arith<PS_ARITH_TORCH>(b, grid, bc.k, cb, f, s);
                     else
-                        launch_tensors_arith<PS_ARITH_OPERATOR>(b, grid, c, s);
+                        launch_tensors_each_arith<PS_ARITH_OPERATOR>(b, grid, bc.k, cb, f, s);
                 });
                 if (rc) return rc;
             }
@@ -1041,7 +1132,10 @@ int ps_adam_step_tensors_each(int optimizer_id, int bias_correction, const ps_ch
         // the device.  The host knows how the calls relate to one another (IncrementStep, cpu_adam.h:143-162, looks
         // only at differences between consecutive calls), which leaves three kinds of operator call and one
         // torch call; the device turns each distinct one into constants.
-        std::vector<PlanClass> classes;
+        ClassTable<PlanClass> table_of_classes;
+        const std::vector<PlanClass>& classes = table_of_classes.records;
+        const std::vector<int>& class_arith = table_of_classes.arith;
+        std::vector<int> class_wd;
         int prev_class = -1;  // of the previous operator call
         int last_operator = -1;
         for (int i = 0; i < n_tensors; ++i) {
@@ -1066,14 +1160,8 @@ int ps_adam_step_tensors_each(int optimizer_id, int bias_correction, const ps_ch
                     k.mode = PLAN_POW;
                 }
             }
-            int c = 0;
-            for (; c < (int)classes.size(); ++c)
-                if (class_arith[c] == arith && memcmp(&classes[c], &k, sizeof(k)) == 0) break;
-            if (c == (int)classes.size()) {
-                classes.push_back(k);
-                class_arith.push_back(arith);
-                class_wd.push_back(wd_mode_of(arith, e.weight_decay, o->adamw));
-            }
+            const int c = table_of_classes.intern(k, arith);
+            if (c == (int)class_wd.size()) class_wd.push_back(wd_mode_of(arith, e.weight_decay, o->adamw));
             class_of[i] = c;
             if (arith != PS_ARITH_TORCH) prev_class = last_operator = c;
         }
@@ -1101,18 +1189,32 @@ int ps_adam_step_tensors_each(int optimizer_id, int bias_correction, const ps_ch
             PS_HIP(hipGetLastError());
             if (n_classes == 0) break;
         }
+        // One pass of launches per (arithmetic, weight-decay form); inside it, tensors of any class.  A launch names
+        // its tensors' classes in 16 bits, relative to the window of 65536 records it is handed.
+        constexpr int kWindow = 1 << 16;
         std::vector<TensorItem> items;
-        for (int k = 0; k < n_classes; ++k) {
-            items.clear();
-            for (int i = 0; i < n_tensors; ++i)
-                if (class_of[i] == k && numels[i] != 0) items.push_back(tensor_item(tensors, numels, i));
-            int rc = for_each_tensor_batch(items, tensors, -1, [&](const TensorBatch& b, dim3 grid) {
-                if (class_arith[k] == PS_ARITH_TORCH)
-                    launch_tensors_planned_arith<PS_ARITH_TORCH>(b, grid, class_wd[k], table + k, d_state, s);
-                else
-                    launch_tensors_planned_arith<PS_ARITH_OPERATOR>(b, grid, class_wd[k], table + k, d_state, s);
-            });
-            if (rc) return rc;
+        for (int window = 0; window < n_classes; window += kWindow) {
+            for (int arith : {PS_ARITH_OPERATOR, PS_ARITH_TORCH}) {
+                for (int wd_mode : {WD_NONE, WD_L2, WD_DECOUPLED}) {
+                    items.clear();
+                    for (int i = 0; i < n_tensors; ++i) {
+                        const int k = class_of[i];
+                        if (numels[i] == 0 || k < window || k >= window + kWindow) continue;
+                        if (class_arith[k] != arith || class_wd[k] != wd_mode) continue;
+                        items.push_back(tensor_item(tensors, numels, i));
+                        items.back().cls = k - window;
+                    }
+                    if (items.empty()) continue;
+                    int rc = for_each_tensor_batch(items, tensors, -1, 0,
+                                                   [&](const TensorBatch& b, dim3 grid, const BatchClasses& bc) {
+                        if (arith == PS_ARITH_TORCH)
+                            launch_tensors_planned_arith<PS_ARITH_TORCH>(b, grid, bc.k, wd_mode, table + window, d_state, s);
+                        else
+                            launch_tensors_planned_arith<PS_ARITH_OPERATOR>(b, grid, bc.k, wd_mode, table + window, d_state, s);
+                    });
+                    if (rc) return rc;
+                }
+            }
         }
         return 0;
     } catch (const std::exception&) {  // nothing may throw across the boundary

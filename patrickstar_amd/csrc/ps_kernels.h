@@ -240,20 +240,53 @@ __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
                                                       numel, 0, first ? numel : 0);
 }
 
-// Step constants of one distinct call of a device-decided step whose tensors carry their own step numbers and
-// hyper-parameters, formed on the device by plan_consts_kernel (below) before the update kernels run.
+// A step whose tensors carry their own step numbers and hyper-parameters: calls that come out with the same constants
+// form a class.  One launch takes tensors of ANY class (the launch shape depends on the tensors' lengths only, so a
+// list in which every tensor is a class of its own runs like a list with one class); `ClassIndex` says which record
+// of the launch's constants each tensor of the batch uses.  What a launch cannot mix is what the kernels are
+// compiled for: the arithmetic, the weight-decay form and the way of unscaling.
+struct ClassIndex {
+    uint16_t k[kTensorBatch];
+};
+
+// Host-decided: the constants of up to kLaunchClasses classes travel with the launch (a launch's arguments stay
+// under 4 KiB: 2568 bytes of descriptors, 128 of class indices, 24 x 56 of constants).
+constexpr int kLaunchClasses = 24;
+struct ConstsBatch {
+    StepConsts c[kLaunchClasses];
+};
+static_assert(sizeof(TensorBatch) + sizeof(ClassIndex) + sizeof(ConstsBatch) <= 4096, "kernel arguments of one launch");
+
+// No tensor is "the first call" here: a first call that differs is a class of its own.
+template <int ARITH, int WD, int UNS>
+__global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
+    adam_tensors_each_kernel(TensorBatch b, ClassIndex ci, ConstsBatch cb)
+{
+    const int k = blockIdx.y;
+    const uint64_t nh = b.numel_head[k];
+    const size_t numel = (size_t)(nh & kNumelMask);
+    const int head = (int)(nh >> 56);
+    const ptrdiff_t tile = (ptrdiff_t)blockIdx.x - (head ? 1 : 0);
+    if (tile < 0) {
+        adam_head<ARITH, WD, UNS>(cb.c[ci.k[k]], b.t[k], head, false);
+        return;
+    }
+    const size_t base = (size_t)tile * kTile;
+    if (base >= numel) return;  // the grid is as wide as the longest tensor of the batch
+    adam_tile_late_consts<ARITH, WD, UNS>([&]() { return cb.c[ci.k[k]]; }, b.t[k], base, numel, 0, 0);
+}
+
+// Device-decided: the constants of every class are formed on the device by plan_consts_kernel (below), one record
+// per class in the caller's workspace, before the update kernels run.
 struct PlannedConsts {
     StepConsts c;
     float beta1_t, beta2_t;  // the operator object's beta^t after this call (unused by the torch formula)
 };
 static_assert(sizeof(PlannedConsts) == 64, "one 64-byte record per class in the caller's workspace");
 
-// The tensor-list step with the constants of the launch's tensors read from device memory: every tensor of the
-// launch belongs to one class of calls.  No tensor is "the first call" here: a first call that differs is a class
-// of its own.
 template <int ARITH, int WD>
 __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
-    adam_tensors_planned_kernel(TensorBatch b, const PlannedConsts* __restrict__ consts,
+    adam_tensors_planned_kernel(TensorBatch b, ClassIndex ci, const PlannedConsts* __restrict__ consts,
                                 const ps_step_state* __restrict__ st)
 {
     const int k = blockIdx.y;
@@ -273,10 +306,10 @@ __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
         return;
     }
     if (tile < 0) {
-        adam_head<ARITH, WD, UNSCALE_RUNTIME>(consts->c, b.t[k], head, false);
+        adam_head<ARITH, WD, UNSCALE_RUNTIME>(consts[ci.k[k]].c, b.t[k], head, false);
         return;
     }
-    adam_tile_late_consts<ARITH, WD, UNSCALE_RUNTIME>([&]() { return consts->c; }, b.t[k], base, numel, 0, 0);
+    adam_tile_late_consts<ARITH, WD, UNSCALE_RUNTIME>([&]() { return consts[ci.k[k]].c; }, b.t[k], base, numel, 0, 0);
 }
 
 __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
@@ -712,7 +745,7 @@ struct PlanClass {
     int32_t mode;
     int32_t prev;  // PLAN_MUL: the class (index in the table) of the call before it
 };
-constexpr int kPlanBatch = 32;
+constexpr int kPlanBatch = 64;  // one lane per class; 64 x 56 bytes of kernel arguments
 struct PlanBatch {
     PlanClass k[kPlanBatch];
 };

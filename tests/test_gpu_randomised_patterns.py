@@ -348,3 +348,77 @@ def test_per_tensor_step_numbers_and_hyper_parameters_under_random_sequences(see
                 oopt.step()
                 R.compare(f"{what} iteration {it}")
         lib.ps_adam_destroy(oid)
+
+
+@pytest.mark.parametrize("gated", [False, True])
+@pytest.mark.parametrize("torch_arith", [False, True])
+def test_more_distinct_calls_in_a_step_than_one_launch_carries(gated, torch_arith):
+    """ps_adam_step_tensors_each over 150 tensors (two of them long enough to get launches of their own) of which nearly
+    every one has its own learning rate and step number, with three weight decays (one of them zero: another kernel
+    form) and two epsilons: far more distinct calls than the constants one launch brings along, in launches that mix
+    them.  Bar: bit-exact against the oracle, three steps, host- and device-decided, both arithmetics (the tensors of
+    chunk 1 stay with the operator)."""
+    lib = _lib.load()
+    rng = np.random.default_rng(77 + 2 * gated + torch_arith)
+    n = 150000
+    R = RawChunks(2, n, seed=5, offs=(0, 0, 0, 0))
+    spans = []
+    for ci in range(2):
+        cuts = [0, 90001] + sorted(set(int(x) for x in rng.integers(90001, n, 73))) + [n]
+        spans += [(ci, a, b - a) for a, b in zip(cuts[:-1], cuts[1:]) if b > a]
+    spans = [spans[i] for i in rng.permutation(len(spans))]
+    oid = 9100 + 2 * gated + torch_arith
+    _lib.check(lib.ps_adam_create(oid, 1e-3, 0.9, 0.999, 1e-8, 0.0, 1, 0), "create")
+    if torch_arith:
+        _lib.check(lib.ps_adam_set_arithmetic(oid, _lib.PS_ARITH_TORCH), "arithmetic")
+    base = 40
+    if gated:
+        kw = dict(init_scale=2.0**10, scale_factor=2, scale_window=2, min_scale=1)
+        scaler = ps.DynamicLossScaler(**kw)
+        scaler.materialize("cuda:0", betas=(0.9, 0.999))
+        scaler._seed_step(base)
+        oscaler = oracle.ScalerOracle(**kw)
+    else:
+        oscaler = oracle.StaticScalerOracle(2.0**12)
+    oopt = oracle.OptimizerStepOracle(R.host, oscaler, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0, use_adamw=True,
+                                      tensors=spans, arithmetic="torch" if torch_arith else "operator", operator_chunks=(1,))
+    for k, span in enumerate(spans):
+        st = oopt.state(span)
+        st["step"] = base + int(rng.integers(0, 30))
+        st["lr"] = 1e-3 * (1.0 + 0.01 * k)
+        st["eps"] = float(rng.choice([1e-8, 1e-6]))
+        st["weight_decay"] = float(rng.choice([0.0, 0.01, 0.1]))
+    assert len({(oopt.state(s)["lr"], oopt.state(s)["step"]) for s in spans}) > 100
+    device_step = base
+    workspace = torch.empty(lib.ps_tensors_each_workspace_bytes(len(spans)), dtype=torch.uint8, device="cuda")
+    stream = _lib.current_stream_handle()
+    rows = [[t[o + off:].data_ptr() for t, o in zip(R.dev[ci], R.offs)] for ci, off, _ in spans]
+    table = _lib.chunk_array(rows)
+    sizes = (ctypes.c_size_t * len(spans))(*[s[2] for s in spans])
+    each = (_lib.ps_tensor_call * len(spans))()
+    for it in range(3):
+        for e, span in zip(each, spans):
+            st = oopt.state(span)
+            e.lr, (e.beta1, e.beta2), e.eps, e.weight_decay = st["lr"], st["betas"], st["eps"], st["weight_decay"]
+            e.step = st["step"] + 1 - (device_step + 1) if gated else st["step"] + 1
+            e.arithmetic = _lib.PS_ARITH_OPERATOR if span[0] == 1 else -1
+        what = f"gated={gated} torch={torch_arith} iteration {it}"
+        if gated:
+            poisoned = it == 1
+            R.new_grads(rng, float(oscaler.loss_scale), poison=(1, 12345) if poisoned else None)
+            _lib.check(lib.ps_overflow_scan_chunks(R.table, 2, n, None, scaler.state_ptr, stream), "scan")
+            _lib.check(lib.ps_adam_step_tensors_each(oid, 1, table, sizes, each, len(spans), -1.0, scaler.state_ptr,
+                                                     workspace.data_ptr(), workspace.numel(), stream), "each")
+            scaler.update_scale(None, operator_calls=sum(1 for s in spans if not (torch_arith and s[0] == 0)))
+            oopt.check_overflow()
+            assert oopt.step() == poisoned, what
+            device_step += not poisoned
+            R.compare(what)
+            assert scaler.loss_scale == oscaler.loss_scale and scaler.adam_step == device_step, what
+        else:
+            R.new_grads(rng, oscaler.loss_scale)
+            _lib.check(lib.ps_adam_step_tensors_each(oid, 1, table, sizes, each, len(spans), float(oscaler.loss_scale), None, None, 0,
+                                                     stream), "each")
+            oopt.step()
+            R.compare(what)
+    lib.ps_adam_destroy(oid)
