@@ -145,13 +145,14 @@ class DynamicLossScaler:
         at ``adam_step`` with the same betas (``cpu_adam.h:143-162``)."""
         if betas is not None:
             self._betas = (float(betas[0]), float(betas[1]))
-        _lib.check(
-            _lib.load().ps_state_seed_step(
-                self._state.data_ptr(), int(adam_step), self._betas[0], self._betas[1], int(bool(fresh_operator)),
-                _lib.current_stream_handle(),
-            ),
-            "ps_state_seed_step",
-        )
+        with torch.cuda.device(self._state.device):
+            _lib.check(
+                _lib.load().ps_state_seed_step(
+                    self._state.data_ptr(), int(adam_step), self._betas[0], self._betas[1], int(bool(fresh_operator)),
+                    _lib.current_stream_handle(),
+                ),
+                "ps_state_seed_step",
+            )
 
     def enable_log(self, capacity):
         """Record (overflow flag, scale after) of every ``update_scale`` in a device ring of ``capacity`` entries,
