@@ -69,6 +69,8 @@ class _ParamState(dict):
             owner = self._owner()
             if owner is not None:
                 owner._plan = None  # the next step() looks at every parameter's entries again
+                if key == "step":
+                    owner._steps_written = True  # ... and at how the step numbers relate to one another
 
     def items(self):
         self._sync()
@@ -134,6 +136,8 @@ class FP16Adam(torch.optim.Optimizer):
         # count in the loss scaler's device state (adam_step) and this is what it was seeded with.
         self._common_step = 0
         self._offsets = {}  # parameter -> its distance from the common counter (only parameters that have one)
+        self._steps_written = True  # some state[p]["step"] was written since the plan was last made (or none was made yet)
+        self._each_static = None  # what the tensor table of a step with per-tensor numbers keeps between plans
         # HBM staging slots for host-resident chunks (one being filled, one computed on, one drained); the client has
         # budgeted that many when it placed the payloads
         self.staging_slots = getattr(client, "staging_slots", 3)
@@ -417,6 +421,7 @@ class FP16Adam(torch.optim.Optimizer):
     def invalidate_tables(self):
         """Call after re-allocating chunk payloads."""
         self._tables = None
+        self._each_static = None
         if self._plan is not None and self._plan["kind"] == "each":
             self._plan["table"] = None
 
@@ -500,37 +505,54 @@ class FP16Adam(torch.optim.Optimizer):
 
         The reference counts ``state[p]["step"]`` per parameter and reads lr / betas / eps / weight_decay per
         parameter, on every step (``fp16_cpu_adam.py:569-606``), and hands each operator call its tensor's own
-        numbers (``:403-428``).  Ordinarily all trainable parameters agree: then ONE counter (on the host, or in the
-        device-resident state of a dynamic loss scaler) stands for all of them and the whole chunk list goes to one
-        fused call ("uniform").  If they do not (a parameter that was frozen for some steps stands behind; somebody
-        wrote ``state[p]["lr"]`` for some parameters; a checkpoint said so) the step goes tensor by tensor through
-        ``ps_adam_step_tensors_each``, every tensor with its own numbers ("each"): its step number is kept as a
-        distance from the common counter, which is all a device-decided step needs to know on the host.
-        Made again whenever ``requires_grad`` of some parameter or a ``state[p]`` entry has changed.
+        numbers (``:403-428``); ``param_groups[0]["lr"]`` is copied into ``state[p]`` once, by the constructor
+        (``:111-116``), and not looked at again, here as there.  Ordinarily all trainable parameters agree: then ONE
+        counter (on the host, or in the device-resident state of a dynamic loss scaler) stands for all of them and
+        the whole chunk list goes to one fused call ("uniform").  If they do not (a parameter that was frozen for some
+        steps stands behind; somebody wrote ``state[p]["lr"]`` for some parameters; a checkpoint said so) the step goes
+        tensor by tensor through ``ps_adam_step_tensors_each``, every tensor with its own numbers ("each"): its step
+        number is kept as a distance from the common counter, which is all a device-decided step needs to know on
+        the host.  Made again whenever ``requires_grad`` of some parameter or a ``state[p]`` entry has changed.
+
+        How the step numbers relate to one another changes only when the set of trainable parameters changes or a
+        ``state[p]["step"]`` is written; only then is the device's counter read back.  Writing hyper-parameters (a
+        learning-rate schedule writes ``state[p]["lr"]`` of every parameter before every step) keeps the distances
+        and waits for nothing.
         """
-        self._sync_steps()  # every state[p]["step"] is now what the steps so far made it
         params = self.param_groups[0]["params"]
-        self._trainable_seen = tuple(p.requires_grad for p in params)
-        self._tables = None
+        flags = tuple(p.requires_grad for p in params)
+        resettle = self._steps_written or flags != self._trainable_seen
+        if resettle:
+            self._sync_steps()  # every state[p]["step"] is now what the steps so far made it
+            self._tables = None
+            self._each_static = None
+        self._trainable_seen = flags
+        self._steps_written = False
         trainable = self._trainable()
         if not trainable:
             self._offsets = {}
             self._plan = {"kind": "empty"}
             return self._plan
-        entries = [self._entries(p) for p in trainable]
-        common = entries[0][4]
-        self._offsets = {p: e[4] - common for p, e in zip(trainable, entries) if e[4] != common}
+        common = self._common_step
+        if resettle:
+            # the common counter moves to the first trainable parameter's step number (a checkpoint was loaded, or
+            # the parameters that defined it were frozen)
+            steps = [dict.__getitem__(self.state[p], "step") for p in trainable]
+            common = steps[0]
+            self._offsets = {p: t - common for p, t in zip(trainable, steps) if t != common}
+        entries = [self._entries(p)[:4] + (self._offsets.get(p, 0),) for p in trainable]
         if all(e == entries[0] for e in entries):
             self._plan = {"kind": "uniform", "hyper": entries[0][:4]}
         else:
             self._plan = {"kind": "each", "trainable": trainable, "entries": entries, "table": None}
-        # the common counter moves to the first trainable parameter's step number (a checkpoint was loaded, or the
-        # parameters that defined it were frozen); for a device-decided step also the betas of the whole-list kernels
+        # a device-decided step keeps the counter and the betas of the whole-list kernels on the device
         betas = entries[0][1]
-        if self._dynamic:
-            if self.loss_scaler._state is not None and (
-                common != self._common_step or (float(betas[0]), float(betas[1])) != self.loss_scaler._betas
-            ):
+        if self._dynamic and self.loss_scaler._state is not None:
+            new_betas = (float(betas[0]), float(betas[1])) != self.loss_scaler._betas
+            if new_betas and not resettle:
+                self._sync_steps()  # seeding needs the counter as it stands
+                common = self._common_step
+            if new_betas or common != self._common_step:
                 # the operator object behind this optimizer stays the one it was (the reference's load_state_dict,
                 # fp16_cpu_adam.py:660-694, does not touch it): whether its running beta^t product continues is
                 # decided on the device, as Adam_Optimizer::IncrementStep would (cpu_adam.h:143-162)
@@ -560,26 +582,31 @@ class FP16Adam(torch.optim.Optimizer):
         """Tensor rows and per-tensor call records of a step whose tensors carry their own numbers."""
         if plan["table"] is None:
             trainable = plan["trainable"]
-            rows, numels, n = self._tensor_rows(trainable)
+            if self._each_static is None:
+                # addresses, lengths, where the state lives and the workspace stay as they are while the same
+                # parameters are trainable (a learning-rate schedule makes a new plan before every step)
+                rows, numels, n = self._tensor_rows(trainable)
+                on_host = {pos.fp16 for pos in self.client.positions() if pos.on_host}
+                index = self.client.chunk_tensor_index
+                host = [index.get_tensor_info(p.ps_attr.data_id()).chunk_id in on_host for p in trainable]
+                workspace = None
+                if self._dynamic:
+                    nbytes = self._lib.ps_tensors_each_workspace_bytes(n)
+                    workspace = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=self.client.device)
+                self._each_static = (rows, numels, n, host, workspace)
+            rows, numels, n, host, workspace = self._each_static
             each = (_lib.ps_tensor_call * n)()
-            on_host = {pos.fp16 for pos in self.client.positions() if pos.on_host}
-            index = self.client.chunk_tensor_index
             operator_calls = 0
-            for i, (p, (lr, (beta1, beta2), eps, weight_decay, _)) in enumerate(zip(trainable, plan["entries"])):
+            offsets = [e[4] for e in plan["entries"]]
+            for i, (lr, (beta1, beta2), eps, weight_decay, d) in enumerate(plan["entries"]):
                 e = each[i]
                 e.lr, e.beta1, e.beta2, e.eps, e.weight_decay = lr, beta1, beta2, eps, weight_decay
                 # optimizer state in host memory is updated by the operator whatever the optimizer's arithmetic
                 # (fp16_cpu_adam.py:415-443); the kernel reads and writes such pinned payloads over the link
-                host = index.get_tensor_info(p.ps_attr.data_id()).chunk_id in on_host
-                e.arithmetic = _lib.PS_ARITH_OPERATOR if (host or self.arithmetic == "operator") else _lib.PS_ARITH_TORCH
+                e.arithmetic = _lib.PS_ARITH_OPERATOR if (host[i] or self.arithmetic == "operator") else _lib.PS_ARITH_TORCH
                 operator_calls += e.arithmetic == _lib.PS_ARITH_OPERATOR
-            workspace = None
-            offsets = [self._offsets.get(p, 0) for p in trainable]
-            if self._dynamic:
-                nbytes = self._lib.ps_tensors_each_workspace_bytes(n)
-                workspace = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=self.client.device)
-                for i, d in enumerate(offsets):
-                    each[i].step = d  # a device-decided step is told every tensor's distance from the device's counter
+                if self._dynamic:
+                    e.step = d  # a device-decided step is told every tensor's distance from the device's counter
             plan["table"] = (rows, numels, n, each, workspace, operator_calls, offsets)
         return plan["table"]
 
@@ -761,6 +788,7 @@ class FP16Adam(torch.optim.Optimizer):
                 else:
                     dict.__setitem__(mine, k, saved[k])
         self._plan = None
+        self._steps_written = True
         if self._dynamic:
             self.loss_scaler.materialize(self.client.device)
             if "loss_scaler" in state_dict:

@@ -188,6 +188,56 @@ def test_hyper_parameters_written_for_some_parameters_only(loss_scale, arithmeti
     assert r.steps() == r.oracle_steps()
 
 
+@pytest.mark.parametrize("layerwise", [False, True])
+def test_a_learning_rate_schedule_waits_for_nothing(layerwise):
+    """The reference's step reads the learning rate from state[p]["lr"] (fp16_cpu_adam.py:596-601; param_groups is
+    copied once, :111-116), so a schedule writes state[p]["lr"] of every parameter before every step.  With a dynamic
+    scaler the step numbers live on the device: re-planning after such writes must not read them back (no host
+    synchronisation inside the training loop), with one rate for all parameters or one per layer, one layer standing
+    two steps behind in the second case.  Bit-exact against the oracle under the same schedule."""
+    r = _Run(0, "operator", seed=5)
+    m = r.module
+    scaler = r.opt.loss_scaler
+    watched, reads = [False], []
+    read = scaler._read
+
+    def counting_read(notify=True):
+        if watched[0]:
+            reads.append(1)
+        return read(notify)
+
+    scaler._read = counting_read
+    step = r.opt.step
+
+    def watched_step(*a, **k):
+        watched[0] = True
+        try:
+            return step(*a, **k)
+        finally:
+            watched[0] = False
+
+    r.opt.step = watched_step
+    if layerwise:
+        m.fc2.weight.requires_grad_(False)
+        r.trainable_changed()
+        r.iterate("fc2.weight sits out, step 1")
+        r.iterate("fc2.weight sits out, step 2")
+        m.fc2.weight.requires_grad_(True)
+        r.trainable_changed()
+        r.iterate("thawed: this plan reads the counter back once")
+        reads.clear()
+    decay = {id(p): (0.8 ** i if layerwise else 1.0) for i, p in enumerate(m.parameters())}
+    for k in range(1, 7):
+        watched[0] = True
+        for p in m.parameters():
+            r.set(p, "lr", 1e-3 * decay[id(p)] * min(1.0, k / 4))  # warm-up, then flat
+        watched[0] = False
+        r.iterate(f"scheduled step {k}", poison=(k == 3))
+        assert r.opt._plan["kind"] == ("each" if layerwise else "uniform")
+    assert not reads, f"{len(reads)} read-backs of the device state inside the loop"
+    assert r.steps() == r.oracle_steps()
+
+
 @pytest.mark.parametrize("arithmetic", ["operator", "torch"])
 @pytest.mark.parametrize("loss_scale", [0, 128])
 def test_betas_changed_after_construction_reach_the_step(loss_scale, arithmetic):
