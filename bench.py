@@ -232,7 +232,7 @@ def run_hybrid(args, with_cpu_baseline=True):
                                                                         "wall_over_link_duplex_floor")}
         release_memory()
     if "skipped" not in out and args.host_chunks:
-        # BASELINE's split (a third of the positions on the host) is given; this GPU's 288 GB hold the whole list, which is
+        # the split of this configuration (a third of the positions on the host) is prescribed; this GPU's 288 GB hold the whole list, which is
         # what the placement rule of the engine (PatrickStarClient.plan_placement) decides when nobody forces a policy
         try:
             out["all_resident"] = run_all_resident(args)
