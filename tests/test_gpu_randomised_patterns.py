@@ -422,3 +422,56 @@ def test_more_distinct_calls_in_a_step_than_one_launch_carries(gated, torch_arit
             oopt.step()
             R.compare(what)
     lib.ps_adam_destroy(oid)
+
+
+@pytest.mark.parametrize("gated", [False, True])
+def test_more_distinct_calls_than_sixteen_bits_number(gated):
+    """66,000 one- to three-element tensors, every one with a learning rate of its own: a launch names its tensors'
+    calls in 16 bits, so a device-decided step hands its launches windows of the table of constants, and a host-decided
+    one cuts its launches by the 24 sets of constants each brings along.  Bit-exact against the oracle, one step."""
+    lib = _lib.load()
+    rng = np.random.default_rng(91 + gated)
+    lengths = rng.integers(1, 4, 66000)
+    starts = np.concatenate([[0], np.cumsum(lengths)[:-1]])
+    n = int(lengths.sum())
+    R = RawChunks(1, n, seed=6, offs=(0, 0, 0, 0))
+    spans = [(0, int(a), int(k)) for a, k in zip(starts, lengths)]
+    oid = 9200 + gated
+    _lib.check(lib.ps_adam_create(oid, 1e-3, 0.9, 0.999, 1e-8, 0.01, 1, 0), "create")
+    base = 6
+    if gated:
+        kw = dict(init_scale=2.0**10, scale_factor=2, scale_window=1000, min_scale=1)
+        scaler = ps.DynamicLossScaler(**kw)
+        scaler.materialize("cuda:0", betas=(0.9, 0.999))
+        scaler._seed_step(base)
+        oscaler = oracle.ScalerOracle(**kw)
+    else:
+        oscaler = oracle.StaticScalerOracle(2.0**10)
+    oopt = oracle.OptimizerStepOracle(R.host, oscaler, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True,
+                                      tensors=spans)
+    each = (_lib.ps_tensor_call * len(spans))()
+    for k, (e, span) in enumerate(zip(each, spans)):
+        st = oopt.state(span)
+        st["step"] = base
+        st["lr"] = 1e-3 * (1.0 + 1e-5 * k)
+        e.lr, e.beta1, e.beta2, e.eps, e.weight_decay, e.arithmetic = st["lr"], 0.9, 0.999, 1e-8, 0.01, -1
+        e.step = 0 if gated else base + 1
+    table = _lib.chunk_array([[t[o + off:].data_ptr() for t, o in zip(R.dev[0], R.offs)] for _, off, _ in spans])
+    sizes = (ctypes.c_size_t * len(spans))(*[s[2] for s in spans])
+    stream = _lib.current_stream_handle()
+    R.new_grads(rng, float(oscaler.loss_scale))
+    if gated:
+        workspace = torch.empty(lib.ps_tensors_each_workspace_bytes(len(spans)), dtype=torch.uint8, device="cuda")
+        _lib.check(lib.ps_overflow_scan_chunks(R.table, 1, n, None, scaler.state_ptr, stream), "scan")
+        _lib.check(lib.ps_adam_step_tensors_each(oid, 1, table, sizes, each, len(spans), -1.0, scaler.state_ptr, workspace.data_ptr(),
+                                                 workspace.numel(), stream), "each")
+        scaler.update_scale(None, operator_calls=len(spans))
+        oopt.check_overflow()
+        assert oopt.step() is False
+        assert scaler.adam_step == base + 1
+    else:
+        _lib.check(lib.ps_adam_step_tensors_each(oid, 1, table, sizes, each, len(spans), float(oscaler.loss_scale), None, None, 0, stream),
+                   "each")
+        oopt.step()
+    R.compare(f"gated={gated}")
+    lib.ps_adam_destroy(oid)
