@@ -285,8 +285,16 @@ typedef struct ps_tensor_call {
                            device-decided step: its distance d from the device's counter, the tensor's step number
                            then being d_state->adam_step + 1 + d (which must come out >= 1) */
     int32_t arithmetic; /* PS_ARITH_OPERATOR, PS_ARITH_TORCH, or -1 for the optimizer's own (ps_adam_set_arithmetic) */
-    int32_t reserved;
+    int32_t flags;      /* 0, or PS_TENSOR_GRAD_F32 */
 } ps_tensor_call;
+
+/* ps_tensor_call::flags.  PS_TENSOR_GRAD_F32: a parameter that PyTorch manages itself in binary32 (the reference's
+ * TORCH_BASED parameters, i.e. embedding weights under "use_cpu_embedding": fp16_cpu_adam.py:345-353 takes their
+ * binary32 .grad and updates the parameter itself, and :459-460 writes no fp16 copy).  The tensor's descriptor then
+ * holds the address of its binary32 GRADIENT in the param_fp16 field; the gradient is only read, and a flagged
+ * device-decided step leaves the tensor alone (the reference restores nothing for it, :301-302).  The gradient clamp
+ * is applied with its binary32 bound, (float)min(65504, clipping * loss_scale). */
+#define PS_TENSOR_GRAD_F32 1
 
 /* Device memory ps_adam_step_tensors_each needs for a device-decided step over n_tensors tensors (the step
  * constants of every distinct call, formed on the device): 64 bytes per tensor at most. */

@@ -329,6 +329,15 @@ class OptimizerStepOracle:
     refreshed fp16 parameters on exit, as in the reference where backward
     overwrites the fp16 parameter slot with the gradient).
 
+    A dict with ``g32`` (float32) in place of ``p16`` stands for parameters
+    that PyTorch manages itself (``ParamType.TORCH_BASED``: the fp32 embedding
+    weights under ``use_cpu_embedding``): their ``.grad`` is float32 and is
+    handed to the operator as it is (``fp16_cpu_adam.py:345-353``; they live
+    on the CPU there, so it is always the operator, ``:415-428``), they are not
+    probed for overflow (``core/hook.py:202-203``), nothing is restored for
+    them on a skipped step (``fp16_cpu_adam.py:301-302``) and no fp16 copy is
+    written (``:459-460``).
+
     ``tensors`` lists the trainable parameters in ``param_groups`` order as
     ``(chunk index, element offset, numel)``; by default every chunk is one
     tensor, in chunk order (what a synthetic chunk list of one flat parameter
@@ -410,7 +419,7 @@ class OptimizerStepOracle:
         for c in self.chunks:
             if self.has_overflow:
                 break
-            if self.loss_scaler.has_overflow(c["p16"]):
+            if "p16" in c and self.loss_scaler.has_overflow(c["p16"]):
                 self.has_overflow = True
 
     def _clamp(self, g):
@@ -420,15 +429,18 @@ class OptimizerStepOracle:
         if self.loss_scaler is not None:
             bound = bound * self.loss_scaler.loss_scale
         bound = min(65504.0, bound)
-        b16 = np.float16(np.float32(bound))
-        g[g < -b16] = -b16
-        g[g > b16] = b16
+        # (a float32 gradient tensor takes the bound as a float: this restatement keeps the bound of the GPU branch
+        # for it too, not the CPU branch's, which multiplies its bound tensor by the loss scale in place on every call)
+        b = np.float16(np.float32(bound)) if g.dtype == np.float16 else np.float32(bound)
+        g[g < -b] = -b
+        g[g > b] = b
 
     def step(self):
         """Returns True when the step was skipped."""
         if self.has_overflow:
             for c in self.chunks:
-                c["p16"][...] = cast_fp32_to_fp16(c["p32"])
+                if "p16" in c:
+                    c["p16"][...] = cast_fp32_to_fp16(c["p32"])
             self.has_overflow = False
             self.loss_scaler.update_scale(True)
             return True
@@ -444,10 +456,11 @@ class OptimizerStepOracle:
         visited = []
         for (ci, off, numel), step, lr, (beta1, beta2), eps, weight_decay in calls:
             c = self.chunks[ci]
-            p, g, m, v = (c[k][off : off + numel] for k in ("p32", "p16", "m", "v"))
+            torch_managed = "g32" in c
+            p, g, m, v = (c[k][off : off + numel] for k in ("p32", "g32" if torch_managed else "p16", "m", "v"))
             if self.gradient_clipping > 0:
                 self._clamp(g)
-            if self.arithmetic == "torch" and ci not in self.operator_chunks:
+            if self.arithmetic == "torch" and ci not in self.operator_chunks and not torch_managed:
                 torch_formula_update(p, g, m, v, step, lr, beta1, beta2, eps, weight_decay, self.use_adamw, scaler_scale)
             else:
                 # one adam_update of the native operator: IncrementStep, update_state, Step
@@ -455,7 +468,7 @@ class OptimizerStepOracle:
                     step, lr, beta1, beta2, eps, weight_decay, True,
                     p, g, m, v, float(scaler_scale if scaler_scale is not None else -1), self.isa,
                 )
-            if ci not in visited:
+            if ci not in visited and not torch_managed:
                 visited.append(ci)
         # the gradients of a chunk have all been read by now: whole-chunk write-back, padding included
         for ci in visited:

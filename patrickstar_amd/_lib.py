@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(PKG_DIR, "libps_adam.so")
 PS_FLAG_FALSE, PS_FLAG_TRUE, PS_FLAG_FROM_DEVICE = 0, 1, 2
 PS_ERR_BAD_ARG, PS_ERR_UNKNOWN_ID, PS_ERR_NO_DEVICE = -10001, -10002, -10003
 PS_ARITH_OPERATOR, PS_ARITH_TORCH = 0, 1
+PS_TENSOR_GRAD_F32 = 1
 PS_ABI_VERSION = 5
 
 
@@ -85,7 +86,7 @@ class ps_tensor_call(ctypes.Structure):
         ("weight_decay", ctypes.c_double),
         ("step", ctypes.c_int64),
         ("arithmetic", ctypes.c_int32),
-        ("reserved", ctypes.c_int32),
+        ("flags", ctypes.c_int32),
     ]
 
 

@@ -349,6 +349,7 @@ struct HyperParams {
     double lr, beta1, beta2, eps, wd;
     double loss_scale;  // <= 0: no loss scaler
     bool bias_correction;
+    bool grad_f32 = false;  // the call's gradient tensor is binary32 (the clamp bound then narrows to float only)
 };
 
 // Host-decided step, operator arithmetic: narrow like the pybind signature of adam_update
@@ -363,7 +364,7 @@ StepConsts operator_step_consts(HostAdam& o, size_t step, const HyperParams& hp,
     o.set((float)hp.lr, (float)hp.eps, (float)hp.wd);
     StepConsts c;
     finish_consts(c, o.alpha, o.beta1, o.beta2, o.eps, o.weight_decay, o.adamw, o.beta1_t,
-                  o.beta2_t, hp.bias_correction, (float)hp.loss_scale, clamp_bound(o.grad_clamp, hp.loss_scale));
+                  o.beta2_t, hp.bias_correction, (float)hp.loss_scale, clamp_bound(o.grad_clamp, hp.loss_scale, hp.grad_f32));
     bias_scalars(o.alpha, first_b1t, first_b2t, hp.bias_correction, &c.first_step_size, &c.first_bc2inv);
     return c;
 }
@@ -379,7 +380,7 @@ StepConsts torch_step_consts(const HostAdam& o, size_t step, const HyperParams& 
     }
     StepConsts c;
     torch_consts(c, hp.lr, hp.beta1, hp.beta2, hp.eps, hp.wd, o.adamw, bc1, bc2, hp.loss_scale,
-                 clamp_bound(o.grad_clamp, hp.loss_scale));
+                 clamp_bound(o.grad_clamp, hp.loss_scale, hp.grad_f32));
     return c;
 }
 
@@ -833,10 +834,10 @@ int check_tensor_list(const ps_chunk* tensors, const size_t* numels, int n_tenso
     return 0;
 }
 
-TensorItem tensor_item(const ps_chunk* tensors, const size_t* numels, int i)
+TensorItem tensor_item(const ps_chunk* tensors, const size_t* numels, int i, bool from_first_element = false)
 {
     const uintptr_t p_addr = reinterpret_cast<uintptr_t>(tensors[i].param_fp32);
-    size_t head = p_addr % sizeof(float) ? 0 : (kTile - (p_addr / sizeof(float)) % kTile) % kTile;
+    size_t head = p_addr % sizeof(float) || from_first_element ? 0 : (kTile - (p_addr / sizeof(float)) % kTile) % kTile;
     if (head > numels[i]) head = numels[i];
     const size_t body = numels[i] - head;
     return TensorItem{i, (uint32_t)head, body, (head ? 1 : 0) + (body + kTile - 1) / kTile, 0};
@@ -910,17 +911,27 @@ int wd_mode_of(int arith, double wd, bool adamw)
     return decay ? (adamw ? WD_DECOUPLED : WD_L2) : WD_NONE;
 }
 
-template <int ARITH>
-void launch_tensors_planned_arith(const TensorBatch& b, dim3 grid, const ClassIndex& ci, int wd_mode,
-                                  const PlannedConsts* d_consts, const ps_step_state* d_state, hipStream_t s)
+template <int ARITH, int WD>
+void launch_tensors_planned_wd(const TensorBatch& b, dim3 grid, const ClassIndex& ci, bool grad_f32,
+                               const PlannedConsts* d_consts, const ps_step_state* d_state, hipStream_t s)
 {
     dim3 block(kBlock);
-    if (wd_mode == WD_DECOUPLED)
-        hipLaunchKernelGGL((adam_tensors_planned_kernel<ARITH, WD_DECOUPLED>), grid, block, kLdsBytes, s, b, ci, d_consts, d_state);
-    else if (wd_mode == WD_L2)
-        hipLaunchKernelGGL((adam_tensors_planned_kernel<ARITH, WD_L2>), grid, block, kLdsBytes, s, b, ci, d_consts, d_state);
+    if (grad_f32)
+        hipLaunchKernelGGL((adam_tensors_planned_f32grad_kernel<ARITH, WD>), grid, block, kLdsBytes, s, b, ci, d_consts, d_state);
     else
-        hipLaunchKernelGGL((adam_tensors_planned_kernel<ARITH, WD_NONE>), grid, block, kLdsBytes, s, b, ci, d_consts, d_state);
+        hipLaunchKernelGGL((adam_tensors_planned_kernel<ARITH, WD>), grid, block, kLdsBytes, s, b, ci, d_consts, d_state);
+}
+
+template <int ARITH>
+void launch_tensors_planned_arith(const TensorBatch& b, dim3 grid, const ClassIndex& ci, int wd_mode, bool grad_f32,
+                                  const PlannedConsts* d_consts, const ps_step_state* d_state, hipStream_t s)
+{
+    if (wd_mode == WD_DECOUPLED)
+        launch_tensors_planned_wd<ARITH, WD_DECOUPLED>(b, grid, ci, grad_f32, d_consts, d_state, s);
+    else if (wd_mode == WD_L2)
+        launch_tensors_planned_wd<ARITH, WD_L2>(b, grid, ci, grad_f32, d_consts, d_state, s);
+    else
+        launch_tensors_planned_wd<ARITH, WD_NONE>(b, grid, ci, grad_f32, d_consts, d_state, s);
 }
 
 // Numbers the distinct records (classes of calls) of a step by their bytes; records are zero-filled before they are
@@ -951,20 +962,40 @@ struct ClassTable {
 // What a launch of the per-tensor-numbers step is compiled for; classes that agree in it share launches.
 struct Flavour {
     int arith, wd_mode, unscale;
-    bool operator==(const Flavour& o) const { return arith == o.arith && wd_mode == o.wd_mode && unscale == o.unscale; }
+    bool grad_f32;  // PS_TENSOR_GRAD_F32 tensors: binary32 gradients, no fp16 copy
+    bool operator==(const Flavour& o) const
+    {
+        return arith == o.arith && wd_mode == o.wd_mode && unscale == o.unscale && grad_f32 == o.grad_f32;
+    }
 };
 
-template <int ARITH, int WD>
-void launch_tensors_each_wd(const TensorBatch& b, dim3 grid, const ClassIndex& ci, const ConstsBatch& cb, int unscale,
-                            hipStream_t s)
+// What ClassTable keeps beside a record: the arithmetic, and whether the tensors' gradients are binary32.
+int class_key(int arith, bool grad_f32) { return arith | (grad_f32 ? 2 : 0); }
+int key_arith(int key) { return key & 1; }
+bool key_grad_f32(int key) { return (key & 2) != 0; }
+static_assert(PS_ARITH_OPERATOR == 0 && PS_ARITH_TORCH == 1, "class_key keeps the arithmetic in one bit");
+
+template <int ARITH, int WD, int UNS>
+void launch_tensors_each_uns(const TensorBatch& b, dim3 grid, const ClassIndex& ci, const ConstsBatch& cb, bool grad_f32,
+                             hipStream_t s)
 {
     dim3 block(kBlock);
-    if (unscale == UNSCALE_MUL)
-        hipLaunchKernelGGL((adam_tensors_each_kernel<ARITH, WD, UNSCALE_MUL>), grid, block, kLdsBytes, s, b, ci, cb);
-    else if (ARITH == PS_ARITH_OPERATOR && unscale == UNSCALE_DIV)  // the torch formula never divides
-        hipLaunchKernelGGL((adam_tensors_each_kernel<ARITH, WD, UNSCALE_DIV>), grid, block, kLdsBytes, s, b, ci, cb);
+    if (grad_f32)
+        hipLaunchKernelGGL((adam_tensors_each_f32grad_kernel<ARITH, WD, UNS>), grid, block, kLdsBytes, s, b, ci, cb);
     else
-        hipLaunchKernelGGL((adam_tensors_each_kernel<ARITH, WD, UNSCALE_NONE>), grid, block, kLdsBytes, s, b, ci, cb);
+        hipLaunchKernelGGL((adam_tensors_each_kernel<ARITH, WD, UNS>), grid, block, kLdsBytes, s, b, ci, cb);
+}
+
+template <int ARITH, int WD>
+void launch_tensors_each_wd(const TensorBatch& b, dim3 grid, const ClassIndex& ci, const ConstsBatch& cb,
+                            const Flavour& f, hipStream_t s)
+{
+    if (f.unscale == UNSCALE_MUL)
+        launch_tensors_each_uns<ARITH, WD, UNSCALE_MUL>(b, grid, ci, cb, f.grad_f32, s);
+    else if (ARITH == PS_ARITH_OPERATOR && f.unscale == UNSCALE_DIV)  // the torch formula never divides
+        launch_tensors_each_uns<ARITH, WD, UNSCALE_DIV>(b, grid, ci, cb, f.grad_f32, s);
+    else
+        launch_tensors_each_uns<ARITH, WD, UNSCALE_NONE>(b, grid, ci, cb, f.grad_f32, s);
 }
 
 template <int ARITH>
@@ -972,11 +1003,11 @@ void launch_tensors_each_arith(const TensorBatch& b, dim3 grid, const ClassIndex
                                const Flavour& f, hipStream_t s)
 {
     if (f.wd_mode == WD_DECOUPLED)
-        launch_tensors_each_wd<ARITH, WD_DECOUPLED>(b, grid, ci, cb, f.unscale, s);
+        launch_tensors_each_wd<ARITH, WD_DECOUPLED>(b, grid, ci, cb, f, s);
     else if (f.wd_mode == WD_L2)
-        launch_tensors_each_wd<ARITH, WD_L2>(b, grid, ci, cb, f.unscale, s);
+        launch_tensors_each_wd<ARITH, WD_L2>(b, grid, ci, cb, f, s);
     else
-        launch_tensors_each_wd<ARITH, WD_NONE>(b, grid, ci, cb, f.unscale, s);
+        launch_tensors_each_wd<ARITH, WD_NONE>(b, grid, ci, cb, f, s);
 }
 
 }  // namespace
@@ -1064,6 +1095,7 @@ int ps_adam_step_tensors_each(int optimizer_id, int bias_correction, const ps_ch
         if (d_state == nullptr && each[i].step < 1)
             return fail(PS_ERR_BAD_ARG, "each[%d].step = %lld: a host-decided step number is at least 1", i,
                         (long long)each[i].step);
+        if (each[i].flags & ~PS_TENSOR_GRAD_F32) return fail(PS_ERR_BAD_ARG, "each[%d].flags = %d", i, each[i].flags);
     }
     if (d_state != nullptr && n_tensors > 0) {
         if (!d_workspace || workspace_bytes < ps_tensors_each_workspace_bytes(n_tensors))
@@ -1075,6 +1107,7 @@ int ps_adam_step_tensors_each(int optimizer_id, int bias_correction, const ps_ch
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool bias = bias_correction != 0;
     auto arith_of = [&](int i) { return each[i].arithmetic < 0 ? o->arith : each[i].arithmetic; };
+    auto grad_f32_of = [&](int i) { return (each[i].flags & PS_TENSOR_GRAD_F32) != 0; };
     try {
         // Calls that come out with the same constants form a class; class_of[i] says which one tensor i belongs to.
         std::vector<int> class_of((size_t)n_tensors, -1);
@@ -1084,21 +1117,21 @@ int ps_adam_step_tensors_each(int optimizer_id, int bias_correction, const ps_ch
             for (int i = 0; i < n_tensors; ++i) {
                 const ps_tensor_call& e = each[i];
                 const int arith = arith_of(i);
-                const HyperParams hp{e.lr, e.beta1, e.beta2, e.eps, e.weight_decay, loss_scale, bias};
+                const HyperParams hp{e.lr, e.beta1, e.beta2, e.eps, e.weight_decay, loss_scale, bias, grad_f32_of(i)};
                 StepConsts c;
                 memset(&c, 0, sizeof(c));
                 if (arith == PS_ARITH_TORCH)
                     c = torch_step_consts(*o, (size_t)e.step, hp);
                 else
                     c = operator_step_consts(*o, (size_t)e.step, hp, 1);
-                class_of[i] = classes.intern(c, arith);
+                class_of[i] = classes.intern(c, class_key(arith, grad_f32_of(i)));
             }
             const std::vector<StepConsts>& consts = classes.records;
             // one pass of launches per flavour (what the kernels are compiled for); inside it, tensors of any class
             std::vector<Flavour> flavours;
             std::vector<int> flavour_of(consts.size());
             for (size_t k = 0; k < consts.size(); ++k) {
-                const Flavour f{classes.arith[k], consts[k].wd_mode, consts[k].unscale};
+                const Flavour f{key_arith(classes.arith[k]), consts[k].wd_mode, consts[k].unscale, key_grad_f32(classes.arith[k])};
                 size_t j = 0;
                 while (j < flavours.size() && !(flavours[j] == f)) ++j;
                 if (j == flavours.size()) flavours.push_back(f);
@@ -1109,7 +1142,7 @@ int ps_adam_step_tensors_each(int optimizer_id, int bias_correction, const ps_ch
                 items.clear();
                 for (int i = 0; i < n_tensors; ++i)
                     if (numels[i] != 0 && flavour_of[class_of[i]] == (int)j) {
-                        items.push_back(tensor_item(tensors, numels, i));
+                        items.push_back(tensor_item(tensors, numels, i, flavours[j].grad_f32));
                         items.back().cls = class_of[i];
                     }
                 const Flavour& f = flavours[j];
@@ -1134,7 +1167,7 @@ int ps_adam_step_tensors_each(int optimizer_id, int bias_correction, const ps_ch
         // torch call; the device turns each distinct one into constants.
         ClassTable<PlanClass> table_of_classes;
         const std::vector<PlanClass>& classes = table_of_classes.records;
-        const std::vector<int>& class_arith = table_of_classes.arith;
+        const std::vector<int>& class_keys = table_of_classes.arith;  // class_key(arithmetic, binary32 gradients)
         std::vector<int> class_wd;
         int prev_class = -1;  // of the previous operator call
         int last_operator = -1;
@@ -1160,7 +1193,8 @@ int ps_adam_step_tensors_each(int optimizer_id, int bias_correction, const ps_ch
                     k.mode = PLAN_POW;
                 }
             }
-            const int c = table_of_classes.intern(k, arith);
+            if (grad_f32_of(i)) k.mode |= PLAN_GRAD_F32;
+            const int c = table_of_classes.intern(k, class_key(arith, grad_f32_of(i)));
             if (c == (int)class_wd.size()) class_wd.push_back(wd_mode_of(arith, e.weight_decay, o->adamw));
             class_of[i] = c;
             if (arith != PS_ARITH_TORCH) prev_class = last_operator = c;
@@ -1194,23 +1228,25 @@ int ps_adam_step_tensors_each(int optimizer_id, int bias_correction, const ps_ch
         constexpr int kWindow = 1 << 16;
         std::vector<TensorItem> items;
         for (int window = 0; window < n_classes; window += kWindow) {
-            for (int arith : {PS_ARITH_OPERATOR, PS_ARITH_TORCH}) {
+            for (int key : {class_key(PS_ARITH_OPERATOR, false), class_key(PS_ARITH_TORCH, false),
+                            class_key(PS_ARITH_OPERATOR, true), class_key(PS_ARITH_TORCH, true)}) {
+                const bool grad_f32 = key_grad_f32(key);
                 for (int wd_mode : {WD_NONE, WD_L2, WD_DECOUPLED}) {
                     items.clear();
                     for (int i = 0; i < n_tensors; ++i) {
                         const int k = class_of[i];
                         if (numels[i] == 0 || k < window || k >= window + kWindow) continue;
-                        if (class_arith[k] != arith || class_wd[k] != wd_mode) continue;
-                        items.push_back(tensor_item(tensors, numels, i));
+                        if (class_keys[k] != key || class_wd[k] != wd_mode) continue;
+                        items.push_back(tensor_item(tensors, numels, i, grad_f32));
                         items.back().cls = k - window;
                     }
                     if (items.empty()) continue;
                     int rc = for_each_tensor_batch(items, tensors, -1, 0,
                                                    [&](const TensorBatch& b, dim3 grid, const BatchClasses& bc) {
-                        if (arith == PS_ARITH_TORCH)
-                            launch_tensors_planned_arith<PS_ARITH_TORCH>(b, grid, bc.k, wd_mode, table + window, d_state, s);
+                        if (key_arith(key) == PS_ARITH_TORCH)
+                            launch_tensors_planned_arith<PS_ARITH_TORCH>(b, grid, bc.k, wd_mode, grad_f32, table + window, d_state, s);
                         else
-                            launch_tensors_planned_arith<PS_ARITH_OPERATOR>(b, grid, bc.k, wd_mode, table + window, d_state, s);
+                            launch_tensors_planned_arith<PS_ARITH_OPERATOR>(b, grid, bc.k, wd_mode, grad_f32, table + window, d_state, s);
                     });
                     if (rc) return rc;
                 }

@@ -63,13 +63,14 @@ __host__ __device__ inline float round_to_half_precision(float f)
 // The bound of the reference's element-wise "gradient clipping" (fp16_cpu_adam.py:364-379, GPU
 // branch): min(65504, clipping * loss_scale) as a Python float, handed to Tensor.clamp_ on an fp16
 // tensor, i.e. narrowed double -> float -> half.  0 when clipping is off.
-__host__ __device__ inline float clamp_bound(double clipping, double loss_scale)
+// For a binary32 gradient tensor (grad_f32) the bound narrows to float only.
+__host__ __device__ inline float clamp_bound(double clipping, double loss_scale, bool grad_f32 = false)
 {
     if (!(clipping > 0.0)) return 0.0f;
     double c = clipping;
     if (loss_scale > 0.0) c = c * loss_scale;
     if (65504.0 < c) c = 65504.0;
-    return round_to_half_precision((float)c);
+    return grad_f32 ? (float)c : round_to_half_precision((float)c);
 }
 
 // A power-of-two scale 2^k with 2^-k a normal float: g/scale == g*(1/scale)

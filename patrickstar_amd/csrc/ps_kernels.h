@@ -276,6 +276,21 @@ __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
     adam_tile_late_consts<ARITH, WD, UNS>([&]() { return cb.c[ci.k[k]]; }, b.t[k], base, numel, 0, 0);
 }
 
+// The same for tensors whose gradient is binary32 and which have no binary16 copy (PS_TENSOR_GRAD_F32): the
+// descriptor's param_fp16 field holds the gradient's address.  Their tile grid starts at the tensor's first element.
+template <int ARITH, int WD, int UNS>
+__global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
+    adam_tensors_each_f32grad_kernel(TensorBatch b, ClassIndex ci, ConstsBatch cb)
+{
+    const int k = blockIdx.y;
+    const size_t numel = (size_t)(b.numel_head[k] & kNumelMask);
+    const size_t base = (size_t)blockIdx.x * kTile;
+    if (base >= numel) return;
+    const ps_chunk& t = b.t[k];
+    adam_tile_f32grad<ARITH, WD, UNS>([&]() { return cb.c[ci.k[k]]; }, t.param_fp32, t.exp_avg, t.exp_avg_sq,
+                                      reinterpret_cast<const float*>(t.param_fp16), base, numel);
+}
+
 // Device-decided: the constants of every class are formed on the device by plan_consts_kernel (below), one record
 // per class in the caller's workspace, before the update kernels run.
 struct PlannedConsts {
@@ -310,6 +325,22 @@ __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
         return;
     }
     adam_tile_late_consts<ARITH, WD, UNSCALE_RUNTIME>([&]() { return consts[ci.k[k]].c; }, b.t[k], base, numel, 0, 0);
+}
+
+// PS_TENSOR_GRAD_F32 tensors of a device-decided step: a flagged step leaves them alone (there is no fp16 copy to
+// restore).
+template <int ARITH, int WD>
+__global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
+    adam_tensors_planned_f32grad_kernel(TensorBatch b, ClassIndex ci, const PlannedConsts* __restrict__ consts,
+                                        const ps_step_state* __restrict__ st)
+{
+    const int k = blockIdx.y;
+    const size_t numel = (size_t)(b.numel_head[k] & kNumelMask);
+    const size_t base = (size_t)blockIdx.x * kTile;
+    if (base >= numel || st->overflow) return;
+    const ps_chunk& t = b.t[k];
+    adam_tile_f32grad<ARITH, WD, UNSCALE_RUNTIME>([&]() { return consts[ci.k[k]].c; }, t.param_fp32, t.exp_avg, t.exp_avg_sq,
+                                                  reinterpret_cast<const float*>(t.param_fp16), base, numel);
 }
 
 __global__ void __launch_bounds__(kBlock) PS_OCCUPANCY
@@ -739,10 +770,12 @@ __device__ inline double pow_int(double base, int64_t n)
 //   PLAN_POW    anything else: (float)pow((double)beta, step)
 //   PLAN_TORCH  the torch formula: 1 - beta ** step in binary64, no operator call
 enum { PLAN_POW = 0, PLAN_FIRST = 1, PLAN_MUL = 2, PLAN_TORCH = 3 };
+constexpr int32_t PLAN_KIND_MASK = 0xFF;
+constexpr int32_t PLAN_GRAD_F32 = 0x100;  // or-ed into PlanClass::mode: the tensors' gradients are binary32 (the clamp bound differs)
 struct PlanClass {
     double lr, beta1, beta2, eps, wd;
     int64_t d;     // the call's step number is adam_step + 1 + d
-    int32_t mode;
+    int32_t mode;  // one of the kinds above, plus PLAN_GRAD_F32
     int32_t prev;  // PLAN_MUL: the class (index in the table) of the call before it
 };
 constexpr int kPlanBatch = 64;  // one lane per class; 64 x 56 bytes of kernel arguments
@@ -766,19 +799,20 @@ __global__ void __launch_bounds__(64)
     const int j = threadIdx.x;
     const int64_t adam_step = st->adam_step;
     const double cur_scale = st->cur_scale;
-    const float clip = clamp_bound(a.grad_clamp, cur_scale);
     const bool bias = a.bias_correction != 0;
-    if (j < a.n && pb.k[j].mode != PLAN_MUL) {
+    if (j < a.n && (pb.k[j].mode & PLAN_KIND_MASK) != PLAN_MUL) {
         const PlanClass& k = pb.k[j];
+        const int kind = k.mode & PLAN_KIND_MASK;
+        const float clip = clamp_bound(a.grad_clamp, cur_scale, (k.mode & PLAN_GRAD_F32) != 0);
         const int64_t t = adam_step + 1 + k.d;
         PlannedConsts out;
-        if (k.mode == PLAN_TORCH) {
+        if (kind == PLAN_TORCH) {
             torch_consts(out.c, k.lr, k.beta1, k.beta2, k.eps, k.wd, a.adamw != 0, bias ? 1.0 - pow_int(k.beta1, t) : 1.0,
                          bias ? 1.0 - pow_int(k.beta2, t) : 1.0, cur_scale, clip);
             out.beta1_t = out.beta2_t = 0.0f;
         } else {
             const float b1 = (float)k.beta1, b2 = (float)k.beta2;
-            const bool follows = k.mode == PLAN_FIRST && st->operator_beta1 == b1 && st->operator_beta2 == b2 &&
+            const bool follows = kind == PLAN_FIRST && st->operator_beta1 == b1 && st->operator_beta2 == b2 &&
                                  st->operator_step + 1 == t;
             out.beta1_t = follows ? st->beta1_t_cur * b1 : (float)pow_int((double)b1, t);
             out.beta2_t = follows ? st->beta2_t_cur * b2 : (float)pow_int((double)b2, t);
@@ -794,7 +828,8 @@ __global__ void __launch_bounds__(64)
     // a call that multiplies needs the call before it: in order, by one lane
     for (int i = 0; i < a.n; ++i) {
         const PlanClass& k = pb.k[i];
-        if (k.mode != PLAN_MUL) continue;
+        if ((k.mode & PLAN_KIND_MASK) != PLAN_MUL) continue;
+        const float clip = clamp_bound(a.grad_clamp, cur_scale, (k.mode & PLAN_GRAD_F32) != 0);
         const int q = k.prev - a.first_class;  // an earlier class: of this launch, or of a launch before it
         const float p1 = q >= 0 ? b1t_of[q] : table[k.prev].beta1_t;
         const float p2 = q >= 0 ? b2t_of[q] : table[k.prev].beta2_t;

@@ -323,6 +323,61 @@ __device__ __forceinline__ void adam_tile(const StepConsts& c, const ps_chunk& c
     }
 }
 
+// One tile of a tensor whose gradient is binary32 and which has no binary16 copy (a parameter that PyTorch manages
+// itself, fp16_cpu_adam.py:345-353,459-460): `g32` is only read.  Whole tiles with all four addresses 16-byte
+// aligned take one 16-byte access per lane and array, everything else goes element by element.  As in
+// adam_tile_late_consts the constants are formed after the loads have been issued.
+template <int ARITH, int WD, int UNS, typename MakeConsts>
+__device__ __forceinline__ void adam_tile_f32grad(MakeConsts make_consts, float* __restrict__ p32, float* __restrict__ m32,
+                                                  float* __restrict__ v32, const float* __restrict__ g32, size_t base,
+                                                  size_t numel)
+{
+    const size_t end = base + kTile;
+    if (end <= numel && aligned16(p32, m32, v32, g32)) {
+        float4v g[kUnroll][kQuads], p[kUnroll][kQuads], m[kUnroll][kQuads], v[kUnroll][kQuads];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const size_t i = base + ((size_t)u * kBlock + threadIdx.x) * kLaneElems;
+#pragma unroll
+            for (int q = 0; q < kQuads; ++q) {
+                g[u][q] = ld_f4(g32 + i + 4 * q);
+                p[u][q] = ld_f4(p32 + i + 4 * q);
+                m[u][q] = ld_f4(m32 + i + 4 * q);
+                v[u][q] = ld_f4(v32 + i + 4 * q);
+            }
+        }
+        const StepConsts c = make_consts();
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const size_t i = base + ((size_t)u * kBlock + threadIdx.x) * kLaneElems;
+#pragma unroll
+            for (int q = 0; q < kQuads; ++q) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float pe = p[u][q][e], me = m[u][q][e], ve = v[u][q][e];
+                    element_any<ARITH, WD, UNS>(c, c.step_size, c.bc2inv, g[u][q][e], pe, me, ve);
+                    p[u][q][e] = pe;
+                    m[u][q][e] = me;
+                    v[u][q][e] = ve;
+                }
+                st_f4(p32 + i + 4 * q, p[u][q]);
+                st_f4(m32 + i + 4 * q, m[u][q]);
+                st_f4(v32 + i + 4 * q, v[u][q]);
+            }
+        }
+    } else {
+        const StepConsts c = make_consts();
+        const size_t last = end < numel ? end : numel;
+        for (size_t i = base + threadIdx.x; i < last; i += kBlock) {
+            float p = p32[i], m = m32[i], v = v32[i];
+            element_any<ARITH, WD, UNS>(c, c.step_size, c.bc2inv, g32[i], p, m, v);
+            p32[i] = p;
+            m32[i] = m;
+            v32[i] = v;
+        }
+    }
+}
+
 // fp16 <- RNE(fp32) for one tile (the restore of a skipped step and the
 // stand-alone write-back).
 __device__ __forceinline__ void restore_tile(const float* __restrict__ p32,

@@ -475,3 +475,123 @@ def test_more_distinct_calls_than_sixteen_bits_number(gated):
         oopt.step()
     R.compare(f"gated={gated}")
     lib.ps_adam_destroy(oid)
+
+
+class _TorchManaged:
+    """fp32 tensors that PyTorch manages itself (the reference's TORCH_BASED parameters): fp32 parameter, momentum,
+    variance and a fp32 gradient, on the device (element offset `skew` into their buffers) and mirrored as an
+    oracle chunk without a `p16` entry."""
+
+    def __init__(self, n, seed, skew=0):
+        rng = np.random.default_rng(seed)
+        self.n, self.skew = n, skew
+        self.host = {"p32": rng.normal(0, 0.02, n).astype(np.float32), "m": rng.normal(0, 1e-4, n).astype(np.float32),
+                     "v": np.abs(rng.normal(0, 1e-6, n)).astype(np.float32), "g32": np.zeros(n, np.float32)}
+        self.dev = {}
+        for key, arr in self.host.items():
+            self.dev[key] = torch.zeros(n + 8, dtype=torch.float, device="cuda")
+            self.dev[key][skew:skew + n].copy_(torch.from_numpy(arr))
+
+    def row(self, off):
+        return [self.dev[key][self.skew + off:].data_ptr() for key in ("p32", "m", "v", "g32")]
+
+    def new_grads(self, rng, scale):
+        self.host["g32"][...] = (rng.normal(0, 1e-3, self.n) * scale).astype(np.float32)
+        self.dev["g32"][self.skew:self.skew + self.n].copy_(torch.from_numpy(self.host["g32"]))
+
+    def compare(self, what):
+        torch.cuda.synchronize()
+        for key in ("p32", "m", "v", "g32"):
+            assert_bits_equal(self.dev[key][self.skew:self.skew + self.n].cpu().numpy(), self.host[key], f"{what}: torch-managed {key}")
+
+
+@pytest.mark.parametrize("seed", [11, 12])
+def test_torch_managed_fp32_tensors_take_their_place_in_the_call_sequence(seed):
+    """ps_adam_step_tensors_each with PS_TENSOR_GRAD_F32 tensors among the chunk tensors (the reference's TORCH_BASED
+    parameters: fp32 gradient handed to the operator as it is, no fp16 copy, no overflow probe, nothing restored on
+    a skipped step; fp16_cpu_adam.py:345-353,301-302,459-460): any of them may be the step's first call, they carry
+    their own step numbers and hyper-parameters like every tensor, whole aligned tiles and ragged / unaligned ones,
+    with and without the gradient clamp, host- and device-decided, under both arithmetics of the chunk tensors.
+    Bar: bit-exact against the oracle."""
+    lib = _lib.load()
+    rng = np.random.default_rng(seed)
+    for case in range(16):
+        n = int(rng.choice([700, 1500, 4099]))
+        R = RawChunks(2, n, seed=int(rng.integers(1 << 30)))
+        nt = int(rng.choice([3000, 5000]))
+        T = _TorchManaged(nt, seed=int(rng.integers(1 << 30)), skew=int(rng.choice([0, 0, 1, 4])))
+        spans = []
+        for ci in range(2):
+            cuts = sorted(set([0, n] + [int(x) for x in rng.integers(0, n + 1, int(rng.integers(1, 4)))]))
+            spans += [(ci, a, b - a) for a, b in zip(cuts[:-1], cuts[1:])]
+        cuts = sorted(set([0, 2048, nt] + [int(x) for x in rng.integers(2048, nt + 1, int(rng.integers(0, 3)))]))
+        spans += [(2, a, b - a) for a, b in zip(cuts[:-1], cuts[1:])]
+        spans = [spans[i] for i in rng.permutation(len(spans))]
+        torch_arith = rng.random() < 0.4
+        gated = bool(rng.integers(0, 2))
+        adamw = bool(rng.integers(0, 2))
+        clip = float(rng.choice([-1, -1, 0.5]))
+        base = int(rng.integers(0, 50))
+        oid = 9300 + case
+        _lib.check(lib.ps_adam_create(oid, 1e-3, 0.9, 0.999, 1e-8, 0.0, int(adamw), 0), "create")
+        if clip > 0:
+            _lib.check(lib.ps_adam_set_grad_clamp(oid, clip), "clamp")
+        if torch_arith:
+            _lib.check(lib.ps_adam_set_arithmetic(oid, _lib.PS_ARITH_TORCH), "arithmetic")
+        if gated:
+            kw = dict(init_scale=float(rng.choice([2.0**10, 1000.0])), scale_factor=2, scale_window=int(rng.integers(1, 4)), min_scale=1)
+            scaler = ps.DynamicLossScaler(**kw)
+            scaler.materialize("cuda:0", betas=(0.9, 0.999))
+            scaler._seed_step(base)
+            oscaler = oracle.ScalerOracle(**kw)
+        else:
+            scale = [None, 8.0, 2.0**12, 1000.0][int(rng.integers(0, 4))]
+            oscaler = oracle.StaticScalerOracle(scale) if scale else None
+        oopt = oracle.OptimizerStepOracle(R.host + [T.host], oscaler, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0,
+                                          use_adamw=adamw, tensors=spans, gradient_clipping=clip,
+                                          arithmetic="torch" if torch_arith else "operator")
+        uniform = rng.random() < 0.4  # every tensor with the same numbers: what an ordinary run looks like
+        for span in spans:
+            st = oopt.state(span)
+            st["step"] = base if uniform else base + int(rng.integers(0, 3))
+            if not uniform:
+                st["lr"] = float(rng.choice([1e-3, 5e-4]))
+                st["weight_decay"] = float(rng.choice([0.0, 0.01]))
+                st["betas"] = [(0.9, 0.999), (0.8, 0.99)][int(rng.integers(0, 2))]
+        device_step = base
+        what = (f"seed {seed} case {case}: n={n} nt={nt} skew={T.skew} tensors={len(spans)} first={spans[0]} torch={torch_arith} "
+                f"gated={gated} adamw={adamw} clip={clip} uniform={uniform}")
+        workspace = torch.empty(64 * len(spans), dtype=torch.uint8, device="cuda")
+        stream = _lib.current_stream_handle()
+        rows = [T.row(off) if ci == 2 else [t[o + off:].data_ptr() for t, o in zip(R.dev[ci], R.offs)] for ci, off, _ in spans]
+        table, sizes = _lib.chunk_array(rows), (ctypes.c_size_t * len(spans))(*[s[2] for s in spans])
+        each = (_lib.ps_tensor_call * len(spans))()
+        n_operator = sum(1 for ci, _, _ in spans if ci == 2 or not torch_arith)
+        for it in range(int(rng.integers(3, 6))):
+            for e, span in zip(each, spans):
+                st = oopt.state(span)
+                e.lr, (e.beta1, e.beta2), e.eps, e.weight_decay = st["lr"], st["betas"], st["eps"], st["weight_decay"]
+                e.step = st["step"] + 1 - (device_step + 1) if gated else st["step"] + 1
+                e.arithmetic = _lib.PS_ARITH_OPERATOR if span[0] == 2 else -1
+                e.flags = _lib.PS_TENSOR_GRAD_F32 if span[0] == 2 else 0
+            cur = float(oscaler.loss_scale) if oscaler else 1.0
+            T.new_grads(rng, cur)
+            if gated:
+                poison = (int(rng.integers(0, 2)), int(rng.integers(0, n))) if rng.random() < 0.3 else None
+                R.new_grads(rng, cur, poison=poison)
+                _lib.check(lib.ps_overflow_scan_chunks(R.table, 2, n, None, scaler.state_ptr, stream), "scan")
+                _lib.check(lib.ps_adam_step_tensors_each(oid, 1, table, sizes, each, len(spans), -1.0, scaler.state_ptr,
+                                                         workspace.data_ptr(), workspace.numel(), stream), "each")
+                scaler.update_scale(None, operator_calls=n_operator)
+                oopt.check_overflow()
+                assert oopt.step() == (poison is not None), what
+                device_step += poison is None
+                assert scaler.loss_scale == oscaler.loss_scale and scaler.adam_step == device_step, what
+            else:
+                R.new_grads(rng, cur)
+                _lib.check(lib.ps_adam_step_tensors_each(oid, 1, table, sizes, each, len(spans), float(oscaler.loss_scale) if oscaler else -1.0,
+                                                         None, None, 0, stream), "each")
+                oopt.step()
+            R.compare(f"{what} iteration {it}")
+            T.compare(f"{what} iteration {it}")
+        lib.ps_adam_destroy(oid)

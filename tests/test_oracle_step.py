@@ -384,3 +384,65 @@ def test_every_tensor_carries_its_own_hyper_parameters():
     assert np.array_equal(cs2[0]["p32"][250:550], before[0]["p32"][250:550])
     want = before[0]["p32"][:250].astype(np.float64) * (1 - 1e-2 * 0.1)
     assert np.allclose(cs2[0]["p32"][:250], want, rtol=1e-6, atol=0)
+
+
+def test_torch_managed_tensors_go_through_the_operator_with_their_fp32_gradients():
+    """A chunk dict with `g32` in place of `p16` (the reference's TORCH_BASED parameters, fp16_cpu_adam.py:345-353):
+    listed first, its tensor is the step's first operator call and takes the multiplying branch; its fp32 gradient
+    reaches the operator unrounded (a gradient of 1e-9 * scale, which fp16 cannot hold after scaling by 1/64, still
+    moves the state); it is the operator's arithmetic also when the chunk tensors take the torch formula; an inf in
+    it is NOT seen by the overflow probe; a skipped step leaves it alone; no fp16 copy exists.  Every tensor against
+    a fresh operator object driven into the branch by hand, and the fp32 path against float64 textbook Adam."""
+    kw = dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0, use_adamw=True)
+    rng = np.random.default_rng(41)
+    for arithmetic in ("operator", "torch"):
+        cs = _chunks(n_chunks=1, n=300, seed=42)
+        managed = {"p32": rng.normal(0, 0.02, 200).astype(np.float32), "m": np.zeros(200, np.float32),
+                   "v": np.zeros(200, np.float32), "g32": np.zeros(200, np.float32)}
+        tensors = [(1, 0, 120), (0, 0, 300), (1, 120, 80)]
+        s = oracle.ScalerOracle(init_scale=64, scale_factor=2, scale_window=1000)
+        opt = oracle.OptimizerStepOracle(cs + [managed], s, tensors=tensors, arithmetic=arithmetic, **kw)
+        for t in (1, 2, 3):
+            cs[0]["p16"][...] = (rng.normal(0, 1e-3, 300) * 64).astype(np.float16)
+            managed["g32"][...] = (rng.normal(0, 1e-9, 200) * 64).astype(np.float32)
+            ref = _copy(cs + [managed])
+            opt.check_overflow()
+            assert opt.step() is False
+            for k, (ci, off, numel) in enumerate(tensors):
+                if ci == 0 and arithmetic == "torch":
+                    continue  # the torch formula is pinned elsewhere; it leaves the operator object alone
+                o = oracle.AdamOracle(1e-3, 0.9, 0.999, 1e-8, 0.0, True)
+                if k == 0 and t > 1:
+                    o.advance(t - 1, 0.9, 0.999)
+                elif k > 0:
+                    o.advance(t, 0.9, 0.999)
+                sl = slice(off, off + numel)
+                o.update(t, 1e-3, 0.9, 0.999, 1e-8, 0.0, True, ref[ci]["p32"][sl], ref[ci]["g32" if ci == 1 else "p16"][sl],
+                         ref[ci]["m"][sl], ref[ci]["v"][sl], 64.0)
+            for ci, (c, r) in enumerate(zip(cs + [managed], ref)):
+                if ci == 0 and arithmetic == "torch":
+                    continue
+                for key in ("p32", "m", "v"):
+                    assert np.array_equal(c[key].view(np.uint32), r[key].view(np.uint32)), (arithmetic, t, ci, key)
+            assert "p16" not in managed
+        # float64 textbook Adam from zero state over the same three gradients would need the history; one step is enough:
+        fresh = {"p32": np.zeros(4, np.float32), "m": np.zeros(4, np.float32), "v": np.zeros(4, np.float32),
+                 "g32": (np.array([1e-9, -3e-9, 2e-7, 5e-4]) * 64).astype(np.float32)}
+        one = oracle.OptimizerStepOracle([fresh], oracle.StaticScalerOracle(64), tensors=[(0, 0, 4)], arithmetic=arithmetic, **kw)
+        one.step()
+        g = fresh["g32"].astype(np.float64) / 64
+        expect = -1e-3 * (0.1 * g / 0.1) / (np.sqrt(0.001 * g * g / 0.001) + 1e-8)
+        np.testing.assert_allclose(fresh["p32"], expect, rtol=2e-5)
+        assert abs(fresh["p32"][0]) > 5e-5  # g = 1e-9 is far below eps after fp16 rounding would have lost it; here it counts
+        # an inf in the fp32 gradient is not probed (core/hook.py:202-203); an inf in the chunk is, and the skipped step
+        # leaves the torch-managed tensors as they are
+        managed["g32"][3] = np.inf
+        cs[0]["p16"][...] = np.float16(0.5)
+        opt.check_overflow()
+        assert opt.has_overflow is False
+        cs[0]["p16"][7] = np.inf
+        before = _copy([managed])[0]
+        opt.check_overflow()
+        assert opt.step() is True and s.loss_scale == 32.0
+        for key in ("p32", "m", "v", "g32"):
+            assert np.array_equal(managed[key].view(np.uint32), before[key].view(np.uint32))
