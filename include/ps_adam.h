@@ -321,7 +321,8 @@ size_t ps_tensors_each_workspace_bytes(int n_tensors);
  *                    with ps_scaler_update (operator_calls = the number of operator-arithmetic calls), which
  *                    adopts it on a clean step and drops it on a skipped one.
  * Addresses may be pinned host memory (host-resident optimizer state is then read and written over the link in
- * place).  The clamp of ps_adam_set_grad_clamp applies. */
+ * place).  The clamp of ps_adam_set_grad_clamp applies.  Tensors flagged PS_TENSOR_GRAD_F32 (above) take part in
+ * the call sequence like any other. */
 int ps_adam_step_tensors_each(int optimizer_id, int bias_correction, const ps_chunk* tensors,
                               const size_t* numels, const ps_tensor_call* each, int n_tensors,
                               double loss_scale, ps_step_state* d_state, void* d_workspace,

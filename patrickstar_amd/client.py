@@ -67,6 +67,7 @@ class PatrickStarClient:
         self.chunk_tensor_index = ChunkTensorIndex(default_chunk_size)
         self.param_fp16_to_param_fp32_map: Dict[torch.nn.Parameter, torch.nn.Parameter] = {}
         self.chunk_based_param_fp16: List[torch.nn.Parameter] = []
+        self.torch_managed_params: List[torch.nn.Parameter] = []  # fp32 parameters outside the chunk lists (use_cpu_embedding)
         self.module = None
         self.optimizer = None
         self._param_idx = 0
@@ -193,10 +194,40 @@ class PatrickStarClient:
             )
         self.host_chunk_policy = planned.__contains__
 
-    def register_model(self, model):
+    def register_torch_managed_embedding(self, module):
+        """``use_cpu_embedding`` of the reference (``patrickstar/core/preprocess.py:351-364``,
+        ``patrickstar/ops/embedding.py:81-104``): the weights of an ``nn.Embedding`` stay fp32 parameters that PyTorch
+        manages itself (``ParamType.TORCH_BASED``), outside the chunk lists; the lookup runs in fp32 and its output
+        is cast to half.  The reference keeps such weights in host memory and looks them up on the CPU; here they
+        stay in HBM (this package has no CPU compute path), which changes where the work runs, not its numbers.
+        The optimizer updates them with the operator's arithmetic from their fp32 gradients
+        (``patrickstar/ops/fp16_cpu_adam.py:345-353``).  As in the reference (``preprocess.py:260-282``) an empty
+        fp16 parameter is put in front of the module's own, so that code which takes a model's dtype from its
+        first parameter still sees half."""
+        for name, param in module.named_parameters(recurse=False):
+            if is_param_registered(param):
+                continue
+            register_param(param, ParamType.TORCH_BASED, torch.float, f"embedding_{name}")
+            param.data = param.data.to(self.device, torch.float)
+            self.torch_managed_params.append(param)
+        if "dummy" not in module._parameters:
+            module.dummy = torch.nn.Parameter(torch.tensor([], dtype=torch.half, device=self.device), requires_grad=False)
+            register_param(module.dummy, ParamType.TORCH_BASED, torch.half, "embedding_dummy")
+            others = [(k, module._parameters.pop(k)) for k in list(module._parameters) if k != "dummy"]
+            module._parameters.update(others)  # "dummy" is now the first entry
+        lookup = module.forward
+
+        def forward_to_half(input_):
+            return lookup(input_).to(torch.half)
+
+        module.forward = forward_to_half
+
+    def register_model(self, model, use_cpu_embedding=False):
         """Register every module's own parameters in module CONSTRUCTION order (children finish
         constructing before their parent does), copy the initial values into the fp16 and fp32
-        payloads and re-point each parameter at its fp16 chunk slot."""
+        payloads and re-point each parameter at its fp16 chunk slot.  ``use_cpu_embedding``: the
+        weights of ``nn.Embedding`` modules stay fp32 parameters of PyTorch's own (see
+        ``register_torch_managed_embedding``)."""
         self.module = model
         # a module's parameters are views of the fp16 payloads, which forward and backward need in HBM:
         # positions selected by the host-chunk policy keep only their optimizer state in host memory
@@ -205,7 +236,10 @@ class PatrickStarClient:
         def visit(m):
             for child in m.children():
                 visit(child)
-            self.register_module_params(m)
+            if use_cpu_embedding and isinstance(m, torch.nn.Embedding):
+                self.register_torch_managed_embedding(m)
+            else:
+                self.register_module_params(m)
 
         visit(model)
         self.plan_placement()
@@ -321,6 +355,8 @@ class PatrickStarClient:
     # -- tensor views -----------------------------------------------------------
     def access_data(self, param, device=None):
         """The tensor of ``param`` inside its chunk payload (a view; nothing moves)."""
+        if param.ps_attr.param_type == ParamType.TORCH_BASED:
+            return param.data  # PyTorch's own tensor (patrickstar/core/client.py:552-553)
         info = self.chunk_tensor_index.get_tensor_info(param.ps_attr.data_id())
         payload = self.chunk_list[info.chunk_id].payload
         if payload is None:

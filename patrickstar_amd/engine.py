@@ -214,7 +214,9 @@ def initialize_engine(model_func, local_rank, config=None, client=None):
         # needs it when it places the payloads
         client.use_hybrid_adam = bool(parse_config(config)[1].get("use_hybrid_adam", True))
         model = model_func()
-        client.register_model(model)
+        # "use_cpu_embedding" (the reference's default is True, patrickstar/runtime/__init__.py:62-69; here it has to
+        # be asked for): embedding weights stay fp32 parameters of PyTorch's own and are updated from fp32 gradients
+        client.register_model(model, use_cpu_embedding=bool(cfg.get("use_cpu_embedding", False)))
     engine = PatrickStarEngine(model=model, client=client, config=config)
     client.start_mem_tracer()
     return (engine, engine.optimizer)

@@ -154,7 +154,14 @@ class FP16Adam(torch.optim.Optimizer):
                 dict.__setitem__(st, "eps", group["eps"])
                 dict.__setitem__(st, "step", 0)
                 if p.ps_attr.param_type == ParamType.TORCH_BASED:
-                    raise NotImplementedError("torch-managed (CPU embedding) parameters are outside this path")
+                    # a parameter PyTorch manages itself (fp32 embedding weights under use_cpu_embedding): plain fp32
+                    # moments beside it (fp16_cpu_adam.py:122-131)
+                    if p.requires_grad:
+                        for key in ("exp_avg", "exp_avg_sq"):
+                            sp = torch.nn.Parameter(torch.zeros_like(p.data, dtype=torch.float), requires_grad=False)
+                            register_param(sp, ParamType.TORCH_BASED, torch.float, f"{p.ps_attr.name}.{key}")
+                            dict.__setitem__(st, key, sp)
+                    continue
                 if not p.ps_attr.is_local():
                     continue
                 name = p.ps_attr.name
@@ -228,6 +235,10 @@ class FP16Adam(torch.optim.Optimizer):
         """The parameters ``step()`` updates, in the order the reference visits them (``fp16_cpu_adam.py:566-605``)."""
         return [p for group in self.param_groups for p in group["params"] if p.requires_grad and p.ps_attr.is_local()]
 
+    @staticmethod
+    def _torch_managed(p):
+        return p.ps_attr.param_type == ParamType.TORCH_BASED
+
     def _build_tables(self):
         """Descriptors of what one step covers, and how the reference would have cut it into operator calls.
 
@@ -238,7 +249,7 @@ class FP16Adam(torch.optim.Optimizer):
         """
         cl = self.client.chunk_list
         index = self.client.chunk_tensor_index
-        trainable = self._trainable()
+        trainable = [p for p in self._trainable() if not self._torch_managed(p)]  # the chunk lists' part of the step
         live_ids = {p.ps_attr.data_id() for p in trainable}
         chunk_of = {p: index.get_tensor_info(p.ps_attr.data_id()).chunk_id for p in trainable}
         live_chunks = set(chunk_of.values())
@@ -310,6 +321,13 @@ class FP16Adam(torch.optim.Optimizer):
         rows, numels = [], []
         for p in params:
             st = self.state[p]
+            if self._torch_managed(p):
+                # the parameter itself is the fp32 master; the fourth address is its fp32 gradient's, which is a new
+                # tensor after every backward: _step_each writes it in before every step
+                rows.append([p.data_ptr(), dict.__getitem__(st, "exp_avg").data_ptr(), dict.__getitem__(st, "exp_avg_sq").data_ptr(),
+                             p.data_ptr()])
+                numels.append(p.numel())
+                continue
             quad = (self.client.param_fp16_to_param_fp32_map[p], dict.__getitem__(st, "exp_avg"),
                     dict.__getitem__(st, "exp_avg_sq"), p)
             if slot is None:
@@ -541,7 +559,9 @@ class FP16Adam(torch.optim.Optimizer):
             common = steps[0]
             self._offsets = {p: t - common for p, t in zip(trainable, steps) if t != common}
         entries = [self._entries(p)[:4] + (self._offsets.get(p, 0),) for p in trainable]
-        if all(e == entries[0] for e in entries):
+        # parameters that PyTorch manages itself (fp32, with fp32 gradients) are tensors of their own kind: with them
+        # the step always goes tensor by tensor
+        if all(e == entries[0] for e in entries) and not any(self._torch_managed(p) for p in trainable):
             self._plan = {"kind": "uniform", "hyper": entries[0][:4]}
         else:
             self._plan = {"kind": "each", "trainable": trainable, "entries": entries, "table": None}
@@ -588,7 +608,8 @@ class FP16Adam(torch.optim.Optimizer):
                 rows, numels, n = self._tensor_rows(trainable)
                 on_host = {pos.fp16 for pos in self.client.positions() if pos.on_host}
                 index = self.client.chunk_tensor_index
-                host = [index.get_tensor_info(p.ps_attr.data_id()).chunk_id in on_host for p in trainable]
+                host = [not self._torch_managed(p) and index.get_tensor_info(p.ps_attr.data_id()).chunk_id in on_host
+                        for p in trainable]
                 workspace = None
                 if self._dynamic:
                     nbytes = self._lib.ps_tensors_each_workspace_bytes(n)
@@ -598,21 +619,36 @@ class FP16Adam(torch.optim.Optimizer):
             each = (_lib.ps_tensor_call * n)()
             operator_calls = 0
             offsets = [e[4] for e in plan["entries"]]
+            managed = []  # (row, parameter) of the tensors PyTorch manages itself
             for i, (lr, (beta1, beta2), eps, weight_decay, d) in enumerate(plan["entries"]):
                 e = each[i]
                 e.lr, e.beta1, e.beta2, e.eps, e.weight_decay = lr, beta1, beta2, eps, weight_decay
                 # optimizer state in host memory is updated by the operator whatever the optimizer's arithmetic
-                # (fp16_cpu_adam.py:415-443); the kernel reads and writes such pinned payloads over the link
-                e.arithmetic = _lib.PS_ARITH_OPERATOR if (host[i] or self.arithmetic == "operator") else _lib.PS_ARITH_TORCH
+                # (fp16_cpu_adam.py:415-443); the kernel reads and writes such pinned payloads over the link.  The
+                # reference keeps the parameters PyTorch manages itself on the CPU, so theirs is the operator's too.
+                own = self._torch_managed(trainable[i])
+                e.arithmetic = _lib.PS_ARITH_OPERATOR if (host[i] or own or self.arithmetic == "operator") else _lib.PS_ARITH_TORCH
                 operator_calls += e.arithmetic == _lib.PS_ARITH_OPERATOR
+                if own:
+                    e.flags = _lib.PS_TENSOR_GRAD_F32
+                    managed.append((i, trainable[i]))
                 if self._dynamic:
                     e.step = d  # a device-decided step is told every tensor's distance from the device's counter
-            plan["table"] = (rows, numels, n, each, workspace, operator_calls, offsets)
+            plan["table"] = (rows, numels, n, each, workspace, operator_calls, offsets, managed)
         return plan["table"]
 
     def _step_each(self, plan, stream):
         """One step through ``ps_adam_step_tensors_each``."""
-        rows, numels, n, each, workspace, operator_calls, offsets = self._each_table(plan)
+        rows, numels, n, each, workspace, operator_calls, offsets, managed = self._each_table(plan)
+        for i, p in managed:
+            # fp16_cpu_adam.py:345-353: the gradient PyTorch left on the parameter, fp32, read where it is
+            g = p.grad
+            if g is None or g.dtype != torch.float or not g.is_contiguous() or g.device != p.device:
+                raise RuntimeError(
+                    f"{p.ps_attr.name}: a parameter that PyTorch manages itself needs a contiguous fp32 .grad on "
+                    f"{p.device} when step() runs (got {None if g is None else (g.dtype, g.device, g.is_contiguous())})"
+                )
+            rows[i].param_fp16 = g.data_ptr()
         if self._dynamic:
             scaler = self.loss_scaler
             _lib.check(

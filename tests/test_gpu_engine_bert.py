@@ -111,11 +111,14 @@ def test_bert_base_at_the_reference_chunk_size_matches_the_oracle():
     assert np.isfinite(float(loss.detach()))
 
 
-def test_checkpoint_reload_reproduces_the_losses_exactly():
+@pytest.mark.parametrize("use_cpu_embedding", [False, True])
+def test_checkpoint_reload_reproduces_the_losses_exactly(use_cpu_embedding):
     """The reference's checkpoint test (unitest/test_checkpoint.py:95-181) on a small BERT: train 5 steps, save model and
     optimizer, train 5 more on recorded batches, reload, and require (a) the loss right after reloading to EQUAL the
     loss at the save point and (b) the loss after re-training on the same 5 batches to EQUAL the loss of the first
-    run.  Both need the fp32 masters, m, v, the step counter and the loss-scaler state to come back bit for bit."""
+    run.  Both need the fp32 masters, m, v, the step counter and the loss-scaler state to come back bit for bit.
+    The reference's test sets "use_cpu_embedding": True (:100): the three embedding tables are then fp32 parameters
+    of PyTorch's own, updated from fp32 gradients and saved with the model as they are."""
     transformers = pytest.importorskip("transformers")
     cfg = transformers.BertConfig(
         vocab_size=256, hidden_size=64, num_hidden_layers=2, num_attention_heads=4, intermediate_size=128,
@@ -126,10 +129,14 @@ def test_checkpoint_reload_reproduces_the_losses_exactly():
         "optimizer": {"type": "Adam", "params": {"lr": 1e-3, "betas": (0.9, 0.999), "eps": 1e-6, "weight_decay": 0, "use_hybrid_adam": True}},
         "fp16": {"enabled": True, "loss_scale": 0, "initial_scale_power": 10, "loss_scale_window": 4, "hysteresis": 2, "min_loss_scale": 1},
         "default_chunk_size": 32 * 1024,
+        "use_cpu_embedding": use_cpu_embedding,
     }
     model, optimizer = ps.initialize_engine(
         model_func=lambda: transformers.BertForSequenceClassification(cfg), local_rank=0, config=config
     )
+    emb = model.module.bert.embeddings
+    assert emb.word_embeddings.weight.dtype == (torch.float if use_cpu_embedding else torch.half)
+    assert (optimizer._make_plan()["kind"] == "each") == use_cpu_embedding
     gen = torch.Generator(device="cuda")
     gen.manual_seed(1)
 

@@ -488,7 +488,7 @@ def test_hyper_parameters_are_read_from_the_state_entries_per_parameter():
     assert opt._plan is not None and opt._hyper()[0] == 1e-3
     opt.state[model.b.weight]["lr"] = 5e-4
     assert opt._plan is None and opt._hyper() == "each"
-    rows, numels, n, each, workspace, operator_calls, offsets = opt._each_table(opt._plan)
+    rows, numels, n, each, workspace, operator_calls, offsets, managed = opt._each_table(opt._plan)
     trainable = [model.scale, model.a.weight, model.b.weight, model.b.bias]  # parameters() order without a.bias
     assert n == 4 == operator_calls and workspace is None and list(numels) == [p.numel() for p in trainable]
     assert [each[i].lr for i in range(4)] == [1e-3, 1e-3, 5e-4, 1e-3]
