@@ -41,7 +41,7 @@ def _snap(t):
     return t.detach().to("cpu", copy=True).numpy()
 
 
-def _config(loss_scale, arithmetic, clip=None):
+def _config(loss_scale, arithmetic, clip=None, host=()):
     cfg = {
         "optimizer": {"type": "AdamW", "params": {"lr": 1e-3, "betas": (0.9, 0.999), "eps": 1e-8, "weight_decay": 0.05,
                                                   "arithmetic": arithmetic}},
@@ -52,13 +52,16 @@ def _config(loss_scale, arithmetic, clip=None):
     }
     if clip is not None:
         cfg["gradient_clipping"] = clip
+    if host:
+        cfg["client"] = {"host_chunk_policy": lambda position: position in host}
+        cfg["default_chunk_size"] = 520  # fc1 (500 elements) fills the first position, fc2 (168) goes to a second
     return cfg
 
 
 class _Run:
-    def __init__(self, loss_scale, arithmetic, clip=None, seed=0):
+    def __init__(self, loss_scale, arithmetic, clip=None, seed=0, host=()):
         torch.manual_seed(seed)
-        self.config = _config(loss_scale, arithmetic, clip)
+        self.config = _config(loss_scale, arithmetic, clip, host)
         self.engine, self.opt = ps.initialize_engine(model_func=_EmbNet, local_rank=0, config=self.config)
         self.client, self.module = self.engine.client, self.engine.module
         self.cl, self.pos = self.client.chunk_list, self.client.positions()
@@ -86,7 +89,7 @@ class _Run:
         self.spans = spans
         self.oopt = oracle.OptimizerStepOracle(
             self.chunks + self.own, self.oscaler, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.05, use_adamw=True,
-            tensors=spans, arithmetic=arithmetic, gradient_clipping=clip if clip is not None else -1)
+            tensors=spans, arithmetic=arithmetic, gradient_clipping=clip if clip is not None else -1, operator_chunks=tuple(host))
 
     def iterate(self, what, poison=False):
         poison = poison and self.dynamic
@@ -158,6 +161,19 @@ def test_per_parameter_numbers_and_freezing_apply_to_them_too(loss_scale):
     r.iterate("and on")
     skipped = 1 if r.dynamic else 0
     assert r.opt.state[m.pos.weight]["step"] == 4 - skipped and r.opt.state[m.emb.weight]["step"] == 6 - skipped
+
+
+@pytest.mark.parametrize("arithmetic", ["operator", "torch"])
+def test_with_optimizer_state_of_a_chunk_position_in_host_memory(arithmetic):
+    """The second chunk position keeps fp32 master, momentum and variance in pinned host memory (hybrid Adam): its
+    tensors take the operator's arithmetic whatever the optimizer's, the embeddings theirs, the first position the
+    optimizer's."""
+    r = _Run(0, arithmetic, seed=6, host=(1,))
+    assert len(r.pos) == 2 and r.pos[1].on_host and not r.pos[0].on_host
+    for k in (1, 2):
+        r.iterate(f"step {k}")
+    r.iterate("poisoned", poison=True)
+    r.iterate("step 3")
 
 
 def test_gradient_clamp_reaches_the_fp32_gradients():
