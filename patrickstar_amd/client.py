@@ -215,12 +215,8 @@ class PatrickStarClient:
             register_param(module.dummy, ParamType.TORCH_BASED, torch.half, "embedding_dummy")
             others = [(k, module._parameters.pop(k)) for k in list(module._parameters) if k != "dummy"]
             module._parameters.update(others)  # "dummy" is now the first entry
-        lookup = module.forward
-
-        def forward_to_half(input_):
-            return lookup(input_).to(torch.half)
-
-        module.forward = forward_to_half
+        # the lookup itself runs in fp32; what the rest of the model sees is half (ops/embedding.py:104)
+        module.register_forward_hook(lambda mod, args, output: output.to(torch.half))
 
     def register_model(self, model, use_cpu_embedding=False):
         """Register every module's own parameters in module CONSTRUCTION order (children finish
