@@ -421,3 +421,59 @@ def test_padding_is_skipped_only_while_zeros_stay_zeros():
                         assert np.array_equal(got[used:][keep], oc[1][key][used:][keep]), (what, key)
             tail = h.download(1)[0][used:]
             assert np.all(tail == 0) if eps > 0 else np.all(np.isnan(tail))
+
+
+@pytest.mark.parametrize("seed", [21, 22, 23])
+@pytest.mark.parametrize("loss_scale", [0, 128])
+def test_random_schedules_of_freezing_and_state_writes(loss_scale, seed):
+    """Thirty iterations in which, before each step, something a user may do to the optimizer happens at random:
+    parameters are frozen and thawed, learning rates are written for all parameters (a schedule) or for one, weight
+    decay, eps or betas for one or for all, step numbers are read (a read-back) or written by hand, the whole state goes
+    through state_dict() / load_state_dict(); with a dynamic scaler some iterations overflow.  After every step every
+    payload must equal the oracle's bit for bit, and every parameter's step number the reference's count."""
+    rng = np.random.default_rng(seed)
+    arithmetic = "torch" if seed == 23 else "operator"
+    r = _Run(loss_scale, arithmetic, seed=seed)
+    params = list(r.module.parameters())
+    number = {id(p): i for i, p in enumerate(params)}
+    for it in range(30):
+        what = f"seed {seed} iteration {it}"
+        for _ in range(int(rng.integers(0, 3))):
+            action = int(rng.integers(0, 8))
+            if action == 0:  # freeze or thaw one parameter (never the last trainable one)
+                p = params[int(rng.integers(0, len(params)))]
+                if not p.requires_grad or sum(q.requires_grad for q in params) > 1:
+                    p.requires_grad_(not p.requires_grad)
+                    r.trainable_changed()
+                    what += f"; requires_grad[{number[id(p)]}]={p.requires_grad}"
+            elif action == 1:  # a learning-rate schedule
+                lr = float(rng.choice([1e-3, 8e-4, 5e-4]))
+                for p in params:
+                    r.set(p, "lr", lr)
+                what += f"; lr={lr} for all"
+            elif action == 2:
+                p = params[int(rng.integers(0, len(params)))]
+                r.set(p, "lr", float(rng.choice([1e-3, 2e-3])))
+                what += f"; lr[{number[id(p)]}]"
+            elif action == 3:
+                p = params[int(rng.integers(0, len(params)))]
+                key, value = [("weight_decay", 0.0), ("weight_decay", 0.05), ("eps", 1e-6), ("eps", 1e-8)][int(rng.integers(0, 4))]
+                r.set(p, key, value)
+                what += f"; {key}[{number[id(p)]}]={value}"
+            elif action == 4:
+                betas = [(0.9, 0.999), (0.85, 0.98)][int(rng.integers(0, 2))]
+                targets = params if rng.random() < 0.5 else [params[int(rng.integers(0, len(params)))]]
+                for p in targets:
+                    r.set(p, "betas", betas)
+                what += f"; betas={betas} for {len(targets)}"
+            elif action == 5:  # somebody looks at the step numbers
+                assert r.steps() == r.oracle_steps(), what
+            elif action == 6:  # ... or writes one
+                p = params[int(rng.integers(0, len(params)))]
+                r.set(p, "step", int(rng.integers(0, 40)))
+                what += f"; step[{number[id(p)]}] written"
+            else:  # the optimizer's state out and in again (the same optimizer: its operator object runs on)
+                r.opt.load_state_dict(r.opt.state_dict())
+                what += "; state reloaded"
+        r.iterate(what, poison=rng.random() < 0.15)
+    assert r.steps() == r.oracle_steps()
