@@ -446,6 +446,72 @@ int main()
         PS_OK(ps_adam_destroy(35));
     }
 
+    // ---- a tensor with a binary32 gradient and no fp16 copy (PS_TENSOR_GRAD_F32: what the reference's loop does for
+    //      parameters PyTorch manages itself) as the step's FIRST operator call, in front of two whole chunks
+    {
+        const size_t nf = 256 * 5 + 19;
+        std::vector<float> fp(nf), fm(nf, 0.0f), fv(nf, 0.0f), fg(nf);
+        for (size_t i = 0; i < nf; ++i) fp[i] = (float)(rng.normal() * 0.02);
+        float *dp = nullptr, *dm = nullptr, *dv = nullptr, *dg = nullptr;
+        HIP_OK(hipMalloc(&dp, nf * 4));
+        HIP_OK(hipMalloc(&dm, nf * 4));
+        HIP_OK(hipMalloc(&dv, nf * 4));
+        HIP_OK(hipMalloc(&dg, nf * 4));
+        HIP_OK(hipMemcpy(dp, fp.data(), nf * 4, hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(dm, fm.data(), nf * 4, hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(dv, fv.data(), nf * 4, hipMemcpyHostToDevice));
+        PS_OK(ps_adam_create(36, lr, b1, b2, eps, wd, 1, 0));
+        oracle_adam_init(&native, lr, b1, b2, eps, wd, 1);
+        ps_chunk rows[3];
+        size_t lens[3] = {nf, n, n};
+        rows[0].param_fp32 = dp, rows[0].exp_avg = dm, rows[0].exp_avg_sq = dv;
+        rows[0].param_fp16 = reinterpret_cast<uint16_t*>(dg);  // the address of the binary32 gradient
+        for (int c = 0; c < 2; ++c)
+            rows[1 + c].param_fp32 = dev[c].p, rows[1 + c].exp_avg = dev[c].m, rows[1 + c].exp_avg_sq = dev[c].v,
+                     rows[1 + c].param_fp16 = dev[c].h;
+        ps_tensor_call each[3];
+        for (uint64_t step = 1; step <= 3; ++step) {
+            for (size_t i = 0; i < nf; ++i) fg[i] = (float)(rng.normal() * 1e-3 * scale);
+            HIP_OK(hipMemcpy(dg, fg.data(), nf * 4, hipMemcpyHostToDevice));
+            for (int c = 0; c < 2; ++c) {
+                new_gradients(rng, host[c], scale);
+                if (upload(host[c], dev[c], n)) return 2;
+            }
+            for (int k = 0; k < 3; ++k)
+                each[k] = ps_tensor_call{lr, b1, b2, eps, wd, (int64_t)step, -1, k == 0 ? PS_TENSOR_GRAD_F32 : 0};
+            PS_OK(ps_adam_step_tensors_each(36, 1, rows, lens, each, 3, scale, NULL, NULL, 0, stream));
+            HIP_OK(hipStreamSynchronize(stream));
+            oracle_adam_advance(&native, step, b1, b2);
+            oracle_adam_set(&native, lr, eps, wd, 1);
+            if (oracle_adam_span(&native, fp.data(), fg.data(), 0, fm.data(), fv.data(), nf, (float)scale, 0) <= 0) return 5;
+            for (int c = 0; c < 2; ++c) {
+                oracle_adam_advance(&native, step, b1, b2);
+                oracle_adam_set(&native, lr, eps, wd, 1);
+                if (oracle_adam_span(&native, host[c].p.data(), host[c].h.data(), 1, host[c].m.data(), host[c].v.data(), n,
+                                     (float)scale, 0) <= 0)
+                    return 5;
+                oracle_cast_f32_to_f16(host[c].p.data(), host[c].h.data(), n);
+                if (int rc = compare(host[c], dev[c], n, "step with a binary32-gradient tensor", c)) return rc;
+            }
+            std::vector<float> back(nf);
+            const float* src[4] = {dp, dm, dv, dg};
+            const std::vector<float>* want[4] = {&fp, &fm, &fv, &fg};
+            for (int k = 0; k < 4; ++k) {
+                HIP_OK(hipMemcpy(back.data(), src[k], nf * 4, hipMemcpyDeviceToHost));
+                if (memcmp(back.data(), want[k]->data(), nf * 4) != 0) {
+                    fprintf(stderr, "binary32-gradient tensor: array %d differs from the CPU restatement at step %llu\n", k,
+                            (unsigned long long)step);
+                    return 4;
+                }
+            }
+        }
+        HIP_OK(hipFree(dp));
+        HIP_OK(hipFree(dm));
+        HIP_OK(hipFree(dv));
+        HIP_OK(hipFree(dg));
+        PS_OK(ps_adam_destroy(36));
+    }
+
     // ---- a chunk list whose last chunk ends in zero padding: the step leaves the padding alone, same bits
     {
         const size_t used_last = 256 * 6 + 9;
@@ -501,7 +567,7 @@ int main()
         HIP_OK(hipFree(d_flag));
     }
     printf("c abi gpu check ok: 3 host-decided and 8 device-decided steps (2 skipped), 3 steps with host-resident chunks, "
-           "3 tensor-list steps in two calls each, 5 steps with per-tensor step numbers and hyper-parameters, 2 over a padded list, "
+           "3 tensor-list steps in two calls each, 5 steps with per-tensor step numbers and hyper-parameters, 3 with a binary32-gradient tensor as the first call, 2 over a padded list, "
            "the allocation-free probe, over %d x %zu elements\n", C, n);
     return 0;
 }
