@@ -26,8 +26,9 @@ class PermutedLayout:
         rng = np.random.default_rng(seed)
         self.sizes = sizes
         total = sum(sizes)
+        rot = 7 % len(sizes)
         order = {"p": list(range(len(sizes))), "m": list(reversed(range(len(sizes)))),
-                 "v": list(range(7, len(sizes))) + list(range(7))}
+                 "v": list(range(rot, len(sizes))) + list(range(rot))}
         self.off = {}
         for key, seq in order.items():
             cur, offs = 0, {}
@@ -231,3 +232,60 @@ def test_one_step_spread_over_two_tensor_list_calls_under_one_call_pattern(gated
     torch.cuda.synchronize()
     L.compare("after the refused calls")
     lib.ps_adam_destroy(oid)
+
+
+def test_long_tensors_through_the_tensor_list_entry_points():
+    """Tensors of up to 51 M elements (launch grids hundreds of thousands of tiles wide, one launch per long tensor) in
+    the permuted layout, whole lists compared: ps_adam_step_tensors, then ps_adam_step_tensors_each host-decided and
+    device-decided with three sets of numbers among the tensors."""
+    lib = _lib.load()
+    sizes = [50257 * 1024, 4096 * 1600, 1600, 2_000_001, 1600 * 1600, 7]
+    scale = 2.0**10
+    L = PermutedLayout(sizes, seed=3, scale=scale)
+    rng = np.random.default_rng(4)
+    lr, b1, b2, eps, wd = 1e-3, 0.9, 0.999, 1e-8, 0.01
+    _lib.check(lib.ps_adam_create(871, lr, b1, b2, eps, wd, 1, 0), "create")
+    native = oracle.AdamOracle(lr, b1, b2, eps, wd, True)
+    stream = _lib.current_stream_handle()
+    for step in (1, 2):
+        if step > 1:
+            L.new_grads(rng, scale)
+        _lib.check(lib.ps_adam_step_tensors(871, step, lr, b1, b2, eps, wd, 1, L.table, L.numels, len(sizes), None, scale, None, stream),
+                   "ps_adam_step_tensors")
+        for i in range(len(sizes)):
+            p, g, m, v = L.views(i)
+            native.update(step, lr, b1, b2, eps, wd, True, p, g, m, v, scale)
+            g[...] = oracle.cast_fp32_to_fp16(p)
+        L.compare(f"tensor list, step {step}")
+    # every tensor its own numbers: the long one two steps behind, two at another learning rate
+    made = [0, 2, 2, 2, 2, 2]
+    lrs = [lr, lr, 5e-4, lr, 5e-4, lr]
+    each = (_lib.ps_tensor_call * len(sizes))()
+    for gated in (False, True):
+        if gated:
+            kw = dict(init_scale=2**10, scale_factor=2, scale_window=1000, min_scale=1)
+            scaler = ps.DynamicLossScaler(**kw)
+            scaler.materialize("cuda:0", betas=(b1, b2))
+            scaler._seed_step(made[1])  # the counter of the steps made so far, behind it a fresh operator object
+            native = oracle.AdamOracle(lr, b1, b2, eps, wd, True)  # ... on both sides
+            workspace = torch.empty(lib.ps_tensors_each_workspace_bytes(len(sizes)), dtype=torch.uint8, device="cuda")
+        for it in range(2):
+            L.new_grads(rng, scale)
+            for i, e in enumerate(each):
+                e.lr, e.beta1, e.beta2, e.eps, e.weight_decay, e.arithmetic = lrs[i], b1, b2, eps, wd, -1
+                e.step = made[i] - made[1] if gated else made[i] + 1
+            if gated:
+                _lib.check(lib.ps_adam_step_tensors_each(871, 1, L.table, L.numels, each, len(sizes), -1.0, scaler.state_ptr,
+                                                         workspace.data_ptr(), workspace.numel(), stream), "each")
+                scaler.update_scale(None, operator_calls=len(sizes))
+            else:
+                _lib.check(lib.ps_adam_step_tensors_each(871, 1, L.table, L.numels, each, len(sizes), scale, None, None, 0, stream), "each")
+            for i in range(len(sizes)):
+                made[i] += 1
+                p, g, m, v = L.views(i)
+                native.update(made[i], lrs[i], b1, b2, eps, wd, True, p, g, m, v, scale)
+                g[...] = oracle.cast_fp32_to_fp16(p)
+            L.compare(f"per-tensor numbers, gated={gated}, iteration {it}")
+        if gated:
+            assert scaler.adam_step == made[1] and scaler.loss_scale == 2**10
+    lib.ps_adam_destroy(871)
