@@ -477,3 +477,53 @@ def test_random_schedules_of_freezing_and_state_writes(loss_scale, seed):
                 what += "; state reloaded"
         r.iterate(what, poison=rng.random() < 0.15)
     assert r.steps() == r.oracle_steps()
+
+
+def test_a_step_with_per_tensor_numbers_replays_from_a_hip_graph():
+    """The device-decided per-tensor step (probe, the small kernel that forms every call's constants from the
+    device-resident state, the update kernels, the scale update) is a fixed sequence of launches too: tensors stand at
+    fixed DISTANCES from the device's counter, so one captured graph serves later iterations, clean and poisoned.
+    Every replay is compared with the oracle, with eager work and synchronisation in between."""
+    kw = dict(init_scale=2**10, scale_factor=2, scale_window=3, min_scale=1)
+    scaler = ps.DynamicLossScaler(**kw)
+    h = ChunkHarness(3, 256 * 9 + 7, scaler, seed=78, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
+    h.fill_state()
+    oc = h.oracle_chunks()
+    oscaler = oracle.ScalerOracle(**kw)
+    oopt = oracle.OptimizerStepOracle(oc, oscaler, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, use_adamw=True)
+    spans = list(oopt.tensors)
+    # the second tensor at another learning rate, the third four steps ahead of the others
+    h.opt.state[h.params[1]]["lr"] = 5e-4
+    oopt.state(spans[1])["lr"] = 5e-4
+    h.opt.state[h.params[2]]["step"] = 4
+    oopt.state(spans[2])["step"] = 4
+
+    def one_iteration(run_step, it):
+        h.fill_grads(1e-3, float(oscaler.loss_scale))
+        if it in (2, 5):
+            h.payloads(it % 3)[3][it] = float("inf") if it == 2 else float("nan")
+        for i, c in enumerate(oc):
+            c["p16"][...] = h.download(i)[3]
+        run_step()
+        torch.cuda.synchronize()
+        oopt.check_overflow()
+        assert oopt.step() is (it in (2, 5))
+        h.compare(oc, what=f"iteration {it}")
+        assert scaler.loss_scale == oscaler.loss_scale
+
+    one_iteration(h.opt.step, 0)  # eager: makes the plan, the tensor table and the workspace; nothing is allocated afterwards
+    assert h.opt._plan["kind"] == "each"
+    graph = torch.cuda.CUDAGraph()
+    h.fill_grads(1e-3, float(oscaler.loss_scale))
+    for i, c in enumerate(oc):
+        c["p16"][...] = h.download(i)[3]
+    with torch.cuda.graph(graph):
+        h.opt.step()
+    graph.replay()
+    torch.cuda.synchronize()
+    oopt.check_overflow()
+    assert oopt.step() is False
+    h.compare(oc, what="first replay")
+    for it in range(2, 9):
+        one_iteration(graph.replay, it)
+    assert [h.opt.state[p]["step"] for p in h.params] == [7, 7, 11] == [oopt.state(s)["step"] for s in spans]
