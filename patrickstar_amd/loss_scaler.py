@@ -3,7 +3,7 @@
 ``LossScaler`` (static) and ``DynamicLossScaler`` keep the constructor
 arguments, methods and semantics of ``patrickstar/fp16/loss_scaler.py:46-190``.
 The dynamic scaler's state (current scale, iteration, last overflow iteration,
-hysteresis credit) lives in a 192-byte device struct (``ps_step_state``) that the
+hysteresis credit) lives in a 256-byte device struct (``ps_step_state``) that the
 HIP kernels read and update, so the optimizer step never has to ask the host
 whether gradients overflowed.  Reading a field from Python
 (``loss_scale``, ``cur_iter``, ...) copies the struct back, which is the only
