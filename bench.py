@@ -24,7 +24,8 @@ same run:
   unfused_gpu_baseline   the reference's GPU branch restated with torch kernels;
   cpu_baseline   the CPU oracle (a port of the reference's AVX/OpenMP Adam) on this host: reported baseline only.
 `--mode ceiling` measures the memory system itself (pure read, pure write, 1:1 copy, the step's access pattern without
-arithmetic) with plain streaming kernels on the same buffers, next to the library's kernels.
+arithmetic) with plain streaming kernels on the same buffers, next to the library's kernels.  `--mode aux` times the
+kernels around the step (inf / nan probe, fp32 -> fp16 write-back, cast, backward-side gradient copy), each alone.
 """
 import argparse
 import ctypes
@@ -64,12 +65,13 @@ def parse_args():
     ap.add_argument("--host-fp16", choices=["host", "hbm"], default="host",
                     help="hybrid leg: where a host-resident position keeps its fp16 payload (host: the whole "
                     "position is streamed, 14 B/element each way; hbm: only fp32 param / m / v are, 12 B/element)")
-    ap.add_argument("--mode", choices=["static", "dynamic", "hybrid", "ceiling", "operator"], default="static",
+    ap.add_argument("--mode", choices=["static", "dynamic", "hybrid", "ceiling", "operator", "aux"], default="static",
                     help="static: the 1.5 B-parameter configuration as specified (static loss scale, one fused kernel per step) "
                     "plus the extra legs. dynamic: the headline numbers are those of the dynamic step. hybrid: only the "
                     "hybrid-placement leg, as its own JSON line. ceiling: streaming-kernel ceilings of the memory system. "
                     "operator: the per-tensor operator (ps_adam_update, what an unchanged FP16Adam loop calls) and the "
-                    "chunk-list step on ONE 64 Mi-element tensor / chunk")
+                    "chunk-list step on ONE 64 Mi-element tensor / chunk. aux: the kernels around the step (probe, write-back, cast, "
+                    "backward-side gradient copy), each alone")
     ap.add_argument("--arithmetic", choices=["operator", "torch"], default="operator",
                     help="operator: the native operator's order of operations (default, the headline line); "
                     "torch: the formula of the reference's GPU branch")
@@ -893,6 +895,87 @@ def operator_mode(args):
     print(json.dumps(out))
 
 
+def aux_mode(args):
+    """The kernels around the fused step, each alone on the buffers of the 1.5 B configuration: the inf / nan probe over
+    the fp16 payloads (patrickstar/fp16/loss_scaler.py:133-155 once per parameter there), its allocation-free form, the
+    fp32 -> fp16 write-back of a skipped step (patrickstar/ops/fp16_cpu_adam.py:287-310), the stand-alone cast
+    (patrickstar/ops/chunk_io_buff.py:116-126) and the backward-side gradient copy with its probe
+    (patrickstar/core/hook.py:200-230) next to Tensor.copy_ on the same tensors.  One JSON line; every entry is over
+    `--steps` launches, each timed with its own pair of events on the launch stream."""
+    import torch
+
+    import patrickstar_amd as ps
+    from patrickstar_amd import _lib
+
+    dev = torch.device("cuda:0")
+    C, N = args.chunks, args.chunk_size
+    client = ps.PatrickStarClient(0, N)
+    params = client.append_flat_chunks(C)
+    scaler = ps.DynamicLossScaler(init_scale=2**12, scale_factor=2, scale_window=1000, min_scale=1)
+    opt = ps.FP16Adam(client, params, loss_scaler=scaler, use_adamw=True, **HYPER)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(0)
+    cl = client.chunk_list
+    for pos in client.positions():
+        cl[pos.fp32].payload.normal_(0, 0.02, generator=gen)
+        cl[pos.fp16].payload.copy_(torch.empty(N, device=dev).normal_(0, 1e-3, generator=gen).mul_(2.0**12))
+    lib = _lib.load()
+    table, n_dev, _ = opt._build_tables()
+    state = scaler.state_ptr
+    flag = torch.zeros(1, dtype=torch.int32, device=dev)
+
+    def entry(fn, nbytes, what, steps=None):
+        _, ms = time_steps(torch, fn, steps or args.steps, args.warmup)
+        avg, med = sum(ms) / len(ms), sorted(ms)[len(ms) // 2]
+        gbps = nbytes / (avg * 1e-3) / 1e9
+        return {"what": what, "bytes": nbytes, "avg_device_ms": avg, "median_device_ms": med, "min_device_ms": min(ms),
+                "achieved_GBps": gbps, "frac": gbps / HBM_PEAK_GBS}
+
+    def stream():
+        return _lib.current_stream_handle()
+
+    out = {
+        "metric": "achieved HBM GB/s of the kernels around the fused Adam step, 1 GPU",
+        "config": {"workload": f"{C} chunks x {N} elements resident in HBM (probe, write-back); one tensor of {N} elements "
+                   "(cast, gradient copy)", "chunks": C, "chunk_numel": N},
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "unit": "GB/s", "dtype": "f16/f32", "data": "synthetic",
+        "scan_chunks": entry(lambda: _lib.check(lib.ps_overflow_scan_chunks(table, n_dev, N, None, state, stream()), "scan"),
+                             2 * C * N, "ps_overflow_scan_chunks: inf / nan probe of every fp16 payload (2 B/element), alone"),
+        "scan_chunks_noalloc": entry(lambda: _lib.check(lib.ps_overflow_scan_chunks_noalloc(table, n_dev, N, flag.data_ptr(), stream()),
+                                                        "scan_noalloc"),
+                                     2 * C * N, "ps_overflow_scan_chunks_noalloc: the same probe without atomics or a caller-owned state "
+                                     "(two kernels, partial words in the library's static device array)"),
+        "restore_fp16_chunks": entry(lambda: _lib.check(lib.ps_restore_fp16_chunks(table, n_dev, N, None, stream()), "restore"),
+                                     6 * C * N, "ps_restore_fp16_chunks: fp16 parameters rewritten from the fp32 masters (6 B/element)"),
+    }
+    src32 = cl[client.positions()[0].fp32].payload
+    dst16 = cl[client.positions()[0].fp16].payload
+    out["cast_fp32_to_fp16"] = entry(lambda: _lib.check(lib.ps_cast_fp32_to_fp16(src32.data_ptr(), dst16.data_ptr(), N, stream()), "cast"),
+                                     6 * N, "ps_cast_fp32_to_fp16 on one tensor (6 B/element)")
+    out["scan_one_tensor_f16"] = entry(lambda: _lib.check(lib.ps_overflow_scan(dst16.data_ptr(), N, state, stream()), "scan16"),
+                                       2 * N, "ps_overflow_scan on one fp16 tensor (2 B/element)")
+    out["scan_one_tensor_f32"] = entry(lambda: _lib.check(lib.ps_overflow_scan_f32(src32.data_ptr(), N, state, stream()), "scan32"),
+                                       4 * N, "ps_overflow_scan_f32 on one fp32 tensor (4 B/element)")
+    # the backward-side producer: a gradient tensor of PyTorch's own into its slot of the fp16 payload, probed on the way
+    copies = {}
+    for name, dtype, so, do in (("f16_aligned", torch.half, 0, 0), ("f16_other_phase", torch.half, 3, 5),
+                                ("f32_aligned", torch.float, 0, 0), ("f32_other_phase", torch.float, 1, 3)):
+        g = torch.empty(N + 16, device=dev).normal_(0, 1.0, generator=gen).to(dtype)
+        slot = torch.zeros(N + 16, dtype=torch.half, device=dev)
+        b = (2 if dtype == torch.half else 4) + 2
+        src, dst = g[so:so + N], slot[do:do + N]
+        mine = entry(lambda: _lib.check(lib.ps_grad_to_chunk(src.data_ptr(), int(dtype == torch.half), dst.data_ptr(), N, state, stream()),
+                                        "grad_to_chunk"),
+                     b * N, f"ps_grad_to_chunk, {dtype} gradient at element {so} into the slot at element {do} ({b} B/element), probe included")
+        mine["torch_copy_"] = entry(lambda: dst.copy_(src), b * N, "Tensor.copy_ on the same tensors (no probe)")
+        copies[name] = mine
+        del g, slot
+    out["grad_to_chunk"] = copies
+    out["value"] = out["scan_chunks"]["achieved_GBps"]
+    out["ms_per_step"] = out["scan_chunks"]["avg_device_ms"]
+    print(json.dumps(out))
+
+
 PROBE_SOURCE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "bench_kernels", "ps_stream_probe.hip")
 PROBE_PATH = os.path.join(os.path.dirname(PROBE_SOURCE), "libps_stream_probe.so")
 
@@ -1066,6 +1149,8 @@ def main():
         return ceiling(args)
     if args.mode == "operator":
         return operator_mode(args)
+    if args.mode == "aux":
+        return aux_mode(args)
     if args.mode == "hybrid":
         leg = run_hybrid(args, with_cpu_baseline=not args.no_cpu_baseline)
         if "skipped" in leg:

@@ -1554,9 +1554,9 @@ int ps_overflow_scan_f32(const float* d_grads_fp32, size_t numel, ps_step_state*
     if (!d_state) return fail(PS_ERR_BAD_ARG, "d_state is NULL");
     if (numel == 0) return 0;
     if (!d_grads_fp32) return fail(PS_ERR_BAD_ARG, "d_grads_fp32 is NULL");
-    size_t blocks = (numel + (size_t)kAuxBlock * 16 - 1) / ((size_t)kAuxBlock * 16);
-    hipLaunchKernelGGL(scan_f32_kernel, dim3(grid_1d(blocks, kAuxBlock)), dim3(kAuxBlock), 0,
-                       static_cast<hipStream_t>(stream), d_grads_fp32, numel, d_state);
+    size_t n_tiles = (numel + kScanTileF32 - 1) / kScanTileF32;
+    hipLaunchKernelGGL(scan_f32_kernel, dim3(grid_1d(n_tiles, kScanBlock)), dim3(kScanBlock), kScanLdsBytes,
+                       static_cast<hipStream_t>(stream), d_grads_fp32, numel, n_tiles, d_state);
     PS_HIP(hipGetLastError());
     return 0;
 }
@@ -1597,8 +1597,10 @@ int ps_overflow_scan_chunks_noalloc(const ps_chunk* chunks, int n_chunks, size_t
                            scratch + (size_t)first * tiles_per_chunk);
     });
     if (rc) return rc;
-    hipLaunchKernelGGL(scan_reduce_kernel, dim3(1), dim3(kReduceBlock), 0, s, scratch,
-                       (size_t)n_chunks * tiles_per_chunk, d_flag);
+    // a workgroup per 8192 words (a single one took 33 us over the 196,608 words of 24 x 64 Mi elements)
+    const size_t n_words = (size_t)n_chunks * tiles_per_chunk;
+    const unsigned reducers = (unsigned)std::min<size_t>((n_words + 8191) / 8192, 128);
+    hipLaunchKernelGGL(scan_reduce_kernel, dim3(reducers), dim3(kReduceBlock), 0, s, scratch, n_words, d_flag);
     PS_HIP(hipGetLastError());
     return 0;
 }
@@ -1630,24 +1632,26 @@ int ps_grad_to_chunk(const void* d_grad, int grad_is_half, uint16_t* d_slot_fp16
     if (!addressable || numel < 4096) {
         scalar_span(0, numel);
     } else {
-        // elements before the slot's first 16-byte boundary, whole 8-element vectors, remainder
+        // elements before the slot's first 16-byte boundary, whole 8-element vectors, remainder: one launch, whose
+        // last workgroup does the at most 14 elements in front of and behind the vectors
         const size_t head = (size_t)(((16 - dst % 16) % 16) / 2);
         const size_t n_vec = (numel - head) / 8;
         const size_t body_end = head + n_vec * 8;
-        scalar_span(0, head);
-        size_t blocks = (n_vec + kAuxBlock - 1) / kAuxBlock;
-        dim3 grid(grid_1d(blocks, kAuxBlock)), block(kAuxBlock);
+        const CopyEdges edges{d_grad, d_slot_fp16, head, body_end, numel};
+        size_t blocks = (n_vec + kCopyBlock - 1) / kCopyBlock;
+        unsigned body_blocks = grid_1d(blocks, kCopyBlock);
+        if (((size_t)body_blocks + 1) * kCopyBlock > 0xFFFFFFFFull) body_blocks -= 1;  // room for the edge workgroup
+        dim3 grid(body_blocks + 1), block(kCopyBlock);
         uint16_t* dst_al = d_slot_fp16 + head;
         if (grad_is_half) {
             const uintptr_t first = src + head * 2;
             const int shift = (int)((first % 16) / 2);
             const uint16_t* src_al = reinterpret_cast<const uint16_t*>(first - (uintptr_t)shift * 2);
-            hipLaunchKernelGGL(grad_to_chunk_f16_vec_kernel, grid, block, 0, s, src_al, shift, dst_al, n_vec, d_state);
+            hipLaunchKernelGGL(grad_to_chunk_f16_vec_kernel, grid, block, kCopyLdsBytes, s, src_al, shift, dst_al, n_vec, edges, d_state);
         } else {
-            hipLaunchKernelGGL(grad_to_chunk_f32_vec_kernel, grid, block, 0, s,
-                               static_cast<const float*>(d_grad) + head, dst_al, n_vec, d_state);
+            hipLaunchKernelGGL(grad_to_chunk_f32_vec_kernel, grid, block, kCopyLdsBytes, s,
+                               static_cast<const float*>(d_grad) + head, dst_al, n_vec, edges, d_state);
         }
-        scalar_span(body_end, numel);
     }
     PS_HIP(hipGetLastError());
     return 0;

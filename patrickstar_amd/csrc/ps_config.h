@@ -32,6 +32,15 @@
 #ifndef PS_SCAN_LDS_KB
 #define PS_SCAN_LDS_KB 26  // KiB of unused dynamic LDS per workgroup (0: no cap on resident workgroups)
 #endif
+// Launch shape of the backward-side gradient copy's vector kernels (one gradient tensor into its chunk slot).  Swept over
+// 64 / 128 / 256 threads x 0 / 13 / 17 / 26 KiB on 64 Mi-, 10 Mi- and 2.5 Mi-element gradients: nothing beats 256 threads
+// without a cap (fp16 40 us, fp32 71 us for 64 Mi elements; caps only slow single-wave workgroups down).
+#ifndef PS_COPY_BLOCK
+#define PS_COPY_BLOCK 256  // threads per workgroup
+#endif
+#ifndef PS_COPY_LDS_KB
+#define PS_COPY_LDS_KB 0  // KiB of unused dynamic LDS per workgroup (0: no cap on resident workgroups)
+#endif
 #if PS_MAX_WAVES_PER_EU > 0
 #define PS_OCCUPANCY __attribute__((amdgpu_waves_per_eu(1, PS_MAX_WAVES_PER_EU)))
 #else

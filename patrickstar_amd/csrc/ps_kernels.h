@@ -535,15 +535,41 @@ __global__ void __launch_bounds__(kScanBlock)
     block_flag_commit<kScanBlock>(hit, &st->overflow);
 }
 
-__global__ void __launch_bounds__(kAuxBlock)
-    scan_f32_kernel(const float* __restrict__ f, size_t numel, ps_step_state* st)
+// One scan tile of a binary32 buffer (a value is inf or nan iff its eight exponent bits are all set): the same shape,
+// UNROLL 16-byte loads of 4 floats per lane.
+constexpr int kScanTileF32 = kScanBlock * 4 * kScanUnroll;  // floats per tile
+
+__device__ __forceinline__ uint32_t nonfinite_float(uint32_t w) { return ((w & 0x7F800000u) == 0x7F800000u) ? 1u : 0u; }
+
+template <int BLOCK, int UNROLL>
+__device__ __forceinline__ uint32_t scan_tile_f32(const float* __restrict__ f, size_t numel, size_t tile)
+{
+    constexpr size_t kTileFloats = (size_t)BLOCK * 4 * UNROLL;
+    const uint32_t* w32 = reinterpret_cast<const uint32_t*>(f);
+    uint32_t hit = 0;
+    const size_t base = tile * kTileFloats;
+    if (base >= numel) return 0;
+    if ((((uintptr_t)f) & 15u) == 0 && base + kTileFloats <= numel) {
+        uint4v w[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u)
+            w[u] = ld_u4(reinterpret_cast<const uint16_t*>(w32 + base + ((size_t)u * BLOCK + threadIdx.x) * 4));
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u)
+            hit |= nonfinite_float(w[u][0]) | nonfinite_float(w[u][1]) | nonfinite_float(w[u][2]) | nonfinite_float(w[u][3]);
+    } else {
+        size_t end = base + kTileFloats < numel ? base + kTileFloats : numel;
+        for (size_t i = base + threadIdx.x; i < end; i += BLOCK) hit |= nonfinite_float(w32[i]);
+    }
+    return hit;
+}
+
+__global__ void __launch_bounds__(kScanBlock)
+    scan_f32_kernel(const float* __restrict__ f, size_t numel, size_t n_tiles, ps_step_state* st)
 {
     uint32_t hit = 0;
-    const uint32_t* w = reinterpret_cast<const uint32_t*>(f);
-    size_t stride = (size_t)gridDim.x * kAuxBlock;
-    for (size_t i = (size_t)blockIdx.x * kAuxBlock + threadIdx.x; i < numel; i += stride)
-        hit |= ((w[i] & 0x7F800000u) == 0x7F800000u) ? 1u : 0u;
-    block_flag_commit(hit, &st->overflow);
+    for (size_t t = blockIdx.x; t < n_tiles; t += gridDim.x) hit |= scan_tile_f32<kScanBlock, kScanUnroll>(f, numel, t);
+    block_flag_commit<kScanBlock>(hit, &st->overflow);
 }
 
 __global__ void __launch_bounds__(kScanBlock)
@@ -554,7 +580,7 @@ __global__ void __launch_bounds__(kScanBlock)
 }
 
 // The same probe without atomics and without a caller-side state: every workgroup leaves the OR over its tile in
-// its own word of a partial-result array; a second, single-workgroup kernel ORs those words into the caller's flag.
+// its own word of a partial-result array; a second, small kernel ORs those words into the caller's flag.
 __global__ void __launch_bounds__(kAuxBlock)
     scan_chunks_partial_kernel(ChunkBatch b, uint32_t* __restrict__ partial)
 {
@@ -578,9 +604,13 @@ __global__ void __launch_bounds__(kReduceBlock)
     scan_reduce_kernel(const uint32_t* __restrict__ partial, size_t n_words, uint32_t* flag)
 {
     __shared__ uint32_t wave_hit[kReduceBlock / 64];
+    // every workgroup takes one slice of the words; those that find a hit all store the same 1
+    const size_t per = (n_words + gridDim.x - 1) / gridDim.x;
+    const size_t lo = (size_t)blockIdx.x * per;
+    const size_t hi = lo + per < n_words ? lo + per : n_words;
     uint32_t hit = 0;
 #pragma unroll 8
-    for (size_t i = threadIdx.x; i < n_words; i += kReduceBlock) hit |= partial[i];
+    for (size_t i = lo + threadIdx.x; i < hi; i += kReduceBlock) hit |= partial[i];
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) hit |= (uint32_t)__shfl_xor((int)hit, off, 64);
     if ((threadIdx.x & 63) == 0) wave_hit[threadIdx.x >> 6] = hit;
@@ -632,13 +662,18 @@ __device__ __forceinline__ uint4v shift_halves(const uint4v& a, const uint4v& b)
     return o;
 }
 
+// Launch shape of the vector copy kernels: threads per workgroup and an unused dynamic-LDS request that caps the
+// resident workgroups per CU (0: no cap).
+constexpr int kCopyBlock = PS_COPY_BLOCK;
+constexpr size_t kCopyLdsBytes = (size_t)PS_COPY_LDS_KB * 1024;
+
 template <int S>
 __device__ __forceinline__ uint32_t copy_shifted_f16(const uint16_t* src_al, uint16_t* dst_al,
-                                                      size_t n_vec)
+                                                      size_t n_vec, unsigned body_blocks)
 {
     uint32_t hit = 0;
-    size_t stride = (size_t)gridDim.x * kAuxBlock;
-    for (size_t j = (size_t)blockIdx.x * kAuxBlock + threadIdx.x; j < n_vec; j += stride) {
+    size_t stride = (size_t)body_blocks * kCopyBlock;
+    for (size_t j = (size_t)blockIdx.x * kCopyBlock + threadIdx.x; j < n_vec; j += stride) {
         uint4v a = ld_u4(src_al + 8 * j);
         uint4v b = a;
         if (S != 0) b = ld_u4(src_al + 8 * j + 8);
@@ -650,44 +685,79 @@ __device__ __forceinline__ uint32_t copy_shifted_f16(const uint16_t* src_al, uin
     return hit;
 }
 
-__global__ void __launch_bounds__(kAuxBlock)
-    grad_to_chunk_f16_vec_kernel(const uint16_t* __restrict__ src_al, int shift,
-                                 uint16_t* __restrict__ dst_al, size_t n_vec, ps_step_state* st)
+// The elements in front of the slot's first 16-byte boundary and behind its last whole vector (at most 7 each), by
+// the LAST workgroup of the vector kernels' launch: a gradient costs one launch wherever its slot starts.
+struct CopyEdges {
+    const void* src;  // the gradient's first element
+    uint16_t* dst;    // the slot's first element
+    size_t head;      // elements [0, head) and [body_end, numel) go element by element
+    size_t body_end, numel;
+};
+
+template <bool SRC_HALF>
+__device__ __forceinline__ uint32_t copy_edges(const CopyEdges& e)
 {
+    const uint16_t* sh = static_cast<const uint16_t*>(e.src);
+    const float* sf = static_cast<const float*>(e.src);
+    const size_t n_edge = e.head + (e.numel - e.body_end);
     uint32_t hit = 0;
-    switch (shift) {
-        case 0: hit = copy_shifted_f16<0>(src_al, dst_al, n_vec); break;
-        case 1: hit = copy_shifted_f16<1>(src_al, dst_al, n_vec); break;
-        case 2: hit = copy_shifted_f16<2>(src_al, dst_al, n_vec); break;
-        case 3: hit = copy_shifted_f16<3>(src_al, dst_al, n_vec); break;
-        case 4: hit = copy_shifted_f16<4>(src_al, dst_al, n_vec); break;
-        case 5: hit = copy_shifted_f16<5>(src_al, dst_al, n_vec); break;
-        case 6: hit = copy_shifted_f16<6>(src_al, dst_al, n_vec); break;
-        default: hit = copy_shifted_f16<7>(src_al, dst_al, n_vec); break;
+    for (size_t j = threadIdx.x; j < n_edge; j += kCopyBlock) {
+        const size_t i = j < e.head ? j : e.body_end + (j - e.head);
+        uint32_t h = SRC_HALF ? (uint32_t)sh[i] : float_to_half_bits(sf[i]);
+        e.dst[i] = (uint16_t)h;
+        hit |= ((h & 0x7C00u) == 0x7C00u) ? 1u : 0u;
     }
-    if (st != nullptr) block_flag_commit(hit, &st->overflow);
+    return hit;
+}
+
+__global__ void __launch_bounds__(kCopyBlock)
+    grad_to_chunk_f16_vec_kernel(const uint16_t* __restrict__ src_al, int shift,
+                                 uint16_t* __restrict__ dst_al, size_t n_vec, CopyEdges edges, ps_step_state* st)
+{
+    const unsigned body_blocks = gridDim.x - 1;
+    uint32_t hit = 0;
+    if (blockIdx.x == body_blocks) {
+        hit = copy_edges<true>(edges);
+    } else {
+        switch (shift) {
+            case 0: hit = copy_shifted_f16<0>(src_al, dst_al, n_vec, body_blocks); break;
+            case 1: hit = copy_shifted_f16<1>(src_al, dst_al, n_vec, body_blocks); break;
+            case 2: hit = copy_shifted_f16<2>(src_al, dst_al, n_vec, body_blocks); break;
+            case 3: hit = copy_shifted_f16<3>(src_al, dst_al, n_vec, body_blocks); break;
+            case 4: hit = copy_shifted_f16<4>(src_al, dst_al, n_vec, body_blocks); break;
+            case 5: hit = copy_shifted_f16<5>(src_al, dst_al, n_vec, body_blocks); break;
+            case 6: hit = copy_shifted_f16<6>(src_al, dst_al, n_vec, body_blocks); break;
+            default: hit = copy_shifted_f16<7>(src_al, dst_al, n_vec, body_blocks); break;
+        }
+    }
+    if (st != nullptr) block_flag_commit<kCopyBlock>(hit, &st->overflow);
 }
 
 // fp32 gradients: eight dword-aligned floats per output vector (multi-dword loads need dword alignment only).
-__global__ void __launch_bounds__(kAuxBlock)
+__global__ void __launch_bounds__(kCopyBlock)
     grad_to_chunk_f32_vec_kernel(const float* __restrict__ src, uint16_t* __restrict__ dst_al,
-                                 size_t n_vec, ps_step_state* st)
+                                 size_t n_vec, CopyEdges edges, ps_step_state* st)
 {
+    const unsigned body_blocks = gridDim.x - 1;
     uint32_t hit = 0;
-    size_t stride = (size_t)gridDim.x * kAuxBlock;
-    for (size_t j = (size_t)blockIdx.x * kAuxBlock + threadIdx.x; j < n_vec; j += stride) {
-        float4v x = *(const PS_GLOBAL float4v_dword_aligned*)(src + 8 * j);
-        float4v y = *(const PS_GLOBAL float4v_dword_aligned*)(src + 8 * j + 4);
-        uint4v o;
-        o[0] = float_to_half_bits(x[0]) | (float_to_half_bits(x[1]) << 16);
-        o[1] = float_to_half_bits(x[2]) | (float_to_half_bits(x[3]) << 16);
-        o[2] = float_to_half_bits(y[0]) | (float_to_half_bits(y[1]) << 16);
-        o[3] = float_to_half_bits(y[2]) | (float_to_half_bits(y[3]) << 16);
-        hit |= nonfinite_halves(o[0]) | nonfinite_halves(o[1]) | nonfinite_halves(o[2]) |
-               nonfinite_halves(o[3]);
-        st_u4(dst_al + 8 * j, o);
+    if (blockIdx.x == body_blocks) {
+        hit = copy_edges<false>(edges);
+    } else {
+        size_t stride = (size_t)body_blocks * kCopyBlock;
+        for (size_t j = (size_t)blockIdx.x * kCopyBlock + threadIdx.x; j < n_vec; j += stride) {
+            float4v x = *(const PS_GLOBAL float4v_dword_aligned*)(src + 8 * j);
+            float4v y = *(const PS_GLOBAL float4v_dword_aligned*)(src + 8 * j + 4);
+            uint4v o;
+            o[0] = float_to_half_bits(x[0]) | (float_to_half_bits(x[1]) << 16);
+            o[1] = float_to_half_bits(x[2]) | (float_to_half_bits(x[3]) << 16);
+            o[2] = float_to_half_bits(y[0]) | (float_to_half_bits(y[1]) << 16);
+            o[3] = float_to_half_bits(y[2]) | (float_to_half_bits(y[3]) << 16);
+            hit |= nonfinite_halves(o[0]) | nonfinite_halves(o[1]) | nonfinite_halves(o[2]) |
+                   nonfinite_halves(o[3]);
+            st_u4(dst_al + 8 * j, o);
+        }
     }
-    if (st != nullptr) block_flag_commit(hit, &st->overflow);
+    if (st != nullptr) block_flag_commit<kCopyBlock>(hit, &st->overflow);
 }
 
 // ------------------------------------------------ device-resident step state

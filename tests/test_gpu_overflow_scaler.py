@@ -43,6 +43,31 @@ def test_overflow_scan_positions_and_values(n):
     assert ps.DynamicLossScaler._has_inf_or_nan(f32) is True
 
 
+@pytest.mark.parametrize("n", [1, 5, 2047, 2048, 2049, 4096 + 3, 2048 * 5, 2048 * 37 + 11, 1 << 20])
+def test_overflow_scan_of_binary32_gradients_positions_and_values(n):
+    """The probe on fp32 gradients (what check_overflow sees when backward leaves binary32 .grad tensors): 16-byte loads
+    on whole tiles, element by element on the ragged end and on views that do not start on a 16-byte boundary."""
+    probe = ps.DynamicLossScaler._has_inf_or_nan
+    base = torch.randn(n, device="cuda") * 1e3
+    base[::7] = torch.finfo(torch.float32).max   # the largest finite values and subnormals are not an overflow
+    base[3::11] = 1e-45
+    assert probe(base) is False
+    for pos in sorted({0, n - 1, n // 2, max(0, n - 9), min(n - 1, 2047), min(n - 1, 2048)}):
+        for bad in (float("inf"), float("-inf"), float("nan")):
+            x = base.clone()
+            x[pos] = bad
+            assert probe(x) is True, (n, pos, bad)
+            for skip in (1, 3, 4):  # views at a 4-, 12- and 16-byte offset
+                if n > skip:
+                    assert probe(x[skip:]) is (pos >= skip), (n, pos, bad, skip)
+    # a quiet nan with payload bits and a negative nan
+    x = base.clone().view(torch.int32)
+    x[n // 3] = 0x7FC12345
+    assert probe(x.view(torch.float32)) is True
+    x[n // 3] = -1  # 0xFFFFFFFF
+    assert probe(x.view(torch.float32)) is True
+
+
 def test_overflow_scan_empty_and_sticky_flag():
     s = ps.DynamicLossScaler(init_scale=2**16)
     s.scan(torch.zeros(0, dtype=torch.half, device="cuda"))
