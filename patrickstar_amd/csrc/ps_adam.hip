@@ -1593,7 +1593,7 @@ int ps_overflow_scan_chunks_noalloc(const ps_chunk* chunks, int n_chunks, size_t
     if (int rc = scratch_address(&scratch)) return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
     int rc = for_each_batch(a, [&](const ChunkBatch& b, dim3 grid, int first) {
-        hipLaunchKernelGGL(scan_chunks_partial_kernel, grid, dim3(kAuxBlock), 0, s, b,
+        hipLaunchKernelGGL(scan_chunks_partial_kernel, grid, dim3(kPartialBlock), kScanLdsBytes, s, b,
                            scratch + (size_t)first * tiles_per_chunk);
     });
     if (rc) return rc;
