@@ -595,10 +595,35 @@ def dynamic_leg(cfg, steps, warmup):
 
     ms, kernel_ms = time_steps(torch, step, steps, warmup)
     st = scaler._read()
-    lib.ps_adam_destroy(992)
     elements = cfg.C * cfg.N
     avg = sum(kernel_ms) / len(kernel_ms)
+
+    # a step that the device skips (the flag is up when the gated kernel starts): the fp16 parameters are rewritten from the
+    # fp32 masters (read 4, write 2 bytes per element beside the probe's 2) and the scale is lowered, all without the host
+    skipper = ps.DynamicLossScaler(init_scale=2**40, scale_factor=2, scale_window=1000, min_scale=1)
+    skipper.materialize(cfg.dev, betas=HYPER["betas"])
+    off = _lib.ps_step_state.overflow.offset
+    flag = skipper._state[off:off + 4].view(torch.int32)
+
+    def skipped():
+        s = _lib.current_stream_handle()
+        _lib.check(lib.ps_overflow_scan_chunks(table, n_dev, cfg.N, None, skipper.state_ptr, s), "scan")
+        flag.fill_(1)  # as if the probe had found an inf
+        _lib.check(lib.ps_adam_step_chunks_gated(992, HYPER["lr"], HYPER["eps"], HYPER["weight_decay"], 1, table, n_dev, cfg.N, None,
+                                                 calls, skipper.state_ptr, s), "gated")
+        skipper.update_scale(None, operator_calls=cfg.C)
+
+    n_skip = max(3, steps // 4)
+    skip_ms, skip_kernel_ms = time_steps(torch, skipped, n_skip, 1)
+    skip_avg = sum(skip_kernel_ms) / len(skip_kernel_ms)
+    sk = skipper._read()
+    lib.ps_adam_destroy(992)
     return {
+        "skipped_step": {"ms_per_step": skip_ms, "avg_device_ms": skip_avg, "steps": n_skip,
+                         "algorithmic_bytes_per_step": 8 * elements, "achieved_GBps": 8 * elements / (skip_avg * 1e-3) / 1e9,
+                         "skipped_steps": int(sk.skipped_steps), "adam_step_after": int(sk.adam_step),
+                         "what": "the same sequence with the overflow flag up: probe, fp16 parameters restored from the fp32 masters, "
+                                 "scale lowered; fp32 param / m / v and the step counter untouched"},
         "value": elements / (ms * 1e-3), "unit": "params/s", "ms_per_step": ms, "avg_device_ms": avg,
         "kernels": "scan_chunks_kernel + adam_chunks_gated_kernel + scaler_update_kernel, no host sync",
         "algorithmic_bytes_per_step": 30 * elements, "achieved_GBps": 30 * elements / (avg * 1e-3) / 1e9,
